@@ -1,0 +1,183 @@
+/*
+ * C ABI of libmoe_gfx950.so -- MI355X (gfx950) kernels for the MoE context-encoding
+ * path of aws-neuron/nki-library.
+ *
+ * The reference has no FFI: its operator boundary is the pair of Python kernels
+ *   moe_cte(...)               src/nkilib_src/nkilib/core/moe/moe_cte/moe_cte.py:252-277
+ *   rmsnorm_quant_kernel(...)  src/nkilib_src/nkilib/core/rmsnorm/rmsnorm_quant.py:86-92
+ * This header declares what a Python (ctypes) binding of those two functions
+ * calls instead of the NKI device code.  All tensor pointers are DEVICE pointers;
+ * `stream` is a hipStream_t passed as void* (NULL = default stream).  Every
+ * function returns 0 on success or a negative MOE_E_* code; moe_error_string()
+ * turns it into text.  Functions validate shapes before launching anything.
+ * No function allocates device memory: scratch comes from the caller through
+ * (workspace, workspace_bytes), sized by moe_blockwise_workspace_bytes().
+ */
+#ifndef MOE_GFX950_H
+#define MOE_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes ------------------------------------------------------------------- */
+#define MOE_OK 0
+#define MOE_E_BAD_ARG (-1)       /* null pointer, negative size, unknown enum value            */
+#define MOE_E_BAD_SHAPE (-2)     /* shape violates a documented divisibility / range rule     */
+#define MOE_E_WORKSPACE (-3)     /* workspace missing or smaller than *_workspace_bytes()     */
+#define MOE_E_LAUNCH (-4)        /* hipLaunchKernel / hipMemsetAsync reported an error        */
+#define MOE_E_UNSUPPORTED (-5)   /* valid in the reference, not built here                    */
+#define MOE_E_NO_DEVICE (-6)     /* current device is not gfx950                              */
+
+const char* moe_error_string(int code);
+/* ABI version of this header; bumped on any signature change. */
+int moe_abi_version(void);
+/* 0 when the current HIP device is gfx950, MOE_E_NO_DEVICE otherwise. */
+int moe_check_device(void);
+
+/* ---- element types ----------------------------------------------------------------- */
+#define MOE_DT_BF16 0
+#define MOE_DT_FP16 1
+#define MOE_DT_FP32 2
+#define MOE_DT_FP8_E4M3 3 /* OCP e4m3fn bit patterns; Neuron float8_e4m3 is the |v|<=240 subset */
+
+/* ---- RMSNorm + quantise front end -------------------------------------------------- */
+
+/* Replaces rmsnorm_quant_kernel with QuantizationType.ROW
+ * (rmsnorm_quant.py:86-171, _row_quantize_tile :526-620, store :342-403).
+ * x [rows, H] (x_dtype bf16/fp16/fp32), gamma [H] (gamma_dtype) or NULL when do_norm == 0.
+ * out: uint8 [rows, H+4]; bytes [0,H) are e4m3 codes of n/dq, bytes [H,H+4) the
+ * little-endian fp32 dequant scale dq = max(amax/240, 1e-6).
+ * n = x * (1/(sqrt(mean(x^2)) + eps)) * gamma  (the test golden's form,
+ * test/integration/nkilib/core/rmsnorm/test_rmsnorm_quant.py:73-75).
+ * lower_bound > 0 clips amax and n to +-lower_bound first.  H <= 16384. */
+int moe_rmsnorm_quant_fp8_row(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out,
+                              int64_t rows, int64_t H, float eps, float lower_bound, int do_norm,
+                              void* stream);
+
+/* Replaces rmsnorm_quant_kernel with QuantizationType.STATIC (_static_quantize_tile,
+ * rmsnorm_quant.py:623-662).  input_dequant_scale: device fp32, element 0 is used
+ * (the reference broadcasts one scalar to [128,1]).  out: uint8 [rows, H]
+ * = e4m3(clip(n * (1/scale), +-240)). */
+int moe_rmsnorm_quant_fp8_static(const void* x, int x_dtype, const void* gamma, int gamma_dtype,
+                                 const float* input_dequant_scale, void* out, int64_t rows, int64_t H,
+                                 float eps, int do_norm, void* stream);
+
+/* Output layouts of moe_rmsnorm_quant_mxfp8 */
+#define MOE_MX_LAYOUT_TOKEN_MAJOR 0 /* q [rows, H] bytes in k' order, scale [rows, H/32]                     */
+#define MOE_MX_LAYOUT_REF_DENSE 1   /* q x4 [128, H/512, rows], scale [16, H/512, rows]                      */
+#define MOE_MX_LAYOUT_REF_STRIDED 2 /* as 1 but scale [128, H/512, rows], row (s/4)*32 + s%4 holds scale s   */
+
+/* Replaces rmsnorm_mx_quantize_tkg (src/nkilib_src/nkilib/core/subkernels/rmsnorm_mx_quantize_tkg.py:29-40;
+ * golden test/integration/nkilib/core/subkernels/test_rmsnorm_mx_quantize_tkg.py:100-137) and the online
+ * activation quantisation of the MX MoE kernel (moe_cte_mx_utils.py:730-771).
+ * n = bf16(x * (1/sqrt(sum(x^2)/hidden_actual + eps)) * gamma) when do_norm, else bf16(x);
+ * then MXFP8-e4m3 with one E8M0 scale per 32 consecutive k', k' = tile*512 + p*4 + q for
+ * h = q*(H/4) + tile*128 + p.  H % 512 == 0, H <= 16384.
+ * out_norm (nullable): bf16 [128, rows, H/128], element [p, t, h1] = n[t, h1*128 + p]. */
+int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out_q,
+                            void* out_scale, void* out_norm, int64_t rows, int64_t H, float eps,
+                            int64_t hidden_actual, int do_norm, int layout, void* stream);
+
+/* ---- token -> block index construction ---------------------------------------------- */
+
+/* Device version of generate_token_position_to_id_and_experts
+ * (test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:199-264), bit exact.
+ * topk_ids int32 [T, k] (distinct expert ids per row; ids outside [0,E) are ignored).
+ * Writes token_position_to_id int32[N*B], block_to_expert int32[N], conditions int32[n_conditions]
+ * (nullable; ones for the first N - n_padding_blocks entries... exactly: the trailing
+ * n_padding_blocks + (n_conditions - N) entries are 0).  pad id = T, or -1 when skip_token.
+ * workspace: >= moe_build_blocks_workspace_bytes(E) bytes.  Returns MOE_E_BAD_SHAPE through
+ * *status_out (device int32, nullable) == 1 when N is too small for the routing. */
+size_t moe_build_blocks_workspace_bytes(int64_t E);
+int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                     int skip_token, int use_split_padding, int32_t* token_position_to_id,
+                     int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
+                     void* workspace, size_t workspace_bytes, int32_t* status_out, void* stream);
+
+/* ---- blockwise MoE ------------------------------------------------------------------- */
+
+#define MOE_KIND_BF16 0    /* bf16 activations, bf16 weights or fp8 weights + per-channel fp32 scales */
+#define MOE_KIND_FP8_ROW 1 /* fp8 activations with per-row scale ([T1, H+4] records), fp8 weights      */
+#define MOE_KIND_MXFP8 2   /* MXFP8 weights (reference x4 layouts), activations quantised to MXFP8     */
+
+/* ActFnType values, src/nkilib_src/nkilib/core/utils/common_types.py:32-36 */
+#define MOE_ACT_SILU 0
+#define MOE_ACT_GELU 1
+#define MOE_ACT_GELU_TANH 2
+#define MOE_ACT_SWISH 3
+/* ExpertAffinityScaleMode values, common_types.py:48-52 */
+#define MOE_SCALE_NONE 0
+#define MOE_SCALE_POST 1
+#define MOE_SCALE_PRE 2
+#define MOE_SCALE_PRE_DELAYED 3
+
+#define MOE_CLAMP_GATE_HI 1
+#define MOE_CLAMP_GATE_LO 2
+#define MOE_CLAMP_UP_HI 4
+#define MOE_CLAMP_UP_LO 8
+
+typedef struct moe_bwmm_args {
+  /* -- tensors, named as the arguments of moe_cte (moe_cte.py:253-277) ------------------
+   * hidden_states:
+   *   BF16 kind     bf16 [T1, H]
+   *   FP8_ROW kind  uint8 [T1, H+4]: rmsnorm_quant ROW records (codes + fp32 scale)
+   *   MXFP8 kind    bf16 [T1, H] (quantised online, hidden_states_scale == NULL), or
+   *                 uint8 [T1, H] e4m3 codes in k' order with hidden_states_scale uint8 [T1, H/32]
+   * T1 = T+1 (row T is the all-zero padding token) or T when skip_token. */
+  const void* hidden_states;
+  const void* hidden_states_scale;
+  const void* expert_affinities_masked; /* [T1*E], affinity_dtype (bf16 or fp32), row-major [T1, E] */
+  /* BF16: [E,H,2,I] weight_dtype (bf16 | fp8);  FP8_ROW: uint8 [E,H,2,I];
+   * MXFP8: uint8 [E,128,2,H/512,I,4] (x4: byte q of element i)                              */
+  const void* gate_up_proj_weight;
+  /* BF16: [E,I_pad,H];  FP8_ROW: uint8 [E,I_pad,H];  MXFP8: uint8 [E,p_I,ceil(I/512),H,4]    */
+  const void* down_proj_weight;
+  /* BF16/FP8_ROW: fp32 [E or 1, 1, 2I] / [E or 1, 1, H] (NULL = unquantised bf16 weights);
+   * MXFP8: uint8 [E,16,2,H/512,I] / [E,ceil(p_I/8),ceil(I/512),H]                            */
+  const void* gate_up_proj_scale;
+  const void* down_proj_scale;
+  /* bias_dtype; BF16/FP8_ROW: [E,2,I], [E,H];  MXFP8: [E,p_I,2,ceil(I/512),4], [E,H]; nullable */
+  const void* gate_and_up_proj_bias;
+  const void* down_proj_bias;
+  const int32_t* token_position_to_id; /* [N*B] */
+  const int32_t* block_to_expert;      /* [N]   */
+  const int32_t* conditions;           /* nullable, [n_conditions]; blocks from the first 0 on are skipped */
+  void* output;                        /* bf16; row t at output + t*out_row_stride elements, T1 rows written */
+  void* workspace;
+  size_t workspace_bytes;
+  /* -- sizes --------------------------------------------------------------------------- */
+  int64_t T1, H, I, E, B, N;
+  int64_t I_pad;          /* rows of down_proj_weight per expert (BF16 / FP8_ROW); 0 = I          */
+  int64_t n_conditions;   /* entries readable in conditions                                       */
+  int64_t out_row_stride; /* in elements; H for [T1,H], 2H for slot 0 of [T1,2,H]                 */
+  int32_t scale_experts;  /* leading dim of the fp32 scales: E or 1 (BF16 / FP8_ROW)              */
+  /* -- options ------------------------------------------------------------------------- */
+  int32_t kind;           /* MOE_KIND_*                                                           */
+  int32_t weight_dtype;   /* BF16 kind: MOE_DT_BF16 or MOE_DT_FP8_E4M3                            */
+  int32_t affinity_dtype; /* MOE_DT_BF16 or MOE_DT_FP32                                           */
+  int32_t bias_dtype;     /* MOE_DT_BF16 or MOE_DT_FP32                                           */
+  int32_t act_fn;         /* MOE_ACT_*                                                            */
+  int32_t scaling_mode;   /* MOE_SCALE_*                                                          */
+  int32_t skip_token;     /* 1: padding id is -1 and tables have T rows                           */
+  int32_t clamp_mask;     /* MOE_CLAMP_* bits                                                     */
+  float gate_clamp_upper, gate_clamp_lower, up_clamp_upper, up_clamp_lower;
+} moe_bwmm_args;
+
+/* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /
+ * bwmm_shard_on_block_mx (moe_cte.py:348-489): for every block b before the first
+ * conditions[b]==0, rows x = hidden[token_position_to_id[b*B..]], expert e = block_to_expert[b]:
+ * out[token] += bf16( down(act(gate(x)) * up(x)) * affinity[token*E+e] ), accumulated per
+ * token in block order in bf16, exactly as the golden does
+ * (test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:267-447).
+ * Rows of `output` not reached by any block are set to zero. */
+size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* args);
+int moe_blockwise(const moe_bwmm_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_GFX950_H */

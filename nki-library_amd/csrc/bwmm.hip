@@ -1,0 +1,478 @@
+// Blockwise expert GEMMs for gfx950: gate/up projection with fused act(gate)*up (stage 1) and
+// down projection with fused bias / affinity (stage 2), for three precisions:
+//   BF16     v_mfma_f32_16x16x32_bf16, weights bf16 or fp8 (+ per-channel fp32 scale)
+//   FP8_ROW  v_mfma_scale_f32_16x16x128_f8f6f4 with unit block scales; per-row activation and
+//            per-channel weight scales applied to the fp32 accumulators
+//   MXFP8    v_mfma_scale_f32_16x16x128_f8f6f4, E8M0 block scales of both operands applied by
+//            the matrix core
+// This file holds the general tiled kernel: a 256-thread workgroup owns 128 rows of one block
+// (one expert) and 128 output columns (256 in stage 1: gate and up), stages one 128-byte
+// K-slice of both operands in LDS in K-contiguous order and lets each of the four waves run
+// 2 x (8|16) MFMA tiles over it.  Rows are gathered through token_position_to_id while the A
+// operand is staged (the gather is fused into the load, no gathered copy exists in HBM).
+//
+// Reference semantics: generate_blockwise_numpy_golden,
+//   test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:267-447 (bf16 / fp8 weight),
+//   test/integration/nkilib/core/moe/moe_cte/test_utils.py:474-735 with
+//   test/integration/nkilib/core/mlp/test_mlp_common.py:550-682 (MXFP8),
+//   test/integration/nkilib/core/mlp/test_mlp_common.py:978-1022,1114-1116 (fp8 row scales).
+#include "bwmm.hpp"
+
+namespace moe {
+
+constexpr int GT = 256;       // threads per workgroup
+constexpr int TM = 128;       // rows per workgroup tile
+constexpr int LROW = 144;     // LDS bytes per staged row: 128 bytes of K + 16 pad (16-byte aligned)
+
+__device__ __forceinline__ float load_aff(const void* aff, int dtype, int64_t idx) {
+  return dtype == MOE_DT_BF16 ? bf16_bits_to_f32(((const uint16_t*)aff)[idx]) : ((const float*)aff)[idx];
+}
+__device__ __forceinline__ float load_bias(const void* p, int dtype, int64_t idx) {
+  return dtype == MOE_DT_BF16 ? bf16_bits_to_f32(((const uint16_t*)p)[idx]) : ((const float*)p)[idx];
+}
+
+__device__ __forceinline__ v8i lds_read32(const uint8_t* p) {
+  const v4i lo = *(const v4i*)p;
+  const v4i hi = *(const v4i*)(p + 16);
+  v8i r;
+  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+  return r;
+}
+
+template <int KIND, int STAGE>
+__global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
+  constexpr int NCOLS = (STAGE == 1) ? 256 : 128;
+  constexpr int NT = NCOLS / 16;
+  __shared__ __attribute__((aligned(16))) uint8_t sA[TM * LROW];
+  __shared__ __attribute__((aligned(16))) uint8_t sB[NCOLS * LROW];
+  __shared__ uint32_t sAs[TM];   // MX: the 4 E8M0 bytes of this k-step; FP8_ROW: fp32 row scale bits
+  __shared__ uint32_t sBs[NCOLS];
+  __shared__ int s_tok[TM];
+  __shared__ float s_aff[TM];
+
+  const int tid = threadIdx.x;
+  const int rt = blockIdx.y;
+  const int b = rt / a.tiles_per_block;
+  const int r0 = (rt % a.tiles_per_block) * TM;
+  if (b >= *a.n_active) return;
+  const int vr = a.valid_rows[b];
+  if (r0 >= vr) return;
+  const int e = a.b2e[b];
+  const int64_t slot0 = (int64_t)b * a.B + r0;
+
+  // ---- column tile geometry -------------------------------------------------------------
+  // MX stage 1: blockIdx.x = tI*4 + pg; columns are (gu, q, pl) with weight column
+  // i = tI*512 + q*Pt + p0 + pl, Pt = valid partitions of intermediate tile tI.
+  int tI = 0, p0 = 0, Pt = 0;
+  int64_t c0 = 0;  // first output column (BF16 / FP8_ROW stage 1: i0; stage 2: h0)
+  if (KIND == MOE_KIND_MXFP8 && STAGE == 1) {
+    tI = blockIdx.x >> 2;
+    p0 = (blockIdx.x & 3) * 32;
+    const int rows_t = (int)((a.I - (int64_t)tI * 512 < 512) ? (a.I - (int64_t)tI * 512) : 512);
+    Pt = rows_t / 4;
+    if (p0 >= Pt) return;
+  } else {
+    c0 = (int64_t)blockIdx.x * 128;
+  }
+
+  if (tid < TM) {
+    const int r = r0 + tid;
+    int id = -1;
+    if (r < a.B) id = a.tp2id[(int64_t)b * a.B + r];
+    if (id < 0 || id >= a.n_real) id = -1;
+    s_tok[tid] = id;
+    float af = 0.f;
+    if (id >= 0 && a.aff) af = load_aff(a.aff, a.aff_dtype, (int64_t)id * a.E + e);
+    s_aff[tid] = af;
+    if (KIND == MOE_KIND_FP8_ROW) {
+      float rs = 0.f;
+      if (STAGE == 1) {
+        if (id >= 0) rs = *(const float*)(a.A + (int64_t)id * a.a_stride + a.H);
+      } else {
+        if (r < vr) rs = ((const float*)a.A_scale)[slot0 + tid];
+      }
+      sAs[tid] = __float_as_uint(rs);
+    }
+  }
+  __syncthreads();
+
+  const int lane = tid & 63, w = tid >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int m0 = w * 32;
+
+  v4f acc[NT][2];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) acc[nt][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  // ---- K loop ---------------------------------------------------------------------------
+  int nks;
+  if (KIND == MOE_KIND_MXFP8) nks = (STAGE == 1) ? (int)(a.H / 128) : a.nI * 4;
+  else if (KIND == MOE_KIND_BF16) nks = (int)((a.K + 63) / 64);
+  else nks = (int)((a.K + 127) / 128);
+
+  for (int ks = 0; ks < nks; ++ks) {
+    // position of this k-step
+    int kt = 0, pb = 0, Ptk = 128;      // MX: K tile (H or I tile), partition group, valid partitions
+    int64_t a_off;                      // byte offset of the slice inside an A row
+    int a_valid = 128;                  // valid bytes of the slice
+    if (KIND == MOE_KIND_MXFP8) {
+      kt = ks >> 2; pb = ks & 3;
+      if (STAGE == 2) {
+        const int rows_t = (int)((a.I - (int64_t)kt * 512 < 512) ? (a.I - (int64_t)kt * 512) : 512);
+        Ptk = rows_t / 4;
+        if (pb * 32 >= Ptk) continue;
+        a_valid = (Ptk - pb * 32) * 4 < 128 ? (Ptk - pb * 32) * 4 : 128;
+      }
+      a_off = (int64_t)kt * 512 + pb * 128;
+    } else {
+      a_off = (int64_t)ks * 128;
+      const int64_t kbytes = (KIND == MOE_KIND_BF16) ? a.K * 2 : a.K;
+      a_valid = (int)((kbytes - a_off < 128) ? (kbytes - a_off) : 128);
+    }
+
+    // ---- stage A: 128 rows x 128 bytes, 8 threads per row ---------------------------------
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = (tid >> 3) + 32 * j;
+      const int ch = tid & 7;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      const uint8_t* src = nullptr;
+      if (STAGE == 1) {
+        const int tok = s_tok[row];
+        if (tok >= 0) src = a.A + (int64_t)tok * a.a_stride;
+      } else {
+        if (r0 + row < vr) src = a.A + (slot0 + row) * a.a_stride;
+      }
+      if (src != nullptr && ch * 16 + 16 <= a_valid) {
+        src += a_off + ch * 16;
+        if (KIND == MOE_KIND_FP8_ROW && STAGE == 1) {  // rows are only 4-byte aligned
+          const uint32_t* s4 = (const uint32_t*)src;
+          val = make_uint4(s4[0], s4[1], s4[2], s4[3]);
+        } else {
+          val = *(const uint4*)src;
+        }
+      }
+      *(uint4*)(sA + row * LROW + ch * 16) = val;
+    }
+    if (KIND == MOE_KIND_MXFP8 && tid < TM) {
+      uint32_t sv = 0;
+      if (STAGE == 1) {
+        const int tok = s_tok[tid];
+        if (tok >= 0) sv = *(const uint32_t*)(a.A_scale + (int64_t)tok * a.a_scale_stride + ks * 4);
+      } else {
+        if (r0 + tid < vr) sv = *(const uint32_t*)(a.A_scale + (slot0 + tid) * a.a_scale_stride + kt * 16 + pb * 4);
+        const int kbv = a_valid >> 5;  // valid 32-blocks in this slice
+        if (kbv < 4) sv &= (1u << (8 * kbv)) - 1u;
+      }
+      sAs[tid] = sv;
+    }
+
+    // ---- stage B, transposed into K-contiguous rows ---------------------------------------
+    if (KIND == MOE_KIND_MXFP8) {
+      const uint32_t* W4 = (const uint32_t*)a.W;
+      if (STAGE == 1) {
+        // column = tid: (gu, q, pl); rows rho = partitions 32*pb + rho of H tile kt
+        const int gu = tid >> 7, q = (tid >> 5) & 3, pl = tid & 31;
+        const bool cv = (p0 + pl) < Pt;
+        const int64_t i = (int64_t)tI * 512 + (int64_t)q * Pt + p0 + pl;
+        const int64_t nH = a.H / 512;
+        const int64_t pstride = 2 * nH * a.I;
+        const int64_t base = ((((int64_t)e * 128 + pb * 32) * 2 + gu) * nH + kt) * a.I + i;
+#pragma unroll 8
+        for (int rho = 0; rho < 32; ++rho) {
+          const uint32_t v = cv ? W4[base + rho * pstride] : 0u;
+          *(uint32_t*)(sB + tid * LROW + rho * 4) = v;
+        }
+        uint32_t sv = 0;
+        if (cv) {
+          const int64_t sbase = ((((int64_t)e * 16 + pb * 4) * 2 + gu) * nH + kt) * a.I + i;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) sv |= (uint32_t)a.W_scale[sbase + k * pstride] << (8 * k);
+        }
+        sBs[tid] = sv;
+      } else {
+        const int col = tid & 127, half = tid >> 7;
+        const int64_t h = c0 + col;
+        const bool cv = h < a.H;
+        const int64_t pstride = (int64_t)a.nI * a.H;
+        const int64_t base = (((int64_t)e * a.pI + pb * 32) * a.nI + kt) * a.H + h;
+#pragma unroll 8
+        for (int j = 0; j < 16; ++j) {
+          const int rho = 2 * j + half;
+          const uint32_t v = (cv && pb * 32 + rho < Ptk) ? W4[base + rho * pstride] : 0u;
+          *(uint32_t*)(sB + col * LROW + rho * 4) = v;
+        }
+        if (half == 0) {
+          uint32_t sv = 0;
+          const int64_t sbase = (((int64_t)e * ((a.pI + 7) / 8) + pb * 4) * a.nI + kt) * a.H + h;
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            if (cv && (pb * 4 + k) * 8 < Ptk) sv |= (uint32_t)a.W_scale[sbase + k * pstride] << (8 * k);
+          sBs[col] = sv;
+        }
+      }
+    } else if (KIND == MOE_KIND_BF16) {
+      // 64 k-rows x NCOLS columns of bf16 (or fp8 widened to bf16)
+      constexpr int CP = NCOLS / 2;        // column pairs
+      constexpr int RSTEP = GT / CP;       // k-rows covered per pass
+      const int cp = tid % CP, kr0 = tid / CP;
+      const bool w8 = a.weight_dtype == MOE_DT_FP8_E4M3;
+#pragma unroll 4
+      for (int j = 0; j < 64 / RSTEP; ++j) {
+        const int kr = kr0 + RSTEP * j;
+        const int64_t k = (int64_t)ks * 64 + kr;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+          const int col = 2 * cp + cc;
+          uint16_t v = 0;
+          int64_t idx = -1;
+          if (STAGE == 1) {
+            const int gu = col >> 7;
+            const int64_t i = c0 + (col & 127);
+            if (k < a.H && i < a.I) idx = (((int64_t)e * a.H + k) * 2 + gu) * a.I + i;
+          } else {
+            const int64_t h = c0 + col;
+            if (k < a.I && h < a.H) idx = ((int64_t)e * a.I_pad + k) * a.H + h;
+          }
+          if (idx >= 0) v = w8 ? f32_to_bf16_bits(e4m3_to_f32(a.W[idx])) : ((const uint16_t*)a.W)[idx];
+          *(uint16_t*)(sB + col * LROW + kr * 2) = v;
+        }
+      }
+    } else {  // FP8_ROW: 128 k-rows x NCOLS byte columns, byte transpose
+      constexpr int CG = NCOLS / 4;
+      constexpr int RSTEP = GT / CG;
+      const int cg = tid % CG, kr0 = tid / CG;
+#pragma unroll 4
+      for (int j = 0; j < 128 / RSTEP; ++j) {
+        const int kr = kr0 + RSTEP * j;
+        const int64_t k = (int64_t)ks * 128 + kr;
+        uint32_t v = 0;
+        const int col = 4 * cg;
+        if (STAGE == 1) {
+          const int gu = col >> 7;
+          const int64_t i = c0 + (col & 127);
+          if (k < a.H && i < a.I) v = *(const uint32_t*)(a.W + (((int64_t)e * a.H + k) * 2 + gu) * a.I + i);
+        } else {
+          const int64_t h = c0 + col;
+          if (k < a.I && h < a.H) v = *(const uint32_t*)(a.W + ((int64_t)e * a.I_pad + k) * a.H + h);
+        }
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) sB[(col + cc) * LROW + kr] = (uint8_t)((v >> (8 * cc)) & 0xff);
+      }
+    }
+    __syncthreads();
+
+    // ---- MFMA ------------------------------------------------------------------------------
+    if (KIND == MOE_KIND_BF16) {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        v8bf af[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * LROW + sub * 64 + g * 16);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const v8bf bf = *(const v8bf*)(sB + (nt * 16 + c) * LROW + sub * 64 + g * 16);
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt)
+            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bf, acc[nt][mt], 0, 0, 0);
+        }
+      }
+    } else {
+      v8i af[2];
+      int sa[2];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const int row = m0 + 16 * mt + c;
+        af[mt] = lds_read32(sA + row * LROW + g * 32);
+        sa[mt] = (KIND == MOE_KIND_MXFP8) ? (int)((sAs[row] >> (8 * g)) & 0xffu) : 127;
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int col = nt * 16 + c;
+        const v8i bf = lds_read32(sB + col * LROW + g * 32);
+        const int sb = (KIND == MOE_KIND_MXFP8) ? (int)((sBs[col] >> (8 * g)) & 0xffu) : 127;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, sa[mt], 0, sb);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue ----------------------------------------------------------------------------
+  // accumulator element r of tile (nt, mt) is (row m0 + 16*mt + 4*g + r, column nt*16 + c)
+  if (STAGE == 1) {
+    const bool pre = (a.scaling_mode == MOE_SCALE_PRE || a.scaling_mode == MOE_SCALE_PRE_DELAYED);
+    if (KIND == MOE_KIND_MXFP8) {
+      uint8_t* Yq = (uint8_t*)a.out;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int p = p0 + 16 * half + c;
+        const bool pv = p < Pt;
+        float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
+        if (a.bias && pv) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            // bias [E, pI, 2, nI, 4]
+            bg[q] = load_bias(a.bias, a.bias_dtype, ((((int64_t)e * a.pI + p) * 2 + 0) * a.nI + tI) * 4 + q);
+            bu[q] = load_bias(a.bias, a.bias_dtype, ((((int64_t)e * a.pI + p) * 2 + 1) * a.nI + tI) * 4 + q);
+          }
+        }
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = m0 + 16 * mt + 4 * g + r;
+            float y[4];
+            float am = 0.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              float gv = acc[q * 2 + half][mt][r] + bg[q];
+              float uv = acc[8 + q * 2 + half][mt][r] + bu[q];
+              if (a.clamp_mask & MOE_CLAMP_GATE_LO) gv = fmaxf(gv, a.clamp[1]);
+              if (a.clamp_mask & MOE_CLAMP_GATE_HI) gv = fminf(gv, a.clamp[0]);
+              if (a.clamp_mask & MOE_CLAMP_UP_LO) uv = fmaxf(uv, a.clamp[3]);
+              if (a.clamp_mask & MOE_CLAMP_UP_HI) uv = fminf(uv, a.clamp[2]);
+              y[q] = pv ? act_apply(gv, a.act_fn) * uv : 0.f;
+              am = fmaxf(am, fabsf(y[q]));
+            }
+            // MX block = 8 consecutive partitions x 4 q: reduce over the 8-lane group
+            am = fmaxf(am, __shfl_xor(am, 1, 64));
+            am = fmaxf(am, __shfl_xor(am, 2, 64));
+            am = fmaxf(am, __shfl_xor(am, 4, 64));
+            const uint32_t sbyte = mx_scale_byte(am);
+            const float is = mx_inv_scale(sbyte);
+            const uint32_t dw = pack4_e4m3(clip448(y[0] * is), clip448(y[1] * is), clip448(y[2] * is), clip448(y[3] * is));
+            if (pv && r0 + row < vr) {
+              const int64_t slot = slot0 + row;
+              *(uint32_t*)(Yq + slot * a.out_stride + tI * 512 + p * 4) = dw;
+              if ((c & 7) == 0) a.out_scale[slot * a.out_scale_stride + tI * 16 + (p >> 3)] = (uint8_t)sbyte;
+            }
+          }
+        }
+      }
+    } else {
+      const float* wsc = (const float*)a.W_scale;
+      const int64_t wsb = (a.w_scale_experts > 1) ? (int64_t)e * 2 * a.I : 0;
+#pragma unroll
+      for (int nt = 0; nt < 8; ++nt) {
+        const int64_t i = c0 + nt * 16 + c;
+        const bool iv = i < a.I;
+        float sg = 1.f, su = 1.f, bg = 0.f, bu = 0.f;
+        if (iv && wsc) { sg = wsc[wsb + i]; su = wsc[wsb + a.I + i]; }
+        if (iv && a.bias) {
+          bg = load_bias(a.bias, a.bias_dtype, ((int64_t)e * 2 + 0) * a.I + i);
+          bu = load_bias(a.bias, a.bias_dtype, ((int64_t)e * 2 + 1) * a.I + i);
+        }
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = m0 + 16 * mt + 4 * g + r;
+            float gv = acc[nt][mt][r], uv = acc[nt + 8][mt][r];
+            if (KIND == MOE_KIND_BF16) {
+              if (pre) { gv *= s_aff[row]; uv *= s_aff[row]; }
+              gv *= sg; uv *= su;
+            } else {
+              const float rs = __uint_as_float(sAs[row]);
+              gv = (gv * sg) * rs; uv = (uv * su) * rs;
+            }
+            gv += bg; uv += bu;
+            if (a.clamp_mask & MOE_CLAMP_GATE_LO) gv = fmaxf(gv, a.clamp[1]);
+            if (a.clamp_mask & MOE_CLAMP_GATE_HI) gv = fminf(gv, a.clamp[0]);
+            if (a.clamp_mask & MOE_CLAMP_UP_LO) uv = fmaxf(uv, a.clamp[3]);
+            if (a.clamp_mask & MOE_CLAMP_UP_HI) uv = fminf(uv, a.clamp[2]);
+            const float y = iv ? act_apply(gv, a.act_fn) * uv : 0.f;
+            if (r0 + row < vr) {
+              const int64_t slot = slot0 + row;
+              if (KIND == MOE_KIND_BF16) {
+                if (i * 2 < a.out_stride) *(uint16_t*)((uint8_t*)a.out + slot * a.out_stride + i * 2) = f32_to_bf16_bits(y);
+              } else {
+                if (iv) *(float*)((uint8_t*)a.out + slot * a.out_stride + i * 4) = y;
+              }
+            }
+          }
+        }
+      }
+    }
+  } else {
+    uint16_t* D = (uint16_t*)a.out;
+    const float* wsc = (KIND == MOE_KIND_MXFP8) ? nullptr : (const float*)a.W_scale;
+    const int64_t wsb = (a.w_scale_experts > 1) ? (int64_t)e * a.H : 0;
+    const bool post = a.scaling_mode == MOE_SCALE_POST;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int64_t h = c0 + nt * 16 + c;
+      if (h >= a.H) continue;
+      const float sd = wsc ? wsc[wsb + h] : 1.f;
+      const float bd = a.bias ? load_bias(a.bias, a.bias_dtype, (int64_t)e * a.H + h) : 0.f;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = m0 + 16 * mt + 4 * g + r;
+          if (s_tok[row] < 0) continue;
+          float d = acc[nt][mt][r];
+          if (KIND == MOE_KIND_BF16) d *= sd;
+          if (KIND == MOE_KIND_FP8_ROW) d = (d * sd) * __uint_as_float(sAs[row]);
+          d += bd;
+          if (post) d *= s_aff[row];
+          D[(slot0 + row) * a.H + h] = f32_to_bf16_bits(d);
+        }
+      }
+    }
+  }
+}
+
+// Per-row fp8 re-quantisation of the fp8-row intermediate: scale = max(amax/240, 1e-5),
+// q = e4m3(y / scale)  (test_mlp_common.py:978-986).  One workgroup per slot row.
+__global__ __launch_bounds__(256) void row_requant_kernel(const float* __restrict__ Y, uint8_t* __restrict__ Yq,
+                                                          float* __restrict__ ys, const int32_t* __restrict__ n_active,
+                                                          const int32_t* __restrict__ valid_rows, int64_t B, int64_t I,
+                                                          int64_t Iw) {
+  __shared__ float red[16];
+  const int64_t slot = blockIdx.x;
+  const int64_t b = slot / B, r = slot % B;
+  if (b >= *n_active || r >= valid_rows[b]) return;
+  const float* y = Y + slot * I;
+  float am = 0.f;
+  for (int64_t i = threadIdx.x; i < I; i += blockDim.x) am = fmaxf(am, fabsf(y[i]));
+  am = block_max(am, red);
+  const float sc = fmaxf(am / 240.0f, 1e-05f);
+  if (threadIdx.x == 0) ys[slot] = sc;
+  uint8_t* q = Yq + slot * Iw;
+  for (int64_t i = (int64_t)threadIdx.x * 4; i < Iw; i += (int64_t)blockDim.x * 4) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = (i + k < I) ? y[i + k] / sc : 0.f;
+    *(uint32_t*)(q + i) = pack4_e4m3(v[0], v[1], v[2], v[3]);
+  }
+}
+
+template <int KIND, int STAGE>
+static int launch_gemm(const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s) {
+  if (gx == 0 || gy == 0) return MOE_OK;
+  hipLaunchKernelGGL((bwmm_kernel<KIND, STAGE>), dim3(gx, gy), dim3(GT), 0, s, g);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+int launch_gemm_stage(int kind, int stage, const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s) {
+  if (kind == MOE_KIND_BF16) return stage == 1 ? launch_gemm<MOE_KIND_BF16, 1>(g, gx, gy, s) : launch_gemm<MOE_KIND_BF16, 2>(g, gx, gy, s);
+  if (kind == MOE_KIND_FP8_ROW)
+    return stage == 1 ? launch_gemm<MOE_KIND_FP8_ROW, 1>(g, gx, gy, s) : launch_gemm<MOE_KIND_FP8_ROW, 2>(g, gx, gy, s);
+  return stage == 1 ? launch_gemm<MOE_KIND_MXFP8, 1>(g, gx, gy, s) : launch_gemm<MOE_KIND_MXFP8, 2>(g, gx, gy, s);
+}
+
+int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,
+                       int64_t Iw, hipStream_t s) {
+  hipLaunchKernelGGL(row_requant_kernel, dim3((unsigned)(N * B)), dim3(256), 0, s, Y, Yq, ys, k.n_active, k.valid_rows,
+                     B, I, Iw);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+}  // namespace moe

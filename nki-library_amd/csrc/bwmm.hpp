@@ -1,0 +1,44 @@
+// Kernel argument block and launch entry points of the blockwise expert GEMMs.
+#pragma once
+
+#include "combine.hpp"
+
+namespace moe {
+
+struct GemmArgs {
+  // A operand: stage 1 = hidden rows gathered by token id, stage 2 = intermediate rows by slot
+  const uint8_t* A;
+  int64_t a_stride;        // bytes between rows of A
+  const uint8_t* A_scale;  // MXFP8: uint8 [rows, a_scale_stride]; FP8_ROW stage 2: float [slots]
+  int64_t a_scale_stride;
+  int64_t K;               // BF16 / FP8_ROW: contraction length in elements (zero padded on the A side)
+  // B operand: expert weights in the reference layouts
+  const uint8_t* W;
+  const uint8_t* W_scale;  // MXFP8: uint8 E8M0; otherwise float per output channel (nullable)
+  int32_t w_scale_experts;
+  const void* bias;
+  int32_t bias_dtype;
+  const void* aff;
+  int32_t aff_dtype;
+  const int32_t* tp2id;
+  const int32_t* b2e;
+  const int32_t* n_active;
+  const int32_t* valid_rows;
+  // outputs
+  void* out;               // stage 1: intermediate rows; stage 2: bf16 contributions [N*B, H]
+  uint8_t* out_scale;      // MXFP8 stage 1: E8M0 scales of the intermediate
+  int64_t out_stride;      // stage 1: bytes per intermediate row
+  int64_t out_scale_stride;
+  int64_t T1, H, I, E, B, N, I_pad, n_real;
+  int32_t tiles_per_block;
+  int32_t weight_dtype;
+  int32_t act_fn, scaling_mode, clamp_mask;
+  float clamp[4];          // gate hi, gate lo, up hi, up lo
+  int32_t pI, nI;          // MXFP8: partitions per intermediate tile in the down weight, number of tiles
+};
+
+int launch_gemm_stage(int kind, int stage, const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s);
+int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,
+                       int64_t Iw, hipStream_t s);
+
+}  // namespace moe

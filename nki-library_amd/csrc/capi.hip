@@ -1,0 +1,211 @@
+// C ABI entry points of libmoe_gfx950.so that are not tied to one kernel file: error text,
+// device check, workspace planning and the blockwise-MoE driver.
+#include <string.h>
+
+#include "bwmm.hpp"
+
+using namespace moe;
+
+extern "C" int moe_rmsnorm_quant_mxfp8(const void*, int, const void*, int, void*, void*, void*, int64_t, int64_t, float,
+                                       int64_t, int, int, void*);
+
+extern "C" const char* moe_error_string(int code) {
+  switch (code) {
+    case MOE_OK: return "ok";
+    case MOE_E_BAD_ARG: return "bad argument (null pointer, negative size or unknown enum value)";
+    case MOE_E_BAD_SHAPE: return "shape violates a divisibility or range rule of this kernel";
+    case MOE_E_WORKSPACE: return "workspace missing or too small";
+    case MOE_E_LAUNCH: return "HIP launch failed";
+    case MOE_E_UNSUPPORTED: return "option not supported by the gfx950 implementation";
+    case MOE_E_NO_DEVICE: return "current HIP device is not gfx950";
+    default: return "unknown error code";
+  }
+}
+
+extern "C" int moe_abi_version(void) { return 1; }
+
+extern "C" int moe_check_device(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MOE_E_NO_DEVICE;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return MOE_E_NO_DEVICE;
+  return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? MOE_OK : MOE_E_NO_DEVICE;
+}
+
+namespace {
+
+inline size_t al256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct Plan {
+  size_t book, xq, xs, y, yq, ys, d, total;
+  int64_t Iw;      // padded intermediate width (elements) of the stage-2 A operand
+  int64_t pI, nI;  // MXFP8
+};
+
+int validate(const moe_bwmm_args* a) {
+  if (!a || !a->hidden_states || !a->gate_up_proj_weight || !a->down_proj_weight || !a->token_position_to_id ||
+      !a->block_to_expert || !a->output)
+    return MOE_E_BAD_ARG;
+  if (a->T1 <= 0 || a->H <= 0 || a->I <= 0 || a->E <= 0 || a->B <= 0 || a->N <= 0) return MOE_E_BAD_ARG;
+  if (a->kind < MOE_KIND_BF16 || a->kind > MOE_KIND_MXFP8) return MOE_E_BAD_ARG;
+  if (a->act_fn < MOE_ACT_SILU || a->act_fn > MOE_ACT_SWISH) return MOE_E_BAD_ARG;
+  if (a->scaling_mode < MOE_SCALE_NONE || a->scaling_mode > MOE_SCALE_PRE_DELAYED) return MOE_E_BAD_ARG;
+  if (a->scaling_mode != MOE_SCALE_NONE && !a->expert_affinities_masked) return MOE_E_BAD_ARG;
+  if (a->affinity_dtype != MOE_DT_BF16 && a->affinity_dtype != MOE_DT_FP32) return MOE_E_BAD_ARG;
+  if ((a->gate_and_up_proj_bias || a->down_proj_bias) && a->bias_dtype != MOE_DT_BF16 && a->bias_dtype != MOE_DT_FP32)
+    return MOE_E_BAD_ARG;
+  if (a->conditions && a->n_conditions <= 0) return MOE_E_BAD_ARG;
+  if (a->out_row_stride < a->H) return MOE_E_BAD_SHAPE;
+  if (a->E > COMBINE_MAX_K) return MOE_E_UNSUPPORTED;
+  if (a->N * a->B >= ((int64_t)1 << 31) || a->T1 * a->E >= ((int64_t)1 << 31)) return MOE_E_BAD_SHAPE;
+  const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
+  if (Ipad < a->I) return MOE_E_BAD_SHAPE;
+  switch (a->kind) {
+    case MOE_KIND_BF16:
+      if (a->H % 8 != 0) return MOE_E_BAD_SHAPE;  // 16-byte row slices of bf16 hidden states
+      if (a->weight_dtype != MOE_DT_BF16 && a->weight_dtype != MOE_DT_FP8_E4M3) return MOE_E_BAD_ARG;
+      if (a->weight_dtype == MOE_DT_FP8_E4M3 && (!a->gate_up_proj_scale || !a->down_proj_scale)) return MOE_E_BAD_ARG;
+      if ((a->gate_up_proj_scale != nullptr) != (a->down_proj_scale != nullptr)) return MOE_E_BAD_ARG;
+      if (a->gate_up_proj_scale && a->scale_experts != 1 && a->scale_experts != a->E) return MOE_E_BAD_SHAPE;
+      break;
+    case MOE_KIND_FP8_ROW:
+      if (a->H % 16 != 0 || a->I % 4 != 0) return MOE_E_BAD_SHAPE;
+      if (!a->gate_up_proj_scale || !a->down_proj_scale) return MOE_E_BAD_ARG;
+      if (a->scale_experts != 1 && a->scale_experts != a->E) return MOE_E_BAD_SHAPE;
+      if (a->scaling_mode == MOE_SCALE_PRE || a->scaling_mode == MOE_SCALE_PRE_DELAYED) return MOE_E_UNSUPPORTED;
+      if (a->clamp_mask) return MOE_E_UNSUPPORTED;
+      break;
+    case MOE_KIND_MXFP8: {
+      // bwmm_shard_on_block_mx.py:586-633, moe_cte_mx_utils.py:260-264
+      if (a->H % 512 != 0 || a->H < 512 || a->H > 16384) return MOE_E_BAD_SHAPE;
+      const int64_t tail = a->I % 512;
+      if (a->I % 16 != 0 || (tail != 0 && tail % 32 != 0)) return MOE_E_BAD_SHAPE;
+      if (!a->gate_up_proj_scale || !a->down_proj_scale) return MOE_E_BAD_ARG;
+      // POST_SCALE only (test_moe_bwmm_mx_cte.py:163-167)
+      if (a->scaling_mode == MOE_SCALE_PRE || a->scaling_mode == MOE_SCALE_PRE_DELAYED) return MOE_E_UNSUPPORTED;
+      break;
+    }
+  }
+  return MOE_OK;
+}
+
+Plan make_plan(const moe_bwmm_args* a) {
+  Plan p;
+  memset(&p, 0, sizeof(p));
+  const size_t slots = (size_t)(a->N * a->B);
+  size_t off = 0;
+  p.book = off; off += al256(bookkeeping_bytes(a->T1, a->N, a->B));
+  if (a->kind == MOE_KIND_MXFP8) {
+    p.nI = (a->I + 511) / 512;
+    p.pI = a->I > 512 ? 128 : a->I / 4;
+    p.Iw = p.nI * 512;
+    if (!a->hidden_states_scale) {
+      p.xq = off; off += al256((size_t)a->T1 * a->H);
+      p.xs = off; off += al256((size_t)a->T1 * (a->H / 32));
+    }
+    p.yq = off; off += al256(slots * (size_t)p.Iw);
+    p.ys = off; off += al256(slots * (size_t)(p.Iw / 32));
+  } else if (a->kind == MOE_KIND_BF16) {
+    p.Iw = (a->I + 63) / 64 * 64;
+    p.y = off; off += al256(slots * (size_t)p.Iw * 2);
+  } else {
+    p.Iw = (a->I + 127) / 128 * 128;
+    p.y = off; off += al256(slots * (size_t)a->I * 4);
+    p.yq = off; off += al256(slots * (size_t)p.Iw);
+    p.ys = off; off += al256(slots * 4);
+  }
+  p.d = off; off += al256(slots * (size_t)a->H * 2);
+  p.total = off;
+  return p;
+}
+
+}  // namespace
+
+extern "C" size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* a) {
+  if (validate(a) != MOE_OK) return 0;
+  return make_plan(a).total;
+}
+
+extern "C" int moe_blockwise(const moe_bwmm_args* a, void* stream) {
+  int rc = validate(a);
+  if (rc != MOE_OK) return rc;
+  const Plan p = make_plan(a);
+  if (!a->workspace || a->workspace_bytes < p.total) return MOE_E_WORKSPACE;
+  if (((uintptr_t)a->workspace & 255) != 0) return MOE_E_BAD_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  uint8_t* ws = (uint8_t*)a->workspace;
+  const int64_t n_real = a->skip_token ? a->T1 : a->T1 - 1;
+  const Bookkeeping bk = carve_bookkeeping(ws + p.book, a->T1, a->N, a->B);
+  rc = launch_prep(bk, a, n_real, s);
+  if (rc != MOE_OK) return rc;
+
+  GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.aff = a->scaling_mode == MOE_SCALE_NONE ? nullptr : a->expert_affinities_masked;
+  g.aff_dtype = a->affinity_dtype;
+  g.bias_dtype = a->bias_dtype;
+  g.tp2id = a->token_position_to_id;
+  g.b2e = a->block_to_expert;
+  g.n_active = bk.n_active;
+  g.valid_rows = bk.valid_rows;
+  g.T1 = a->T1; g.H = a->H; g.I = a->I; g.E = a->E; g.B = a->B; g.N = a->N;
+  g.I_pad = a->I_pad > 0 ? a->I_pad : a->I;
+  g.n_real = n_real;
+  g.tiles_per_block = (int32_t)((a->B + 127) / 128);
+  g.weight_dtype = a->weight_dtype;
+  g.act_fn = a->act_fn;
+  g.scaling_mode = a->scaling_mode;
+  g.clamp_mask = a->clamp_mask;
+  g.clamp[0] = a->gate_clamp_upper; g.clamp[1] = a->gate_clamp_lower;
+  g.clamp[2] = a->up_clamp_upper; g.clamp[3] = a->up_clamp_lower;
+  g.w_scale_experts = a->scale_experts;
+  g.pI = (int32_t)p.pI; g.nI = (int32_t)p.nI;
+  const unsigned gy = (unsigned)(a->N * g.tiles_per_block);
+
+  GemmArgs g1 = g, g2 = g;
+  g1.W = (const uint8_t*)a->gate_up_proj_weight;
+  g1.W_scale = (const uint8_t*)a->gate_up_proj_scale;
+  g1.bias = a->gate_and_up_proj_bias;
+  g2.W = (const uint8_t*)a->down_proj_weight;
+  g2.W_scale = (const uint8_t*)a->down_proj_scale;
+  g2.bias = a->down_proj_bias;
+  g2.out = ws + p.d;
+  unsigned gx1, gx2 = (unsigned)((a->H + 127) / 128);
+
+  if (a->kind == MOE_KIND_MXFP8) {
+    const uint8_t* xq = (const uint8_t*)a->hidden_states;
+    const uint8_t* xs = (const uint8_t*)a->hidden_states_scale;
+    if (!xs) {
+      // online activation quantisation (moe_cte_mx_utils.py:730-771): bf16 rows -> MXFP8 in k' order
+      rc = moe_rmsnorm_quant_mxfp8(a->hidden_states, MOE_DT_BF16, nullptr, MOE_DT_BF16, ws + p.xq, ws + p.xs, nullptr,
+                                   a->T1, a->H, 0.f, a->H, 0, MOE_MX_LAYOUT_TOKEN_MAJOR, stream);
+      if (rc != MOE_OK) return rc;
+      xq = ws + p.xq;
+      xs = ws + p.xs;
+    }
+    g1.A = xq; g1.a_stride = a->H; g1.A_scale = xs; g1.a_scale_stride = a->H / 32;
+    g1.out = ws + p.yq; g1.out_stride = p.Iw; g1.out_scale = ws + p.ys; g1.out_scale_stride = p.Iw / 32;
+    g2.A = ws + p.yq; g2.a_stride = p.Iw; g2.A_scale = ws + p.ys; g2.a_scale_stride = p.Iw / 32;
+    gx1 = (unsigned)(p.nI * 4);
+  } else if (a->kind == MOE_KIND_BF16) {
+    g1.A = (const uint8_t*)a->hidden_states; g1.a_stride = a->H * 2; g1.K = a->H;
+    g1.out = ws + p.y; g1.out_stride = p.Iw * 2;
+    g2.A = ws + p.y; g2.a_stride = p.Iw * 2; g2.K = p.Iw;
+    gx1 = (unsigned)((a->I + 127) / 128);
+  } else {
+    g1.A = (const uint8_t*)a->hidden_states; g1.a_stride = a->H + 4; g1.K = a->H;
+    g1.out = ws + p.y; g1.out_stride = a->I * 4;
+    g2.A = ws + p.yq; g2.a_stride = p.Iw; g2.K = p.Iw; g2.A_scale = ws + p.ys;
+    gx1 = (unsigned)((a->I + 127) / 128);
+  }
+
+  rc = launch_gemm_stage(a->kind, 1, g1, gx1, gy, s);
+  if (rc != MOE_OK) return rc;
+  if (a->kind == MOE_KIND_FP8_ROW) {
+    rc = launch_row_requant((const float*)(ws + p.y), ws + p.yq, (float*)(ws + p.ys), bk, a->N, a->B, a->I, p.Iw, s);
+    if (rc != MOE_OK) return rc;
+  }
+  rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);
+  if (rc != MOE_OK) return rc;
+  return launch_combine(bk, a, ws + p.d, n_real, s);
+}

@@ -1,0 +1,212 @@
+// Block bookkeeping and the affinity-weighted combine (scatter-add) for the blockwise MoE.
+//
+// The reference accumulates each block's bf16 contribution into the output rows with a
+// read-modify-write scatter in block order (bwmm_shard_on_block.py:1005-1038; golden
+// test_moe_cte_common.py:430-434).  On the GPU the down GEMM writes every slot's contribution
+// once (bf16, already multiplied by the affinity) and one pass per token then adds that
+// token's contributions in ascending slot order -- the same order and the same bf16
+// arithmetic as the golden, deterministic, and without atomics.  HBM traffic: each
+// contribution row is written once and read once, each output row written once.
+#include "combine.hpp"
+
+namespace moe {
+
+// n_active = index of the first zero in conditions (N when there is none / no conditions);
+// valid_rows[b] = 1 + last row of block b holding a real token id (0 for an all-padding block
+// or a block at/after n_active or with an expert id outside [0, E)).
+__global__ __launch_bounds__(256) void prep_blocks_kernel(const int32_t* __restrict__ tp2id,
+                                                          const int32_t* __restrict__ b2e,
+                                                          const int32_t* __restrict__ conditions, int64_t n_conditions,
+                                                          int64_t N, int64_t B, int64_t E, int64_t n_real,
+                                                          int32_t* __restrict__ n_active,
+                                                          int32_t* __restrict__ valid_rows) {
+  __shared__ int s_first_zero;
+  __shared__ int s_red[4];
+  if (threadIdx.x == 0) s_first_zero = (int)N;
+  __syncthreads();
+  if (conditions) {
+    const int64_t lim = n_conditions < N ? n_conditions : N;
+    for (int64_t i = threadIdx.x; i < lim; i += blockDim.x)
+      if (conditions[i] == 0) atomicMin(&s_first_zero, (int)i);
+  }
+  __syncthreads();
+  const int na = s_first_zero;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *n_active = na;
+  for (int64_t b = blockIdx.x; b < N; b += gridDim.x) {
+    int v = 0;
+    const int e = b2e[b];
+    if (b < na && e >= 0 && e < E) {
+      for (int64_t r = threadIdx.x; r < B; r += blockDim.x) {
+        const int id = tp2id[b * B + r];
+        if (id >= 0 && id < n_real) v = (int)r + 1;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) valid_rows[b] = max(max(s_red[0], s_red[1]), max(s_red[2], s_red[3]));
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* __restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void inv_count_kernel(const int32_t* __restrict__ tp2id,
+                                                        const int32_t* __restrict__ valid_rows, int64_t N, int64_t B,
+                                                        int64_t n_real, int32_t* __restrict__ cnt) {
+  const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= N * B) return;
+  const int64_t b = s / B, r = s % B;
+  if (r >= valid_rows[b]) return;
+  const int id = tp2id[s];
+  if (id >= 0 && id < n_real) atomicAdd(&cnt[id], 1);
+}
+
+// Exclusive scan of cnt[0..n) into off[0..n], single workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void inv_scan_kernel(const int32_t* __restrict__ cnt, int32_t* __restrict__ off,
+                                                        int64_t n) {
+  __shared__ int s_part[1024];
+  const int64_t per = (n + 1023) / 1024;
+  const int64_t lo = threadIdx.x * per, hi = (lo + per < n) ? lo + per : n;
+  int sum = 0;
+  for (int64_t i = lo; i < hi; ++i) sum += cnt[i];
+  s_part[threadIdx.x] = sum;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the 1024 partials
+  for (int o = 1; o < 1024; o <<= 1) {
+    int v = (threadIdx.x >= (unsigned)o) ? s_part[threadIdx.x - o] : 0;
+    __syncthreads();
+    s_part[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int run = s_part[threadIdx.x] - sum;
+  for (int64_t i = lo; i < hi; ++i) {
+    off[i] = run;
+    run += cnt[i];
+  }
+  if (threadIdx.x == 1023) off[n] = s_part[1023];
+}
+
+__global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict__ tp2id,
+                                                       const int32_t* __restrict__ valid_rows, int64_t N, int64_t B,
+                                                       int64_t n_real, const int32_t* __restrict__ off,
+                                                       int32_t* __restrict__ cursor, int32_t* __restrict__ list) {
+  const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= N * B) return;
+  const int64_t b = s / B, r = s % B;
+  if (r >= valid_rows[b]) return;
+  const int id = tp2id[s];
+  if (id >= 0 && id < n_real) {
+    const int p = atomicAdd(&cursor[id], 1);
+    list[off[id] + p] = (int32_t)s;
+  }
+}
+
+// One workgroup per output row.  D: bf16 [N*B, H] contributions.
+__global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict__ D, const int32_t* __restrict__ off,
+                                                      const int32_t* __restrict__ list, uint16_t* __restrict__ out,
+                                                      int64_t out_row_stride, int64_t H, int64_t n_real) {
+  __shared__ int s_sorted[COMBINE_MAX_K];
+  const int64_t t = blockIdx.x;
+  int cnt = 0, base = 0;
+  if (t < n_real) {
+    base = off[t];
+    cnt = off[t + 1] - base;
+    if (cnt > COMBINE_MAX_K) cnt = COMBINE_MAX_K;  // rejected on the host: a token has at most E <= MAX_K slots
+  }
+  // rank sort: ascending slot index == block order of the reference's accumulation
+  for (int i = threadIdx.x; i < cnt; i += blockDim.x) {
+    const int mine = list[base + i];
+    int rank = 0;
+    for (int j = 0; j < cnt; ++j) rank += (list[base + j] < mine);
+    s_sorted[rank] = mine;
+  }
+  __syncthreads();
+  uint16_t* orow = out + t * out_row_stride;
+  const bool vec = (H % 8 == 0) && ((out_row_stride % 8) == 0) && (((uintptr_t)out & 15) == 0);
+  if (vec) {
+    for (int64_t c = (int64_t)threadIdx.x * 8; c < H; c += (int64_t)blockDim.x * 8) {
+      float acc[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+      for (int j = 0; j < cnt; ++j) {
+        const uint4 d = *(const uint4*)(D + (int64_t)s_sorted[j] * H + c);
+        const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          acc[2 * k] = round_to_bf16(acc[2 * k] + bf16_bits_to_f32((uint16_t)(w[k] & 0xffff)));
+          acc[2 * k + 1] = round_to_bf16(acc[2 * k + 1] + bf16_bits_to_f32((uint16_t)(w[k] >> 16)));
+        }
+      }
+      uint32_t o[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        o[k] = (uint32_t)f32_to_bf16_bits(acc[2 * k]) | ((uint32_t)f32_to_bf16_bits(acc[2 * k + 1]) << 16);
+      *(uint4*)(orow + c) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
+      float acc = 0.f;
+      for (int j = 0; j < cnt; ++j) acc = round_to_bf16(acc + bf16_bits_to_f32(D[(int64_t)s_sorted[j] * H + c]));
+      orow[c] = f32_to_bf16_bits(acc);
+    }
+  }
+}
+
+// ---- host-side orchestration used by moe_blockwise() -------------------------------------
+
+size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B) {
+  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B], each region 256-byte aligned
+  auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  return al(16) + al((size_t)N * 4) + 2 * al((size_t)T1 * 4) + al((size_t)(T1 + 1) * 4) + al((size_t)N * B * 4);
+}
+
+Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
+  auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  Bookkeeping k;
+  uint8_t* p = (uint8_t*)base;
+  k.n_active = (int32_t*)p; p += al(16);
+  k.valid_rows = (int32_t*)p; p += al((size_t)N * 4);
+  k.cnt = (int32_t*)p; p += al((size_t)T1 * 4);
+  k.cursor = (int32_t*)p; p += al((size_t)T1 * 4);
+  k.off = (int32_t*)p; p += al((size_t)(T1 + 1) * 4);
+  k.list = (int32_t*)p;
+  return k;
+}
+
+int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hipStream_t s) {
+  // cnt and cursor are adjacent: one clear covers both.  A fill kernel rather than a memset
+  // node, so that the sequence stays safe to record into a HIP graph.
+  const int64_t clear_words = (int64_t)((uint8_t*)k.off - (uint8_t*)k.cnt) / 4;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((clear_words + 255) / 256)), dim3(256), 0, s, k.cnt,
+                     clear_words);
+  MOE_CHECK_LAUNCH();
+  const unsigned g = (unsigned)(a->N < 1024 ? a->N : 1024);
+  hipLaunchKernelGGL(prep_blocks_kernel, dim3(g), dim3(256), 0, s, a->token_position_to_id, a->block_to_expert,
+                     a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows);
+  MOE_CHECK_LAUNCH();
+  const int64_t slots = a->N * a->B;
+  const unsigned gs = (unsigned)((slots + 255) / 256);
+  hipLaunchKernelGGL(inv_count_kernel, dim3(gs), dim3(256), 0, s, a->token_position_to_id, k.valid_rows, a->N, a->B,
+                     n_real, k.cnt);
+  MOE_CHECK_LAUNCH();
+  hipLaunchKernelGGL(inv_scan_kernel, dim3(1), dim3(1024), 0, s, k.cnt, k.off, n_real);
+  MOE_CHECK_LAUNCH();
+  hipLaunchKernelGGL(inv_fill_kernel, dim3(gs), dim3(256), 0, s, a->token_position_to_id, k.valid_rows, a->N, a->B,
+                     n_real, k.off, k.cursor, k.list);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, int64_t n_real, hipStream_t s) {
+  hipLaunchKernelGGL(combine_kernel, dim3((unsigned)a->T1), dim3(256), 0, s, (const uint16_t*)D, k.off, k.list,
+                     (uint16_t*)a->output, a->out_row_stride, a->H, n_real);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+}  // namespace moe

@@ -1,0 +1,25 @@
+// Block bookkeeping shared by the blockwise MoE driver and the combine kernels.
+#pragma once
+
+#include "common.hpp"
+
+namespace moe {
+
+constexpr int COMBINE_MAX_K = 512;  // most slots one token may own (one per expert it selected)
+
+struct Bookkeeping {
+  int32_t* n_active;    // [1]  blocks before the first conditions[b] == 0
+  int32_t* valid_rows;  // [N]  rows of block b up to and including its last real token
+  int32_t* cnt;         // [T1] slots per token
+  int32_t* cursor;      // [T1]
+  int32_t* off;         // [T1+1] exclusive scan of cnt
+  int32_t* list;        // [N*B] slot indices grouped by token
+};
+
+size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B);
+Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B);
+// n_real: number of real token rows (ids in [0, n_real) are tokens, everything else is padding).
+int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hipStream_t s);
+int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, int64_t n_real, hipStream_t s);
+
+}  // namespace moe

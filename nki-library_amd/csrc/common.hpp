@@ -1,0 +1,132 @@
+// Shared device/host helpers for the gfx950 MoE kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "moe_gfx950.h"
+
+#define MOE_CHECK_LAUNCH()                           \
+  do {                                               \
+    hipError_t e__ = hipGetLastError();              \
+    if (e__ != hipSuccess) return MOE_E_LAUNCH;      \
+  } while (0)
+
+namespace moe {
+
+constexpr int WAVE = 64;
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+// ---- bf16 <-> fp32 (bit level, round-to-nearest-even) ---------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+__device__ __forceinline__ float fp16_bits_to_f32(uint16_t b) {
+  _Float16 h;
+  __builtin_memcpy(&h, &b, 2);
+  return (float)h;
+}
+
+// Generic scalar load of element i of a tensor of runtime dtype.
+__device__ __forceinline__ float load_as_f32(const void* p, int dtype, int64_t i) {
+  if (dtype == MOE_DT_BF16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+  if (dtype == MOE_DT_FP16) return fp16_bits_to_f32(((const uint16_t*)p)[i]);
+  return ((const float*)p)[i];
+}
+
+// ---- fp8 e4m3fn (OCP) -----------------------------------------------------------------
+// Packs two floats (already clipped by the caller) to two e4m3fn bytes, RNE.
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  return (uint32_t)r;
+}
+
+// Exact decode of one e4m3fn byte.
+__device__ __forceinline__ float e4m3_to_f32(uint32_t byte) {
+  uint32_t s = (byte & 0x80u) << 24;
+  uint32_t em = byte & 0x7fu;
+  float v;
+  if ((em >> 3) == 0) {
+    v = (float)em * 0.001953125f;  // subnormal: m * 2^-9
+  } else {
+    v = __uint_as_float((em << 20) + (120u << 23));  // rebias 7 -> 127
+  }
+  return __uint_as_float(__float_as_uint(v) | s);
+}
+
+// ---- reductions ------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide sum / max over blockDim.x threads (multiple of 64, <= 1024). `red` holds 16 floats.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+// ---- activation functions (ActFnType, common_types.py:32-36) ---------------------------
+__device__ __forceinline__ float act_apply(float x, int kind) {
+  switch (kind) {
+    case MOE_ACT_SILU:
+      return x / (1.0f + expf(-x));
+    case MOE_ACT_GELU:
+      return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+    case MOE_ACT_GELU_TANH: {
+      const float c = 0.79788456080286535588f;
+      return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+    }
+    default:  // MOE_ACT_SWISH: x * sigmoid(1.702 x)
+      return x / (1.0f + expf(-1.702f * x));
+  }
+}
+
+// E8M0 scale byte for a block whose largest magnitude is amax (e4m3 target, max exponent 8),
+// and the exact power-of-two multiplier 2^(127 - scale) that divides by the block scale.
+__device__ __forceinline__ uint32_t mx_scale_byte(float amax) {
+  int e = (int)((__float_as_uint(amax) >> 23) & 0xffu);
+  int s = e - 8;
+  return (uint32_t)(s < 0 ? 0 : s);
+}
+__device__ __forceinline__ float mx_inv_scale(uint32_t sbyte) { return __uint_as_float((254u - sbyte) << 23); }
+
+__device__ __forceinline__ float clip448(float v) { return fminf(fmaxf(v, -448.0f), 448.0f); }
+
+}  // namespace moe

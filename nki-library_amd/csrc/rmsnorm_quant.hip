@@ -1,0 +1,297 @@
+// Fused RMSNorm + quantise front end for gfx950: fp8-e4m3 per-row / static scale, and MXFP8.
+//
+// One 256-thread workgroup owns one row; the row is read once (16-byte coalesced loads),
+// kept in registers across the two reductions (sum of squares, absolute maximum) and written
+// once.  HBM traffic per row is the algorithmic minimum: 2H bytes in, H (+4 or +H/32) out.
+//
+// The fp32 arithmetic follows the reference goldens operation by operation (no FMA
+// contraction) so that quantised codes are reproducible:
+//   ROW / STATIC: test/integration/nkilib/core/rmsnorm/test_rmsnorm_quant.py:46-97
+//   MX:           test/integration/nkilib/core/subkernels/test_rmsnorm_mx_quantize_tkg.py:100-137,
+//                 rms_norm test/integration/nkilib/utils/test_kernel_common.py:26-41,
+//                 quantise rule test/utils/mx_utils.py:55-95
+#include "common.hpp"
+
+#pragma clang fp contract(off)
+
+namespace moe {
+
+constexpr int RQ_THREADS = 256;
+constexpr int RQ_MAX_H = 16384;                       // rmsnorm_quant_constants.py:60-62 (MAX_H)
+constexpr int RQ_MAX_CHUNKS = RQ_MAX_H / (RQ_THREADS * 8);  // 8-element chunks per thread
+
+// Loads 8 consecutive elements starting at element index i (i % 8 == 0, i + 8 <= n guaranteed
+// by the caller when `full`), converting to fp32.
+__device__ __forceinline__ void load8(const void* base, int dtype, int64_t i, int64_t n, bool vec_ok, float* v) {
+  if (dtype == MOE_DT_FP32) {
+    const float* p = (const float*)base + i;
+    if (vec_ok && i + 8 <= n) {
+      float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = (i + k < n) ? p[k] : 0.f;
+    }
+  } else {
+    const uint16_t* p = (const uint16_t*)base + i;
+    uint16_t h[8];
+    if (vec_ok && i + 8 <= n) {
+      uint4 a = *(const uint4*)p;
+      h[0] = a.x & 0xffff; h[1] = a.x >> 16; h[2] = a.y & 0xffff; h[3] = a.y >> 16;
+      h[4] = a.z & 0xffff; h[5] = a.z >> 16; h[6] = a.w & 0xffff; h[7] = a.w >> 16;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) h[k] = (i + k < n) ? p[k] : (uint16_t)0;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = (dtype == MOE_DT_BF16) ? bf16_bits_to_f32(h[k]) : fp16_bits_to_f32(h[k]);
+  }
+}
+
+// MODE 0: per-row scale appended to the row ([H+4] record).  MODE 1: static scale.
+template <int MODE>
+__global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
+    const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
+    const float* __restrict__ static_scale, uint8_t* __restrict__ out, int64_t H, int64_t out_stride, float eps,
+    float lower_bound, int do_norm, int vec_ok) {
+  __shared__ float red[16];
+  const int64_t row = blockIdx.x;
+  const int es = (x_dtype == MOE_DT_FP32) ? 4 : 2;
+  const void* xr = (const uint8_t*)x + row * H * es;
+  const int nchunk = (int)((H + RQ_THREADS * 8 - 1) / (RQ_THREADS * 8));
+
+  float v[RQ_MAX_CHUNKS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < RQ_MAX_CHUNKS; ++j) {
+    if (j < nchunk) {
+      const int64_t i = ((int64_t)j * RQ_THREADS + threadIdx.x) * 8;
+      if (i < H) {
+        load8(xr, x_dtype, i, H, vec_ok, v[j]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[j][k] = 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) ss += v[j][k] * v[j][k];
+    }
+  }
+
+  if (do_norm) {
+    const float total = block_sum(ss, red);
+    const float mean = total / (float)H;
+    const float rms = sqrtf(mean);
+    const float inv = 1.0f / (rms + eps);
+#pragma unroll
+    for (int j = 0; j < RQ_MAX_CHUNKS; ++j) {
+      if (j < nchunk) {
+        const int64_t i = ((int64_t)j * RQ_THREADS + threadIdx.x) * 8;
+        if (i < H) {
+          float g[8];
+          load8(gamma, gamma_dtype, i, H, vec_ok, g);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) v[j][k] = (v[j][k] * inv) * g[k];
+        }
+      }
+    }
+  }
+
+  float qs;  // multiplier applied before the cast
+  if (MODE == 0) {
+    float am = 0.f;
+#pragma unroll
+    for (int j = 0; j < RQ_MAX_CHUNKS; ++j)
+      if (j < nchunk) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) am = fmaxf(am, fabsf(v[j][k]));
+      }
+    am = block_max(am, red);
+    if (lower_bound > 0.f) am = fminf(am, lower_bound);
+    float dq = am / 240.0f;
+    dq = fmaxf(dq, 1e-6f);  // rmsnorm_quant.py:597-604
+    qs = 1.0f / dq;
+    if (threadIdx.x == 0) {
+      uint32_t bits = __float_as_uint(dq);
+      uint8_t* sp = out + row * out_stride + H;
+      sp[0] = bits & 0xff; sp[1] = (bits >> 8) & 0xff; sp[2] = (bits >> 16) & 0xff; sp[3] = (bits >> 24) & 0xff;
+    }
+  } else {
+    qs = 1.0f / static_scale[0];
+  }
+
+  uint8_t* orow = out + row * out_stride;
+  const bool st4 = ((out_stride & 3) == 0) && ((((uintptr_t)out) & 3) == 0);
+#pragma unroll
+  for (int j = 0; j < RQ_MAX_CHUNKS; ++j) {
+    if (j < nchunk) {
+      const int64_t i = ((int64_t)j * RQ_THREADS + threadIdx.x) * 8;
+      if (i < H) {
+        float q[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float t = v[j][k];
+          if (MODE == 0) {
+            if (lower_bound > 0.f) t = fminf(fmaxf(t, -lower_bound), lower_bound);
+            q[k] = t * qs;
+          } else {
+            q[k] = fminf(fmaxf(t * qs, -240.0f), 240.0f);
+          }
+        }
+        const uint32_t lo = pack4_e4m3(q[0], q[1], q[2], q[3]);
+        const uint32_t hi = pack4_e4m3(q[4], q[5], q[6], q[7]);
+        if (st4 && i + 8 <= H) {
+          *(uint32_t*)(orow + i) = lo;
+          *(uint32_t*)(orow + i + 4) = hi;
+        } else {
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (i + k < H) orow[i + k] = (uint8_t)(((k < 4 ? lo : hi) >> (8 * (k & 3))) & 0xff);
+        }
+      }
+    }
+  }
+}
+
+// MXFP8 front end.  Thread t of the row's workgroup owns MX blocks blk = t and t + 256
+// (blk = tile*16 + p8 covers k' in [blk*32, blk*32+32)); its 32 inputs are four runs of 8
+// contiguous elements at h = q*(H/4) + tile*128 + p8*8 + r.
+constexpr int MXQ_MAX_BLK = RQ_MAX_H / 32 / RQ_THREADS;  // 2
+
+__global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
+    const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
+    uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, uint16_t* __restrict__ out_norm, int64_t rows,
+    int64_t H, float eps, float hidden_actual, int do_norm, int layout) {
+  __shared__ float red[16];
+  const int64_t row = blockIdx.x;
+  const int es = (x_dtype == MOE_DT_FP32) ? 4 : 2;
+  const void* xr = (const uint8_t*)x + row * H * es;
+  const int nblk = (int)(H / 32);
+  const int nT = (int)(H / 512);
+  const int64_t Hq = H / 4;
+
+  float v[MXQ_MAX_BLK][4][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < MXQ_MAX_BLK; ++j) {
+    const int blk = j * RQ_THREADS + threadIdx.x;
+    if (blk < nblk) {
+      const int tile = blk >> 4, p8 = blk & 15;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        load8(xr, x_dtype, q * Hq + tile * 128 + p8 * 8, H, true, v[j][q]);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) ss += v[j][q][r] * v[j][q][r];
+      }
+    }
+  }
+  float inv = 1.0f;
+  if (do_norm) {
+    const float total = block_sum(ss, red);
+    const float rms = sqrtf(total / hidden_actual + eps);
+    inv = 1.0f / rms;
+  }
+#pragma unroll
+  for (int j = 0; j < MXQ_MAX_BLK; ++j) {
+    const int blk = j * RQ_THREADS + threadIdx.x;
+    if (blk < nblk) {
+      const int tile = blk >> 4, p8 = blk & 15;
+      float am = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float g[8];
+        if (do_norm) load8(gamma, gamma_dtype, q * Hq + tile * 128 + p8 * 8, H, true, g);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          float t = v[j][q][r];
+          if (do_norm) t = (t * inv) * g[r];
+          t = round_to_bf16(t);
+          v[j][q][r] = t;
+          am = fmaxf(am, fabsf(t));
+        }
+      }
+      if (out_norm != nullptr) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            const int64_t p = p8 * 8 + r, h1 = (int64_t)q * nT + tile;
+            out_norm[(p * rows + row) * (H / 128) + h1] = f32_to_bf16_bits(v[j][q][r]);
+          }
+      }
+      const uint32_t sb = mx_scale_byte(am);
+      const float is = mx_inv_scale(sb);
+      uint32_t d[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r)
+        d[r] = pack4_e4m3(clip448(v[j][0][r] * is), clip448(v[j][1][r] * is), clip448(v[j][2][r] * is),
+                          clip448(v[j][3][r] * is));
+      if (layout == MOE_MX_LAYOUT_TOKEN_MAJOR) {
+        uint4* o = (uint4*)(out_q + row * H + (int64_t)blk * 32);
+        o[0] = make_uint4(d[0], d[1], d[2], d[3]);
+        o[1] = make_uint4(d[4], d[5], d[6], d[7]);
+        out_scale[row * nblk + blk] = (uint8_t)sb;
+      } else {
+        uint32_t* o = (uint32_t*)out_q;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) o[((int64_t)(p8 * 8 + r) * nT + tile) * rows + row] = d[r];
+        const int srow = (layout == MOE_MX_LAYOUT_REF_DENSE) ? p8 : ((p8 >> 2) * 32 + (p8 & 3));
+        out_scale[((int64_t)srow * nT + tile) * rows + row] = (uint8_t)sb;
+      }
+    }
+  }
+}
+
+static bool valid_in_dtype(int d) { return d == MOE_DT_BF16 || d == MOE_DT_FP16 || d == MOE_DT_FP32; }
+
+}  // namespace moe
+
+using namespace moe;
+
+extern "C" int moe_rmsnorm_quant_fp8_row(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out,
+                                         int64_t rows, int64_t H, float eps, float lower_bound, int do_norm,
+                                         void* stream) {
+  if (!x || !out || rows < 0 || H <= 0 || !valid_in_dtype(x_dtype)) return MOE_E_BAD_ARG;
+  if (do_norm && (!gamma || !valid_in_dtype(gamma_dtype))) return MOE_E_BAD_ARG;
+  if (lower_bound < 0.f || eps < 0.f) return MOE_E_BAD_ARG;
+  if (H > RQ_MAX_H) return MOE_E_BAD_SHAPE;
+  if (rows == 0) return MOE_OK;
+  const int vec_ok = (H % 8 == 0) && (((uintptr_t)x & 15) == 0) && (!do_norm || ((uintptr_t)gamma & 15) == 0);
+  hipLaunchKernelGGL(rmsnorm_quant_fp8_kernel<0>, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
+                     x_dtype, gamma, gamma_dtype, (const float*)nullptr, (uint8_t*)out, H, H + 4, eps, lower_bound,
+                     do_norm, vec_ok);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+extern "C" int moe_rmsnorm_quant_fp8_static(const void* x, int x_dtype, const void* gamma, int gamma_dtype,
+                                            const float* input_dequant_scale, void* out, int64_t rows, int64_t H,
+                                            float eps, int do_norm, void* stream) {
+  if (!x || !out || !input_dequant_scale || rows < 0 || H <= 0 || !valid_in_dtype(x_dtype)) return MOE_E_BAD_ARG;
+  if (do_norm && (!gamma || !valid_in_dtype(gamma_dtype))) return MOE_E_BAD_ARG;
+  if (eps < 0.f) return MOE_E_BAD_ARG;
+  if (H > RQ_MAX_H) return MOE_E_BAD_SHAPE;
+  if (rows == 0) return MOE_OK;
+  const int vec_ok = (H % 8 == 0) && (((uintptr_t)x & 15) == 0) && (!do_norm || ((uintptr_t)gamma & 15) == 0);
+  hipLaunchKernelGGL(rmsnorm_quant_fp8_kernel<1>, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
+                     x_dtype, gamma, gamma_dtype, input_dequant_scale, (uint8_t*)out, H, H, eps, 0.f, do_norm, vec_ok);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out_q,
+                                       void* out_scale, void* out_norm, int64_t rows, int64_t H, float eps,
+                                       int64_t hidden_actual, int do_norm, int layout, void* stream) {
+  if (!x || !out_q || !out_scale || rows < 0 || H <= 0 || !valid_in_dtype(x_dtype)) return MOE_E_BAD_ARG;
+  if (do_norm && (!gamma || !valid_in_dtype(gamma_dtype))) return MOE_E_BAD_ARG;
+  if (layout < 0 || layout > 2 || eps < 0.f) return MOE_E_BAD_ARG;
+  if (H % 512 != 0 || H > RQ_MAX_H) return MOE_E_BAD_SHAPE;
+  if (((uintptr_t)x & 15) != 0 || ((uintptr_t)out_q & 15) != 0 || (do_norm && ((uintptr_t)gamma & 15) != 0))
+    return MOE_E_BAD_ARG;
+  if (rows == 0) return MOE_OK;
+  const float ha = (float)(hidden_actual > 0 ? hidden_actual : H);
+  hipLaunchKernelGGL(rmsnorm_quant_mx_kernel, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
+                     x_dtype, gamma, gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H,
+                     eps, ha, do_norm, layout);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}

@@ -1,0 +1,145 @@
+"""Shared host driver of the blockwise MoE kernels: validates tensors the way the
+reference kernels do (kernel_assert), allocates the output in the reference's
+return shape, and calls ``moe_blockwise`` of libmoe_gfx950.so."""
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .... import _native as nv
+from ...utils.common_types import ActFnType, ExpertAffinityScaleMode
+from ...utils.kernel_assert import kernel_assert
+from .moe_cte_utils import SkipMode
+
+
+def _f8_or_u8(t):
+    return t.dtype in (torch.uint8, torch.float8_e4m3fn, torch.int8)
+
+
+def run_blockwise(
+    kind: int,
+    hidden_states: torch.Tensor,
+    expert_affinities_masked: torch.Tensor,
+    gate_up_proj_weight: torch.Tensor,
+    down_proj_weight: torch.Tensor,
+    token_position_to_id: torch.Tensor,
+    block_to_expert: torch.Tensor,
+    block_size: int,
+    out_shape_kind: str,
+    dims: dict,
+    conditions: Optional[torch.Tensor] = None,
+    gate_and_up_proj_bias: Optional[torch.Tensor] = None,
+    down_proj_bias: Optional[torch.Tensor] = None,
+    gate_up_proj_scale: Optional[torch.Tensor] = None,
+    down_proj_scale: Optional[torch.Tensor] = None,
+    hidden_states_scale: Optional[torch.Tensor] = None,
+    activation_function: ActFnType = ActFnType.SiLU,
+    skip_dma: SkipMode = None,
+    expert_affinities_scaling_mode: ExpertAffinityScaleMode = ExpertAffinityScaleMode.POST_SCALE,
+    gate_clamp_upper_limit: Optional[float] = None,
+    gate_clamp_lower_limit: Optional[float] = None,
+    up_clamp_upper_limit: Optional[float] = None,
+    up_clamp_lower_limit: Optional[float] = None,
+    weight_dtype: int = nv.DT_BF16,
+    scale_experts: int = 0,
+):
+    """dims: T1, H, I, E, I_pad.  out_shape_kind: "T2H" ([T1,2,H], slot 0), "2TH" ([2,T1,H], slot 0) or "TH"."""
+    L = nv.lib()
+    skip_dma = skip_dma or SkipMode(False, False)
+    T1, H, I, E = dims["T1"], dims["H"], dims["I"], dims["E"]
+    B = int(block_size)
+    dev = hidden_states.device
+    kernel_assert(B > 0, f"block_size must be positive, got {B}")
+
+    tp2id = nv.require_device_tensor(token_position_to_id, "token_position_to_id").reshape(-1)
+    kernel_assert(tp2id.dtype == torch.int32, f"token_position_to_id must be int32 but got {tp2id.dtype}")
+    kernel_assert(tp2id.numel() % B == 0, f"token_position_to_id length {tp2id.numel()} is not a multiple of B={B}")
+    N = tp2id.numel() // B
+    b2e = nv.require_device_tensor(block_to_expert, "block_to_expert").reshape(-1)
+    kernel_assert(b2e.dtype == torch.int32, f"block_to_expert must be int32 but got {b2e.dtype}")
+    kernel_assert(b2e.numel() == N, f"block_to_expert must have N={N} entries but got {b2e.numel()}")
+    cond = None
+    if conditions is not None:
+        cond = nv.require_device_tensor(conditions, "conditions").reshape(-1)
+        kernel_assert(cond.dtype == torch.int32, f"conditions must be int32 but got {cond.dtype}")
+
+    aff = None
+    if expert_affinities_scaling_mode != ExpertAffinityScaleMode.NO_SCALE:
+        aff = nv.require_device_tensor(expert_affinities_masked, "expert_affinities_masked")
+        kernel_assert(aff.numel() == T1 * E, f"expert_affinities_masked must hold (T+1)*E={T1 * E} values, got {aff.numel()}")
+        kernel_assert(aff.dtype in (torch.bfloat16, torch.float32),
+                      f"expert_affinities_masked must be bfloat16 or float32 but got {aff.dtype}")
+    bias_dt = nv.DT_BF16
+    gub = db = None
+    if gate_and_up_proj_bias is not None or down_proj_bias is not None:
+        kernel_assert(gate_and_up_proj_bias is not None and down_proj_bias is not None,
+                      "gate_and_up_proj_bias and down_proj_bias must be given together")
+        gub = nv.require_device_tensor(gate_and_up_proj_bias, "gate_and_up_proj_bias")
+        db = nv.require_device_tensor(down_proj_bias, "down_proj_bias")
+        kernel_assert(gub.dtype == db.dtype and gub.dtype in (torch.bfloat16, torch.float32),
+                      "bias tensors must both be bfloat16 or both float32")
+        bias_dt = nv.DT_BF16 if gub.dtype == torch.bfloat16 else nv.DT_FP32
+        kernel_assert(db.numel() == E * H, f"down_proj_bias must be [E, H] but got {tuple(db.shape)}")
+
+    if out_shape_kind == "T2H":
+        out = torch.zeros((T1, 2, H), dtype=torch.bfloat16, device=dev)
+        stride = 2 * H
+    elif out_shape_kind == "2TH":
+        out = torch.zeros((2, T1, H), dtype=torch.bfloat16, device=dev)
+        stride = H
+    else:
+        out = torch.zeros((T1, H), dtype=torch.bfloat16, device=dev)
+        stride = H
+
+    a = nv.BwmmArgs()
+    a.hidden_states = nv.ptr(hidden_states)
+    a.hidden_states_scale = nv.ptr(hidden_states_scale)
+    a.expert_affinities_masked = nv.ptr(aff)
+    a.gate_up_proj_weight = nv.ptr(gate_up_proj_weight)
+    a.down_proj_weight = nv.ptr(down_proj_weight)
+    a.gate_up_proj_scale = nv.ptr(gate_up_proj_scale)
+    a.down_proj_scale = nv.ptr(down_proj_scale)
+    a.gate_and_up_proj_bias = nv.ptr(gub)
+    a.down_proj_bias = nv.ptr(db)
+    a.token_position_to_id = nv.ptr(tp2id)
+    a.block_to_expert = nv.ptr(b2e)
+    a.conditions = nv.ptr(cond)
+    a.output = nv.ptr(out)
+    a.T1, a.H, a.I, a.E, a.B, a.N = T1, H, I, E, B, N
+    a.I_pad = dims.get("I_pad", I)
+    a.n_conditions = cond.numel() if cond is not None else 0
+    a.out_row_stride = stride
+    a.scale_experts = scale_experts
+    a.kind = kind
+    a.weight_dtype = weight_dtype
+    a.affinity_dtype = nv.DT_FP32 if (aff is not None and aff.dtype == torch.float32) else nv.DT_BF16
+    a.bias_dtype = bias_dt
+    a.act_fn = activation_function.value
+    a.scaling_mode = expert_affinities_scaling_mode.value
+    a.skip_token = 1 if skip_dma.skip_token else 0
+    mask = 0
+    for bit, v, name in (
+        (nv.CLAMP_GATE_HI, gate_clamp_upper_limit, "gate_clamp_upper"),
+        (nv.CLAMP_GATE_LO, gate_clamp_lower_limit, "gate_clamp_lower"),
+        (nv.CLAMP_UP_HI, up_clamp_upper_limit, "up_clamp_upper"),
+        (nv.CLAMP_UP_LO, up_clamp_lower_limit, "up_clamp_lower"),
+    ):
+        if v is not None:
+            mask |= bit
+            setattr(a, name, float(v))
+    a.clamp_mask = mask
+
+    need = L.moe_blockwise_workspace_bytes(ctypes.byref(a))
+    if need == 0:
+        # validation failed inside the library: run the call to obtain the precise code
+        a.workspace = None
+        a.workspace_bytes = 0
+        nv.check(L.moe_blockwise(ctypes.byref(a), None) or -2, "moe_cte")
+    ws = nv.workspace(dev, need)
+    a.workspace = nv.ptr(ws)
+    a.workspace_bytes = ws.numel()
+    with torch.cuda.device(dev):
+        rc = L.moe_blockwise(ctypes.byref(a), nv.stream_ptr(dev))
+    nv.check(rc, "moe_cte")
+    return out

@@ -1,0 +1,53 @@
+"""Token -> block index construction on the GPU.
+
+The reference builds ``token_position_to_id`` / ``block_to_expert`` / ``conditions`` on the
+host in its test helper ``generate_token_position_to_id_and_experts``
+(test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:199-264); callers of
+``moe_cte`` must produce exactly that layout.  This module produces it on the device from the
+router's top-k expert ids, bit exact with the helper.
+"""
+
+import math
+
+import torch
+
+from .... import _native as nv
+from ...utils.kernel_assert import kernel_assert
+
+
+def get_n_blocks(T, TOPK, E, B, n_block_per_iter=1):
+    """Worst-case number of blocks (test_moe_cte_common.py:95-98)."""
+    N = math.ceil((T * TOPK - (E - 1)) / B) + E - 1
+    return n_block_per_iter * math.ceil(N / n_block_per_iter)
+
+
+def build_token_blocks(topk_ids: torch.Tensor, E: int, B: int, N: int = None, skip_token: bool = False,
+                       use_split_padding: bool = False, n_conditions: int = None, check: bool = False):
+    """topk_ids int32 ``[T, k]`` (distinct expert ids per row) ->
+    (token_position_to_id int32 ``[N*B]``, block_to_expert int32 ``[N]``, conditions int32 ``[n_conditions]``).
+
+    ``n_conditions`` defaults to ``N + 1`` (the non-block-parallel form); pass ``N + 2`` for the MX
+    block-parallel form.  ``check=True`` synchronises and raises if N is too small for the routing.
+    """
+    L = nv.lib()
+    ids = nv.require_device_tensor(topk_ids, "topk_ids")
+    kernel_assert(ids.dim() == 2 and ids.dtype == torch.int32, "topk_ids must be int32 [T, k]")
+    T, k = ids.shape
+    if N is None:
+        N = get_n_blocks(T, k, E, B)
+    if n_conditions is None:
+        n_conditions = N + 1
+    dev = ids.device
+    tp2id = torch.empty(N * B, dtype=torch.int32, device=dev)
+    b2e = torch.empty(N, dtype=torch.int32, device=dev)
+    cond = torch.empty(n_conditions, dtype=torch.int32, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws = torch.empty(L.moe_build_blocks_workspace_bytes(E), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = L.moe_build_blocks(nv.ptr(ids), T, k, E, B, N, 1 if skip_token else 0, 1 if use_split_padding else 0,
+                                nv.ptr(tp2id), nv.ptr(b2e), nv.ptr(cond), n_conditions, nv.ptr(ws), ws.numel(),
+                                nv.ptr(status), nv.stream_ptr(dev))
+    nv.check(rc, "build_token_blocks")
+    if check:
+        kernel_assert(int(status.item()) == 0, f"N={N} blocks cannot hold this routing")
+    return tp2id, b2e, cond

@@ -1,0 +1,82 @@
+"""Intermediate-sharded variants of the reference: same math as ``bwmm_shard_on_block``
+(one golden serves all, test_moe_cte_common.py:267-447); only the return shape differs
+(``[T+1, H]``, src/nkilib_src/nkilib/core/moe/moe_cte/bwmm_shard_on_I.py:293).  The
+Trainium-specific split of I over two cores has no GPU counterpart.  Signatures:
+bwmm_shard_on_I.py:86-114, :326-355, :2013-2036."""
+
+from typing import Optional
+
+import torch
+
+from ...._entry import KernelEntry
+from ...utils.common_types import ActFnType, ExpertAffinityScaleMode
+from ...utils.kernel_assert import kernel_assert
+from .bwmm_shard_on_block import run_dense_variant
+from .moe_cte_utils import SkipMode
+
+
+def _blockwise_mm_baseline_shard_intermediate(
+    hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size, token_position_to_id,
+    block_to_expert, gate_and_up_proj_bias=None, down_proj_bias=None, gate_up_proj_scale=None, down_proj_scale=None,
+    activation_function: ActFnType = ActFnType.SiLU, skip_dma: SkipMode = SkipMode(), compute_dtype=torch.bfloat16,
+    is_tensor_update_accumulating=True, expert_affinities_scaling_mode=ExpertAffinityScaleMode.PRE_SCALE,
+    gate_clamp_upper_limit: Optional[float] = None, gate_clamp_lower_limit: Optional[float] = None,
+    up_clamp_lower_limit: Optional[float] = None, up_clamp_upper_limit: Optional[float] = None,
+    checkpoint_activation=False, expert_affinity_multiply_on_I=False,
+):
+    kernel_assert(not checkpoint_activation, "checkpoint_activation is not supported on gfx950")
+    kernel_assert(not expert_affinity_multiply_on_I, "expert_affinity_multiply_on_I is not supported on gfx950")
+    return run_dense_variant(
+        hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size,
+        token_position_to_id, block_to_expert, "TH", gate_and_up_proj_bias=gate_and_up_proj_bias,
+        down_proj_bias=down_proj_bias, gate_up_proj_scale=gate_up_proj_scale, down_proj_scale=down_proj_scale,
+        activation_function=activation_function, skip_dma=skip_dma,
+        expert_affinities_scaling_mode=expert_affinities_scaling_mode,
+        gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
+        up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit,
+    )
+
+
+def _blockwise_mm_baseline_shard_intermediate_hybrid(
+    conditions, hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size: int,
+    token_position_to_id, block_to_expert, num_static_block: Optional[int] = None, gate_and_up_proj_bias=None,
+    down_proj_bias=None, gate_up_proj_scale=None, down_proj_scale=None, gate_up_activations_T=None,
+    down_activations=None, activation_function: ActFnType = ActFnType.SiLU, skip_dma: SkipMode = SkipMode(),
+    compute_dtype=torch.bfloat16, is_tensor_update_accumulating=True,
+    expert_affinities_scaling_mode=ExpertAffinityScaleMode.POST_SCALE, gate_clamp_upper_limit: Optional[float] = None,
+    gate_clamp_lower_limit: Optional[float] = None, up_clamp_lower_limit: Optional[float] = None,
+    up_clamp_upper_limit: Optional[float] = None,
+):
+    """``conditions`` stops the block loop at its first zero (test_moe_cte_common.py:331-333);
+    ``num_static_block`` only tunes the reference's static/dynamic loop split and is ignored."""
+    kernel_assert(gate_up_activations_T is None and down_activations is None,
+                  "activation checkpoint outputs are not supported on gfx950")
+    return run_dense_variant(
+        hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size,
+        token_position_to_id, block_to_expert, "TH", conditions=conditions,
+        gate_and_up_proj_bias=gate_and_up_proj_bias, down_proj_bias=down_proj_bias,
+        gate_up_proj_scale=gate_up_proj_scale, down_proj_scale=down_proj_scale,
+        activation_function=activation_function, skip_dma=skip_dma,
+        expert_affinities_scaling_mode=expert_affinities_scaling_mode,
+        gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
+        up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit,
+    )
+
+
+def _blockwise_mm_shard_intermediate_dropping(
+    hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size, token_position_to_id,
+    block_to_expert, gate_and_up_proj_bias=None, down_proj_bias=None, gate_up_proj_scale=None, down_proj_scale=None,
+    activation_function: ActFnType = ActFnType.SiLU, skip_dma: SkipMode = SkipMode(), compute_dtype=torch.bfloat16,
+    is_tensor_update_accumulating=True, expert_affinities_scaling_mode=ExpertAffinityScaleMode.PRE_SCALE,
+    expert_affinity_multiply_on_I: bool = False, gate_clamp_upper_limit: Optional[float] = None,
+    gate_clamp_lower_limit: Optional[float] = None, up_clamp_lower_limit: Optional[float] = None,
+    up_clamp_upper_limit: Optional[float] = None,
+):
+    """Token-dropping layer: N == E blocks, one per expert; the block math is unchanged.
+    The reference variant also returns checkpoint activations, which are not built."""
+    kernel_assert(False, "shard_on_i_dropping returns activation checkpoints, which are not supported on gfx950")
+
+
+blockwise_mm_baseline_shard_intermediate = KernelEntry(_blockwise_mm_baseline_shard_intermediate)
+blockwise_mm_baseline_shard_intermediate_hybrid = KernelEntry(_blockwise_mm_baseline_shard_intermediate_hybrid)
+blockwise_mm_shard_intermediate_dropping = KernelEntry(_blockwise_mm_shard_intermediate_dropping)

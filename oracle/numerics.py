@@ -1,0 +1,97 @@
+"""Low-precision number formats used by the goldens (oracle: test infrastructure only).
+
+The reference casts through ``neuron_dtypes.static_cast`` (third party, absent,
+unpinned).  These are the published formats restated from first principles:
+
+* bfloat16: fp32 with the low 16 mantissa bits dropped, round-to-nearest-even.
+* float8 e4m3fn (OCP): 1-4-3, bias 7, no inf, max 448, only S.1111.111 is NaN.
+  Decode closed form as in ``src/nkilib_src/nkilib/core/utils/mx_torch_common.py:109-131``.
+* Neuron ``float8_e4m3`` (max 240, ``src/nkilib_src/nkilib/core/rmsnorm/rmsnorm_quant_constants.py:84-87``)
+  has the same bit patterns as e4m3fn for every |v| <= 240, so one codec serves both.
+* E8M0: uint8 biased exponent, value 2**(byte - 127).
+
+Everything takes / returns numpy arrays.  bf16 values are carried as float32
+arrays whose low 16 bits are zero.
+"""
+
+import numpy as np
+
+E4M3FN_MAX = 448.0
+NEURON_E4M3_MAX = 240.0
+
+
+def to_bf16(x):
+    """Round float32 values to the nearest bfloat16 (ties to even); result stays float32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    bits = x.view(np.uint32).astype(np.uint64)
+    rounded = bits + 0x7FFF + ((bits >> 16) & 1)
+    out = (rounded & 0xFFFF0000).astype(np.uint32)
+    # NaN stays NaN (quiet), do not let the carry turn it into inf / another number.
+    nan = np.isnan(x)
+    if nan.any():
+        out = np.where(nan, np.uint32(0x7FC00000), out)
+    return out.view(np.float32).reshape(x.shape)
+
+
+def bf16_bits(x):
+    """uint16 bit patterns of to_bf16(x)."""
+    return (to_bf16(x).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_from_bits(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def _build_e4m3fn_table():
+    codes = np.arange(256, dtype=np.int64)
+    sign = (codes >> 7) & 1
+    exp = (codes >> 3) & 0xF
+    man = codes & 0x7
+    sub = (man / 8.0) * 2.0**-6
+    nor = (1.0 + man / 8.0) * np.power(2.0, exp - 7.0)
+    val = np.where(exp == 0, sub, nor)
+    val = np.where(sign == 1, -val, val)
+    val[0x7F] = np.nan
+    val[0xFF] = np.nan
+    return val.astype(np.float32)
+
+
+E4M3FN_TABLE = _build_e4m3fn_table()
+
+
+def e4m3fn_decode(codes):
+    """uint8 bit patterns -> float32 (exact)."""
+    return E4M3FN_TABLE[np.asarray(codes, dtype=np.uint8)]
+
+
+def e4m3fn_encode(x):
+    """float32 -> uint8 e4m3fn bit patterns, round-to-nearest-even, saturating at +-448.
+
+    The goldens clip to the format maximum before the cast
+    (``test/utils/mx_utils.py:91-93``), so saturation only matters for values the
+    caller failed to clip.  NaN encodes as 0x7F.
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    bits = x.view(np.uint32)
+    sign = ((bits >> 31) & 1).astype(np.uint8)
+    a = np.abs(x)
+    abits = (bits & 0x7FFFFFFF).astype(np.uint64)
+    # normal path: keep 3 mantissa bits, RNE on the 20 dropped bits
+    r = (abits + 0x7FFFF + ((abits >> 20) & 1)) >> 20  # (exp8 << 3) | man3
+    code_n = r.astype(np.int64) - (120 << 3)  # rebias 127 -> 7
+    # subnormal path (|x| < 2**-6): multiples of 2**-9, RNE; 8 == smallest normal
+    code_s = np.rint(a.astype(np.float64) * 512.0).astype(np.int64)
+    code = np.where(a < 2.0**-6, code_s, code_n)
+    code = np.clip(code, 0, 0x7E)
+    code = np.where(np.isnan(x), 0x7F, code)
+    return (code.astype(np.uint8) | (sign << 7)).reshape(x.shape)
+
+
+def e8m0_decode(b):
+    """uint8 E8M0 -> float64 power of two, 2**(b-127)."""
+    return np.power(2.0, np.asarray(b).astype(np.int32) - 127)
+
+
+def float32_exponent_field(x):
+    """Biased exponent field of float32 values (``test/utils/mx_utils.py:42-45``)."""
+    return (np.ascontiguousarray(x, dtype=np.float32).view(np.uint32) >> 23) & 0xFF

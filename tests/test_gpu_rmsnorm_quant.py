@@ -1,0 +1,179 @@
+"""GPU parity: RMSNorm-Quant front end (fp8 ROW / STATIC, MXFP8) through the C ABI vs the oracle.
+
+Shapes and generators follow the reference's own test table
+(test/integration/nkilib/core/rmsnorm/test_rmsnorm_quant.py:286-304): H = 16384, S in {2, 160, 2048},
+gaussian / duplicate-row / all-ones inputs, lower_bound in {0, 0.5}.
+Bar: codes bit exact except round-half ties (decided by fp32 summation order), dequant scale
+within 2 ulp of the oracle (the reference's own bar is rtol 0.072 / 0.007, :260-266).
+"""
+
+import numpy as np
+import pytest
+
+from helpers import bf16_tensor, f32_tensor
+from oracle import rmsnorm as orn
+from oracle.compare import fp8_codes_match_except_ties
+from oracle.numerics import to_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _unrounded_row(inp, gamma, lower_bound, quant_only, eps=1e-6):
+    """The oracle's value right before the fp8 cast (float64 view of its fp32 pipeline)."""
+    inp = inp.astype(np.float32)
+    if quant_only:
+        norm = inp
+    else:
+        rms = np.sqrt(np.mean(np.square(inp), axis=-1, keepdims=True))
+        norm = inp * np.reciprocal(rms + np.float32(eps)) * gamma.astype(np.float32)
+    amax = np.abs(norm).max(axis=-1, keepdims=True)
+    if lower_bound > 0:
+        amax = np.minimum(amax, np.float32(lower_bound))
+        norm = np.clip(norm, -np.float32(lower_bound), np.float32(lower_bound))
+    dq = np.maximum((amax / np.float32(240.0)).astype(np.float32), np.float32(1e-6))
+    return norm * np.reciprocal(dq)
+
+
+def _gen(kind, rows, H, rng):
+    if kind == "gauss":
+        x = rng.normal(size=(1, rows, H))
+    elif kind == "dup":
+        x = np.broadcast_to(rng.normal(size=(1, 1, H)), (1, rows, H)) / 100.0
+    else:
+        x = np.ones((1, rows, H))
+    g = np.ones((1, H)) if kind == "ones" else rng.random((1, H))
+    return to_bf16(x.astype(np.float32)), to_bf16(g.astype(np.float32))
+
+
+@pytest.mark.parametrize(
+    "rows,H,quant_only,kind,lower_bound",
+    [
+        (2, 16384, True, "gauss", 0.0),
+        (2, 16384, True, "gauss", 0.5),
+        (2, 16384, False, "gauss", 0.0),
+        (2, 16384, False, "gauss", 0.5),
+        (2048, 16384, False, "gauss", 0.0),
+        (160, 16384, False, "dup", 0.0),
+        (160, 16384, False, "ones", 0.0),
+        (160, 16384, True, "gauss", 0.0),
+        (33, 4096, False, "gauss", 0.0),
+        (5, 1000, False, "gauss", 0.0),   # H not a multiple of 8: scalar path
+        (7, 7168, False, "gauss", 0.0),
+    ],
+)
+def test_row_quant(rows, H, quant_only, kind, lower_bound):
+    import torch
+    from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+    from nkilib.core.rmsnorm.rmsnorm_quant import split_row_record
+    from nkilib.core.utils.common_types import NormType, QuantizationType
+
+    rng = np.random.default_rng(0)
+    x, g = _gen(kind, rows, H, rng)
+    dev = torch.device("cuda:0")
+    kargs = RmsNormQuantKernelArgs(lower_bound=lower_bound,
+                                   norm_type=NormType.NO_NORM if quant_only else NormType.RMS_NORM,
+                                   quantization_type=QuantizationType.ROW)
+    out = rmsnorm_quant_kernel[2](bf16_tensor(x, dev), bf16_tensor(g, dev), kargs)
+    assert tuple(out.shape) == (1, rows, H + 4) and out.dtype == torch.float8_e4m3fn
+    codes_t, scale_t = split_row_record(out)
+    codes = codes_t.view(torch.uint8).cpu().numpy()
+    scale = scale_t.cpu().numpy()
+    g_codes, g_scale = orn.rmsnorm_quant_ref(x, g, None, lower_bound, quant_only, "row")
+    # dequant scale: within 2 ulp
+    ulp = np.abs(scale.view(np.int32).astype(np.int64) - g_scale.view(np.int32).astype(np.int64))
+    assert ulp.max() <= 2, f"dequant scale differs by {ulp.max()} ulp"
+    ok, n_bad, n_forgiven = fp8_codes_match_except_ties(codes, g_codes, _unrounded_row(x, g, lower_bound, quant_only))
+    assert ok, f"{n_bad} mismatching codes, only {n_forgiven} are rounding ties"
+    assert n_bad <= max(8, codes.size // 20000), f"too many tie flips: {n_bad} of {codes.size}"
+    if kind == "ones":
+        assert (codes == 0x77).all()  # 240.0
+
+
+@pytest.mark.parametrize("rows,H,quant_only", [(2, 16384, True), (160, 16384, False), (64, 4096, False)])
+def test_static_quant(rows, H, quant_only):
+    import torch
+    from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+    from nkilib.core.utils.common_types import NormType, QuantizationType
+
+    rng = np.random.default_rng(1)
+    x, g = _gen("gauss", rows, H, rng)
+    sc = np.full((128, 1), 0.031, np.float32)
+    dev = torch.device("cuda:0")
+    kargs = RmsNormQuantKernelArgs(norm_type=NormType.NO_NORM if quant_only else NormType.RMS_NORM,
+                                   quantization_type=QuantizationType.STATIC)
+    out = rmsnorm_quant_kernel(bf16_tensor(x, dev), bf16_tensor(g, dev), kargs, f32_tensor(sc, dev))
+    assert tuple(out.shape) == (1, rows, H)
+    codes = out.view(torch.uint8).cpu().numpy()
+    g_codes, _ = orn.rmsnorm_quant_ref(x, g, sc, 0.0, quant_only, "static")
+    xf = x.astype(np.float32)
+    if quant_only:
+        norm = xf
+    else:
+        rms = np.sqrt(np.mean(np.square(xf), axis=-1, keepdims=True))
+        norm = xf * np.reciprocal(rms + np.float32(1e-6)) * g.astype(np.float32)
+    unr = np.clip(norm * np.reciprocal(np.float32(0.031)), -240, 240)
+    ok, n_bad, n_forgiven = fp8_codes_match_except_ties(codes, g_codes, unr)
+    assert ok, f"{n_bad} mismatching codes, only {n_forgiven} are rounding ties"
+
+
+def test_zero_row_follows_kernel_rule():
+    """All-zero row: dq = 1e-6 (the reference kernel's clamp), codes 0; no NaN."""
+    import torch
+    from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+    from nkilib.core.rmsnorm.rmsnorm_quant import split_row_record
+    from nkilib.core.utils.common_types import NormType
+
+    dev = torch.device("cuda:0")
+    x = torch.zeros((3, 512), dtype=torch.bfloat16, device=dev)
+    out = rmsnorm_quant_kernel(x, None, RmsNormQuantKernelArgs(norm_type=NormType.NO_NORM))
+    codes, scale = split_row_record(out)
+    assert (codes.view(torch.uint8) == 0).all()
+    assert torch.equal(scale.cpu(), torch.full((3, 1), 1e-6, dtype=torch.float32))
+
+
+@pytest.mark.parametrize("T,H,do_norm", [(4, 512, True), (64, 2048, True), (33, 7168, True), (16, 16384, True),
+                                          (40, 1024, False)])
+def test_mx_front_end(T, H, do_norm):
+    """RMSNorm -> MXFP8 (token-major and the reference's [128, H/512, T] layouts) vs the oracle."""
+    import torch
+    from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize, rmsnorm_mx_quantize_tkg
+
+    rng = np.random.default_rng(2)
+    x = to_bf16((rng.standard_normal((T, H)) * rng.choice([0.01, 1.0, 30.0], size=(T, 1))).astype(np.float32))
+    g = to_bf16(rng.random((1, H)).astype(np.float32) + 0.5)
+    ref = orn.rmsnorm_mx_quant_ref(x, g if do_norm else None, do_norm=do_norm)
+    dev = torch.device("cuda:0")
+    q, s = rmsnorm_mx_quantize(bf16_tensor(x, dev), bf16_tensor(g, dev) if do_norm else None, do_norm=do_norm)
+    q, s = q.cpu().numpy(), s.cpu().numpy()
+    # scale bytes can only differ where the bf16 rounding of the normalised value differs, i.e. where the fp32
+    # sum-of-squares order decided a tie; count them, then compare values through the dequantised result
+    n_s = int((s != ref["tok_scale"]).sum())
+    assert n_s <= max(2, s.size // 2000), f"{n_s} of {s.size} scale bytes differ"
+    from oracle.numerics import e4m3fn_decode
+
+    deq = e4m3fn_decode(q).astype(np.float64) * np.repeat(np.power(2.0, s.astype(np.float64) - 127), 32, axis=1)
+    gdeq = e4m3fn_decode(ref["tok_quant"]).astype(np.float64) * np.repeat(
+        np.power(2.0, ref["tok_scale"].astype(np.float64) - 127), 32, axis=1)
+    mism = q != ref["tok_quant"]
+    frac = mism.mean()
+    assert frac < 2e-3, f"{frac:.2e} of codes differ"
+    # every differing code is at most one fp8 step away (one e4m3 ulp = 2^-3 relative)
+    rel = np.abs(deq - gdeq) / np.maximum(np.abs(gdeq), 1e-30)
+    assert (rel[mism & (gdeq != 0)] <= 0.1251).all()
+    if not do_norm:
+        assert not mism.any() and n_s == 0  # pure quantisation has no reduction: bit exact
+    if do_norm and T % 4 == 0:
+        nT = H // 512
+        out = torch.empty((128, T, H // 128), dtype=torch.bfloat16, device=dev)
+        oq = torch.empty((128, nT, T), dtype=torch.int32, device=dev)
+        osc = torch.zeros((128, nT, T), dtype=torch.uint8, device=dev)
+        rmsnorm_mx_quantize_tkg(bf16_tensor(x.reshape(1, T, H), dev), bf16_tensor(g, dev), out, oq, osc)
+        oq_b = oq.cpu().numpy().view(np.uint8).reshape(128, nT, T, 4)
+        # same numbers as the token-major call, rearranged
+        assert np.array_equal(oq_b.transpose(2, 1, 0, 3).reshape(T, H), q)
+        rows = (np.arange(16) // 4) * 32 + np.arange(16) % 4
+        assert np.array_equal(osc.cpu().numpy()[rows].transpose(2, 1, 0).reshape(T, H // 32), s)
+        from helpers import from_bf16_tensor
+
+        o = from_bf16_tensor(out)
+        assert np.mean(o != ref["out"]) < 2e-3
