@@ -31,9 +31,14 @@ __device__ __forceinline__ float load_bias(const void* p, int dtype, int64_t idx
   return dtype == MOE_DT_BF16 ? bf16_bits_to_f32(((const uint16_t*)p)[idx]) : ((const float*)p)[idx];
 }
 
-__device__ __forceinline__ v8i lds_read32(const uint8_t* p) {
-  const v4i lo = *(const v4i*)p;
-  const v4i hi = *(const v4i*)(p + 16);
+// Operand fragment of v_mfma_scale_f32_16x16x128_f8f6f4 for one row / column whose 128 K bytes
+// sit contiguously at `row`: lane group g = lane/16 supplies K bytes [16g, 16g+16) in its first
+// four registers and [64+16g, 64+16g+16) in the last four.  With that placement the hardware's
+// K index equals the byte offset, and the scale byte a lane supplies (lanes 16j..16j+15 scale
+// K block j = bytes [32j, 32j+32) of their row) lines up with consecutive 32-byte MX blocks.
+__device__ __forceinline__ v8i lds_read_frag(const uint8_t* row, int g) {
+  const v4i lo = *(const v4i*)(row + 16 * g);
+  const v4i hi = *(const v4i*)(row + 64 + 16 * g);
   v8i r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
   r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
@@ -286,13 +291,13 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         const int row = m0 + 16 * mt + c;
-        af[mt] = lds_read32(sA + row * LROW + g * 32);
+        af[mt] = lds_read_frag(sA + row * LROW, g);
         sa[mt] = (KIND == MOE_KIND_MXFP8) ? (int)((sAs[row] >> (8 * g)) & 0xffu) : 127;
       }
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         const int col = nt * 16 + c;
-        const v8i bf = lds_read32(sB + col * LROW + g * 32);
+        const v8i bf = lds_read_frag(sB + col * LROW, g);
         const int sb = (KIND == MOE_KIND_MXFP8) ? (int)((sBs[col] >> (8 * g)) & 0xffu) : 127;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)

@@ -5,7 +5,9 @@
 // once.  HBM traffic per row is the algorithmic minimum: 2H bytes in, H (+4 or +H/32) out.
 //
 // The fp32 arithmetic follows the reference goldens operation by operation (no FMA
-// contraction) so that quantised codes are reproducible:
+// contraction) so that quantised codes are reproducible.  The one quantity whose value depends
+// on evaluation order, the row's sum of squares, is accumulated in fp64 and rounded once, i.e.
+// it is the correctly rounded fp32 sum that any fp32 summation order approximates:
 //   ROW / STATIC: test/integration/nkilib/core/rmsnorm/test_rmsnorm_quant.py:46-97
 //   MX:           test/integration/nkilib/core/subkernels/test_rmsnorm_mx_quantize_tkg.py:100-137,
 //                 rms_norm test/integration/nkilib/utils/test_kernel_common.py:26-41,
@@ -55,13 +57,14 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
     const float* __restrict__ static_scale, uint8_t* __restrict__ out, int64_t H, int64_t out_stride, float eps,
     float lower_bound, int do_norm, int vec_ok) {
   __shared__ float red[16];
+  __shared__ double redd[16];
   const int64_t row = blockIdx.x;
   const int es = (x_dtype == MOE_DT_FP32) ? 4 : 2;
   const void* xr = (const uint8_t*)x + row * H * es;
   const int nchunk = (int)((H + RQ_THREADS * 8 - 1) / (RQ_THREADS * 8));
 
   float v[RQ_MAX_CHUNKS][8];
-  float ss = 0.f;
+  double ss = 0.0;
 #pragma unroll
   for (int j = 0; j < RQ_MAX_CHUNKS; ++j) {
     if (j < nchunk) {
@@ -73,12 +76,12 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
         for (int k = 0; k < 8; ++k) v[j][k] = 0.f;
       }
 #pragma unroll
-      for (int k = 0; k < 8; ++k) ss += v[j][k] * v[j][k];
+      for (int k = 0; k < 8; ++k) ss += (double)v[j][k] * (double)v[j][k];
     }
   }
 
   if (do_norm) {
-    const float total = block_sum(ss, red);
+    const float total = (float)block_sum_f64(ss, redd);
     const float mean = total / (float)H;
     const float rms = sqrtf(mean);
     const float inv = 1.0f / (rms + eps);
@@ -161,7 +164,7 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
     const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
     uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, uint16_t* __restrict__ out_norm, int64_t rows,
     int64_t H, float eps, float hidden_actual, int do_norm, int layout) {
-  __shared__ float red[16];
+  __shared__ double redd[16];
   const int64_t row = blockIdx.x;
   const int es = (x_dtype == MOE_DT_FP32) ? 4 : 2;
   const void* xr = (const uint8_t*)x + row * H * es;
@@ -170,7 +173,7 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
   const int64_t Hq = H / 4;
 
   float v[MXQ_MAX_BLK][4][8];
-  float ss = 0.f;
+  double ss = 0.0;
 #pragma unroll
   for (int j = 0; j < MXQ_MAX_BLK; ++j) {
     const int blk = j * RQ_THREADS + threadIdx.x;
@@ -180,13 +183,13 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
       for (int q = 0; q < 4; ++q) {
         load8(xr, x_dtype, q * Hq + tile * 128 + p8 * 8, H, true, v[j][q]);
 #pragma unroll
-        for (int r = 0; r < 8; ++r) ss += v[j][q][r] * v[j][q][r];
+        for (int r = 0; r < 8; ++r) ss += (double)v[j][q][r] * (double)v[j][q][r];
       }
     }
   }
   float inv = 1.0f;
   if (do_norm) {
-    const float total = block_sum(ss, red);
+    const float total = (float)block_sum_f64(ss, redd);
     const float rms = sqrtf(total / hidden_actual + eps);
     inv = 1.0f / rms;
   }

@@ -4,7 +4,10 @@ Shapes and generators follow the reference's own test table
 (test/integration/nkilib/core/rmsnorm/test_rmsnorm_quant.py:286-304): H = 16384, S in {2, 160, 2048},
 gaussian / duplicate-row / all-ones inputs, lower_bound in {0, 0.5}.
 Bar: codes bit exact except round-half ties (decided by fp32 summation order), dequant scale
-within 2 ulp of the oracle (the reference's own bar is rtol 0.072 / 0.007, :260-266).
+within 4 ulp of the oracle: the golden's fp32 pairwise ``np.mean`` and the kernel's correctly
+rounded sum differ by an ulp or two, which the three following roundings (rms, reciprocal,
+product with gamma) can stretch to 3-4 ulp of amax.  The reference's own bar is rtol 0.072 for
+values and 0.007 (~6e4 ulp) for the scale (:260-266).
 """
 
 import numpy as np
@@ -79,9 +82,8 @@ def test_row_quant(rows, H, quant_only, kind, lower_bound):
     codes = codes_t.view(torch.uint8).cpu().numpy()
     scale = scale_t.cpu().numpy()
     g_codes, g_scale = orn.rmsnorm_quant_ref(x, g, None, lower_bound, quant_only, "row")
-    # dequant scale: within 2 ulp
     ulp = np.abs(scale.view(np.int32).astype(np.int64) - g_scale.view(np.int32).astype(np.int64))
-    assert ulp.max() <= 2, f"dequant scale differs by {ulp.max()} ulp"
+    assert ulp.max() <= (0 if quant_only else 4), f"dequant scale differs by {ulp.max()} ulp"
     ok, n_bad, n_forgiven = fp8_codes_match_except_ties(codes, g_codes, _unrounded_row(x, g, lower_bound, quant_only))
     assert ok, f"{n_bad} mismatching codes, only {n_forgiven} are rounding ties"
     assert n_bad <= max(8, codes.size // 20000), f"too many tie flips: {n_bad} of {codes.size}"
