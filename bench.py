@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE context-encoding hot path on one MI355X.
+
+One "step" is one pass of the whole path over one batch of synthetic input that is already
+resident in HBM: RMSNorm -> MXFP8 quantise of the hidden states, token -> block index build from
+the router's top-k ids, gate/up GEMM with fused SiLU(gate)*up and MXFP8 re-quantisation, down
+GEMM with fused affinity scaling, and the per-token combine into bf16 rows.
+
+Default workload: BASELINE config 4, DeepSeek-V3-shaped routed experts (T=8192, H=7168, I=2048,
+E=256, top-8, block 128, MXFP8 weights ~11 GB).  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c5-<T>] [--no-cpu-baseline]
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "nki-library_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+METRIC = "MoE layer TFLOP/s and tokens/s (fp8/MXFP8), % of MFMA peak, 1x MI355X"
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c4")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-blocks", type=int, default=6, help="blocks of the workload timed on the CPU oracle")
+    return ap.parse_args()
+
+
+def build_workload(name, dev):
+    import torch
+    from nkilib import synthetic as syn
+
+    if name.startswith("c5"):
+        cfg = dict(syn.CONFIGS["c4"])
+        cfg["T"] = int(name.split("-")[1]) if "-" in name else 128
+        router_kw = dict(uniform_random=True)
+    else:
+        cfg = dict(syn.CONFIGS[name])
+        router_kw = dict(mode="sigmoid") if name == "c4" else dict(mode="softmax", expert_bias_std=0.5 if name == "c3" else 0.0)
+    assert cfg["kind"] == "mxfp8", "bench.py times the MXFP8 layer (configs c3, c4, c5-<T>)"
+    T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
+    t0 = time.time()
+    gu_q, gu_s, d_q, d_s = syn.mx_expert_weights(E, H, I, 0.02, dev, seed=0)
+    ids, aff = syn.route(T, E, k, dev, seed=0, **router_kw)
+    x = syn.hidden_states(T, H, dev, seed=0)
+    gamma = torch.ones((1, H), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    cfg["gen_seconds"] = time.time() - t0
+    return cfg, dict(x=x, gamma=gamma, ids=ids, aff=aff, gu_q=gu_q, gu_s=gu_s, d_q=d_q, d_s=d_s)
+
+
+def cpu_baseline(cfg, t, tp2id, b2e, n_blocks):
+    """The CPU oracle (a port of the reference's numpy golden) on the first ``n_blocks`` non-empty blocks of the
+    same workload: normalise, quantise online, MX gate/up, act, MX down, affinity, accumulate."""
+    import numpy as np
+    import torch
+    from oracle import moe as omoe
+    from oracle import rmsnorm as orn
+    from oracle.numerics import bf16_from_bits
+
+    T, H, I, E, B = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["B"]
+    tp = tp2id.cpu().numpy()
+    be = b2e.cpu().numpy()
+    tpb = tp.reshape(-1, B)
+    keep = [b for b in range(tpb.shape[0]) if (tpb[b] < T).any()][:n_blocks]
+    experts = sorted(set(int(be[b]) for b in keep))
+    remap = {e: i for i, e in enumerate(experts)}
+    sel = torch.tensor(experts, device=t["gu_q"].device)
+    gu_q = t["gu_q"][sel].cpu().numpy()
+    gu_s = t["gu_s"][sel].cpu().numpy()
+    d_q = t["d_q"][sel].cpu().numpy()
+    d_s = t["d_s"][sel].cpu().numpy()
+    x = bf16_from_bits(t["x"].view(torch.int16).cpu().numpy().view(np.uint16))
+    aff_full = bf16_from_bits(t["aff"].view(torch.int16).cpu().numpy().view(np.uint16))
+    aff = np.ascontiguousarray(aff_full[:, experts])
+    tp_s = np.concatenate([tpb[b] for b in keep])
+    be_s = np.array([remap[int(be[b])] for b in keep], dtype=np.int32)
+    rows = int(sum((tpb[b] < T).sum() for b in keep))
+    t0 = time.perf_counter()
+    tok = np.unique(tp_s[tp_s < T])
+    normed = np.zeros_like(x)
+    normed[tok] = orn.to_bf16(orn.rms_norm(x[tok], np.ones((1, H), np.float32)))
+    omoe.moe_blockwise_mx_ref(normed, aff, gu_q, d_q, gu_s, d_s, tp_s, be_s, B)
+    dt = time.perf_counter() - t0
+    flops = 6.0 * rows * H * I
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": os.cpu_count(),
+        "kind": "port",
+        "sample": f"first {len(keep)} non-empty blocks ({rows} routed rows, {len(experts)} experts) of the same workload, "
+                  f"numpy oracle incl. RMSNorm of their tokens, {dt:.1f} s",
+        "tokens_per_s": rows / cfg["k"] / dt,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from nkilib import _native as nv
+    from nkilib.core.moe.moe_cte import (MoECTEImplementation, MoECTESpec, QuantizationConfig, build_token_blocks,
+                                         get_n_blocks, moe_cte)
+    from nkilib.core.moe.moe_cte import _launch
+    from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    dev = torch.device("cuda:0")
+    nv.check(nv.lib().moe_check_device(), "device check")
+    cfg, t = build_workload(args.workload, dev)
+    T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
+    N = get_n_blocks(T, k, E, B, n_block_per_iter=2)
+    spec = MoECTESpec(implementation=MoECTEImplementation.shard_on_block_mx)
+    qcfg = QuantizationConfig(t["gu_s"], t["d_s"])
+    gu_x4 = t["gu_q"].view(torch.int32).reshape(t["gu_q"].shape[:-1])
+
+    names = ["norm_quant", "build_blocks", "prep", "gate_up", "down", "combine"]
+    events = []
+
+    def rec():
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()  # torch's current stream: the stream every kernel of the path is launched on
+        events[-1].append(ev)
+
+    def step(timed):
+        if timed:
+            events.append([])
+            rec()
+        xq, xs = rmsnorm_mx_quantize(t["x"], t["gamma"])
+        if timed:
+            rec()
+        tp2id, b2e, cond = build_token_blocks(t["ids"], E, B, N, n_conditions=N + 2)
+        if timed:
+            rec()
+        _launch.stage_callback = (lambda name: rec()) if timed else None
+        out = moe_cte[2](xq, t["aff"].reshape(-1, 1), gu_x4, t["d_q"], tp2id, b2e, B, spec, conditions=cond,
+                         quantization_config=qcfg, hidden_states_scale=xs)
+        _launch.stage_callback = None
+        return out, tp2id, b2e
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, tp2id, b2e = step(True)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    stage_ms = {n: 0.0 for n in names}
+    for evs in events:
+        assert len(evs) == len(names) + 1, (len(evs), names)
+        for i, n in enumerate(names):
+            stage_ms[n] += evs[i].elapsed_time(evs[i + 1])
+    stage_ms = {n: v / args.steps for n, v in stage_ms.items()}
+
+    routed = int((tp2id.reshape(-1) < T).sum().item())  # == T*k
+    flops_layer = 6.0 * routed * H * I
+    flops_gate_up = 4.0 * routed * H * I
+    tflops = flops_layer / (ms_per_step * 1e-3) / 1e12
+    gate_up_tflops = flops_gate_up / (stage_ms["gate_up"] * 1e-3) / 1e12
+    e_hit = int(torch.unique(t["ids"]).numel())
+    weight_bytes = e_hit * 3 * H * I * (1 + 1 / 32)
+    # HBM-bound front end: bytes = rows*H*(2 in + 1 out) + scales
+    nq_gbs = (T + 1) * H * (3 + 1 / 32) / (stage_ms["norm_quant"] * 1e-3) / 1e9
+    comb_gbs = (routed * H * 2 + (T + 1) * H * 2) / (stage_ms["combine"] * 1e-3) / 1e9
+
+    res = {
+        "metric": METRIC,
+        "value": round(tflops, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp8_e4m3 (E8M0 block scales, fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: MXFP8 blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} "
+                               f"(N={N} blocks, {routed} routed rows), RMSNorm->MXFP8 front end + block build + "
+                               f"gate/up + down + combine",
+                   "T": T, "H": H, "I": I, "E": E, "top_k": k, "block_size": B},
+        "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
+        "pct_of_fp8_mfma_peak": round(100.0 * tflops / PEAK_FP8_TFLOPS, 2),
+        "stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
+        "stage_rates": {
+            "gate_up_TFLOPs": round(gate_up_tflops, 2),
+            "down_TFLOPs": round(2.0 * routed * H * I / (stage_ms["down"] * 1e-3) / 1e12, 2),
+            "norm_quant_GBs": round(nq_gbs, 1),
+            "combine_GBs": round(comb_gbs, 1),
+            "weights_GBs_over_gemm_time": round(weight_bytes / ((stage_ms["gate_up"] + stage_ms["down"]) * 1e-3) / 1e9, 1),
+        },
+        "roofline": {
+            "kernel": "gate/up blockwise MXFP8 GEMM (bwmm_kernel<MXFP8, stage 1>)",
+            "bound": "mfma",
+            "achieved": round(gate_up_tflops, 2),
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(gate_up_tflops / PEAK_FP8_TFLOPS, 4),
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(cfg, t, tp2id, b2e, args.cpu_blocks)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

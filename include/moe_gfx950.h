@@ -177,6 +177,20 @@ typedef struct moe_bwmm_args {
 size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* args);
 int moe_blockwise(const moe_bwmm_args* args, void* stream);
 
+/* The same pipeline, one stage (or any subset, always in pipeline order) per call, so that a
+ * caller can bracket individual kernels with its own events.  moe_blockwise(args, s) ==
+ * moe_blockwise_stages(args, MOE_STAGE_ALL, s).  Stages communicate through `workspace`, which
+ * must be the same buffer for all calls of one pass.  No counterpart in the reference (its
+ * stages are fused into one traced kernel); used by bench.py for per-kernel timing. */
+#define MOE_STAGE_PREP 1u      /* block bookkeeping: active blocks, valid rows, token -> slot lists */
+#define MOE_STAGE_ACT_QUANT 2u /* MXFP8 kind with bf16 hidden_states: online activation quantisation */
+#define MOE_STAGE_GATE_UP 4u   /* gate/up GEMM + act(gate)*up (+ MXFP8 re-quantisation)              */
+#define MOE_STAGE_REQUANT 8u   /* FP8_ROW kind: per-row re-quantisation of the intermediate          */
+#define MOE_STAGE_DOWN 16u     /* down GEMM + bias + affinity                                        */
+#define MOE_STAGE_COMBINE 32u  /* per-token accumulation of the contributions into the output        */
+#define MOE_STAGE_ALL 63u
+int moe_blockwise_stages(const moe_bwmm_args* args, unsigned stages, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -127,6 +127,10 @@ extern "C" size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* a) {
 }
 
 extern "C" int moe_blockwise(const moe_bwmm_args* a, void* stream) {
+  return moe_blockwise_stages(a, MOE_STAGE_ALL, stream);
+}
+
+extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, void* stream) {
   int rc = validate(a);
   if (rc != MOE_OK) return rc;
   const Plan p = make_plan(a);
@@ -136,8 +140,10 @@ extern "C" int moe_blockwise(const moe_bwmm_args* a, void* stream) {
   uint8_t* ws = (uint8_t*)a->workspace;
   const int64_t n_real = a->skip_token ? a->T1 : a->T1 - 1;
   const Bookkeeping bk = carve_bookkeeping(ws + p.book, a->T1, a->N, a->B);
-  rc = launch_prep(bk, a, n_real, s);
-  if (rc != MOE_OK) return rc;
+  if (stages & MOE_STAGE_PREP) {
+    rc = launch_prep(bk, a, n_real, s);
+    if (rc != MOE_OK) return rc;
+  }
 
   GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -177,9 +183,11 @@ extern "C" int moe_blockwise(const moe_bwmm_args* a, void* stream) {
     const uint8_t* xs = (const uint8_t*)a->hidden_states_scale;
     if (!xs) {
       // online activation quantisation (moe_cte_mx_utils.py:730-771): bf16 rows -> MXFP8 in k' order
-      rc = moe_rmsnorm_quant_mxfp8(a->hidden_states, MOE_DT_BF16, nullptr, MOE_DT_BF16, ws + p.xq, ws + p.xs, nullptr,
-                                   a->T1, a->H, 0.f, a->H, 0, MOE_MX_LAYOUT_TOKEN_MAJOR, stream);
-      if (rc != MOE_OK) return rc;
+      if (stages & MOE_STAGE_ACT_QUANT) {
+        rc = moe_rmsnorm_quant_mxfp8(a->hidden_states, MOE_DT_BF16, nullptr, MOE_DT_BF16, ws + p.xq, ws + p.xs,
+                                     nullptr, a->T1, a->H, 0.f, a->H, 0, MOE_MX_LAYOUT_TOKEN_MAJOR, stream);
+        if (rc != MOE_OK) return rc;
+      }
       xq = ws + p.xq;
       xs = ws + p.xs;
     }
@@ -199,13 +207,18 @@ extern "C" int moe_blockwise(const moe_bwmm_args* a, void* stream) {
     gx1 = (unsigned)((a->I + 127) / 128);
   }
 
-  rc = launch_gemm_stage(a->kind, 1, g1, gx1, gy, s);
-  if (rc != MOE_OK) return rc;
-  if (a->kind == MOE_KIND_FP8_ROW) {
+  if (stages & MOE_STAGE_GATE_UP) {
+    rc = launch_gemm_stage(a->kind, 1, g1, gx1, gy, s);
+    if (rc != MOE_OK) return rc;
+  }
+  if (a->kind == MOE_KIND_FP8_ROW && (stages & MOE_STAGE_REQUANT)) {
     rc = launch_row_requant((const float*)(ws + p.y), ws + p.yq, (float*)(ws + p.ys), bk, a->N, a->B, a->I, p.Iw, s);
     if (rc != MOE_OK) return rc;
   }
-  rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);
-  if (rc != MOE_OK) return rc;
-  return launch_combine(bk, a, ws + p.d, n_real, s);
+  if (stages & MOE_STAGE_DOWN) {
+    rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);
+    if (rc != MOE_OK) return rc;
+  }
+  if (stages & MOE_STAGE_COMBINE) return launch_combine(bk, a, ws + p.d, n_real, s);
+  return MOE_OK;
 }

@@ -22,6 +22,8 @@ KIND_BF16, KIND_FP8_ROW, KIND_MXFP8 = 0, 1, 2
 # MOE_MX_LAYOUT_*
 MX_TOKEN_MAJOR, MX_REF_DENSE, MX_REF_STRIDED = 0, 1, 2
 CLAMP_GATE_HI, CLAMP_GATE_LO, CLAMP_UP_HI, CLAMP_UP_LO = 1, 2, 4, 8
+# MOE_STAGE_*
+STAGE_PREP, STAGE_ACT_QUANT, STAGE_GATE_UP, STAGE_REQUANT, STAGE_DOWN, STAGE_COMBINE, STAGE_ALL = 1, 2, 4, 8, 16, 32, 63
 
 EXPORTED_SYMBOLS = (
     "moe_error_string",
@@ -34,6 +36,7 @@ EXPORTED_SYMBOLS = (
     "moe_build_blocks",
     "moe_blockwise_workspace_bytes",
     "moe_blockwise",
+    "moe_blockwise_stages",
 )
 
 
@@ -124,6 +127,8 @@ def lib():
     L.moe_blockwise_workspace_bytes.argtypes = [POINTER(BwmmArgs)]
     L.moe_blockwise.restype = c_int
     L.moe_blockwise.argtypes = [POINTER(BwmmArgs), c_void_p]
+    L.moe_blockwise_stages.restype = c_int
+    L.moe_blockwise_stages.argtypes = [POINTER(BwmmArgs), ctypes.c_uint, c_void_p]
     _lib = L
     return L
 

@@ -13,8 +13,19 @@ from ...utils.kernel_assert import kernel_assert
 from .moe_cte_utils import SkipMode
 
 
-def _f8_or_u8(t):
-    return t.dtype in (torch.uint8, torch.float8_e4m3fn, torch.int8)
+# Profiling hook: when set to a callable, the pipeline is issued one stage per C-ABI call and
+# ``stage_callback(name)`` runs after each stage has been enqueued (bench.py records a HIP event
+# there).  The kernels and their order are identical to the single-call path.
+stage_callback = None
+
+_STAGES = (
+    ("prep", nv.STAGE_PREP),
+    ("act_quant", nv.STAGE_ACT_QUANT),
+    ("gate_up", nv.STAGE_GATE_UP),
+    ("requant", nv.STAGE_REQUANT),
+    ("down", nv.STAGE_DOWN),
+    ("combine", nv.STAGE_COMBINE),
+)
 
 
 def run_blockwise(
@@ -140,6 +151,18 @@ def run_blockwise(
     a.workspace = nv.ptr(ws)
     a.workspace_bytes = ws.numel()
     with torch.cuda.device(dev):
-        rc = L.moe_blockwise(ctypes.byref(a), nv.stream_ptr(dev))
+        if stage_callback is None:
+            rc = L.moe_blockwise(ctypes.byref(a), nv.stream_ptr(dev))
+        else:
+            rc = 0
+            for name, bit in _STAGES:
+                if name == "act_quant" and not (kind == nv.KIND_MXFP8 and hidden_states_scale is None):
+                    continue
+                if name == "requant" and kind != nv.KIND_FP8_ROW:
+                    continue
+                rc = L.moe_blockwise_stages(ctypes.byref(a), bit, nv.stream_ptr(dev))
+                if rc != 0:
+                    break
+                stage_callback(name)
     nv.check(rc, "moe_cte")
     return out
