@@ -416,5 +416,5 @@ def moe_mx_token_ref(x_row, e_list, aff_row, gate_up_proj_weight, gate_up_proj_s
         y = (act_fn(g.astype(np.float32), activation_function) * u.astype(np.float32)).astype(np.float32)
         yk = quantize_vec32(y[i_of_kk])
         wd = mx_dequant_down(down_proj_weight[e], down_proj_scale[e]).astype(np.float64)
-        total += float(to_bf16(np.float32(aff_row[e]))) * (yk.astype(np.float64) @ wd)
+        total += float(to_bf16(np.asarray([aff_row[e]], dtype=np.float32))[0]) * (yk.astype(np.float64) @ wd)
     return total

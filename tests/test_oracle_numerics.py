@@ -1,0 +1,52 @@
+"""Pins oracle/numerics.py against an independent library routine (torch's float8 / bfloat16 casts)
+and the formats' closed forms."""
+
+import numpy as np
+import torch
+
+from oracle import numerics as nm
+
+
+def test_e4m3fn_decode_is_the_closed_form_and_matches_torch():
+    codes = np.arange(256, dtype=np.uint8)
+    v = nm.e4m3fn_decode(codes)
+    tv = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    ok = ~np.isnan(tv)
+    assert np.array_equal(v[ok], tv[ok]) and np.isnan(v[~ok]).all()
+    assert v[0x7E] == 448.0 and v[0x77] == 240.0 and v[0x78] == 256.0 and v[0x01] == 2.0**-9 and v[0x08] == 2.0**-6
+
+
+def test_e4m3fn_encode_matches_torch_rne_on_random_and_boundaries():
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(400000) * rng.choice([1e-4, 1e-2, 1.0, 30.0, 300.0], 400000)).astype(np.float32)
+    x = np.clip(x, -448, 448)
+    # every midpoint between adjacent representable values (ties) and its fp32 neighbours
+    v = np.sort(nm.e4m3fn_decode(np.arange(0, 0x7F, dtype=np.uint8)))
+    mids = ((v[:-1].astype(np.float64) + v[1:]) / 2).astype(np.float32)
+    ties = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)), -mids])
+    x = np.concatenate([x, ties, v, -v])
+    ours = nm.e4m3fn_encode(x)
+    theirs = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(ours, theirs)
+
+
+def test_e4m3fn_roundtrip_every_code():
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    assert np.array_equal(nm.e4m3fn_encode(nm.e4m3fn_decode(codes)), codes)
+
+
+def test_bf16_round_matches_torch():
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(300000) * rng.choice([1e-20, 1e-3, 1.0, 1e4, 1e30], 300000)).astype(np.float32)
+    half = np.array([1.00390625, 1.01171875, -3.0078125], np.float32)  # exact ties between bf16 neighbours
+    x = np.concatenate([x, half])
+    assert np.array_equal(nm.to_bf16(x), torch.from_numpy(x).bfloat16().float().numpy())
+    assert np.array_equal(nm.bf16_from_bits(nm.bf16_bits(x)), nm.to_bf16(x))
+
+
+def test_e8m0_matches_torch():
+    b = np.arange(0, 255, dtype=np.uint8)
+    ours = nm.e8m0_decode(b)
+    theirs = torch.from_numpy(b).view(torch.float8_e8m0fnu).to(torch.float64).numpy()
+    ok = theirs > 0  # byte 0 (2^-127) is subnormal in fp32 and may flush in torch's cast
+    assert np.array_equal(ours[ok], theirs[ok]) and ours[127] == 1.0 and ours[0] == 2.0**-127
