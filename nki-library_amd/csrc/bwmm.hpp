@@ -37,6 +37,38 @@ struct GemmArgs {
   int32_t pI, nI;          // MXFP8: partitions per intermediate tile in the down weight, number of tiles
 };
 
+// Arguments of the large-tile MXFP8 kernels (bwmm_mx.hip).
+struct MxArgs {
+  const uint8_t* A;        // stage 1: MXFP8 activations [T1, H] in k' order; stage 2: intermediate [N*B, y_stride]
+  int64_t a_stride;
+  const uint8_t* A_scale;  // E8M0 [rows, a_scale_stride]
+  int64_t a_scale_stride;
+  const uint32_t* W;       // x4 weights in the reference layout
+  const uint8_t* W_scale;
+  const void* bias;
+  int32_t bias_dtype;
+  const void* aff;
+  int32_t aff_dtype;
+  const int32_t* tp2id;
+  const int32_t* n_chunks;
+  const int32_t* chunk_slot;
+  const int32_t* chunk_rows;
+  const int32_t* chunk_expert;
+  uint8_t* Yq;             // stage 1 output
+  uint8_t* Ys;
+  int64_t y_stride, ys_stride;
+  uint16_t* D;             // stage 2 output, bf16 [N*B, H]
+  int64_t H, I, E, n_real;
+  int32_t pI, nI;
+  int32_t act_fn, scaling_mode, clamp_mask;
+  float clamp[4];
+};
+
+// True when the large-tile kernels cover the shape: every intermediate tile holds a multiple
+// of 32 partitions (I % 128 == 0); other shapes run the general kernel.
+inline bool mx_fast_path_ok(int64_t H, int64_t I) { return H % 512 == 0 && I % 128 == 0; }
+int launch_mx_gemm(int stage, const MxArgs& m, unsigned gx, unsigned gy, hipStream_t s);
+
 int launch_gemm_stage(int kind, int stage, const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s);
 int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,
                        int64_t Iw, hipStream_t s);

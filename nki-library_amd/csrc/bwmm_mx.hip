@@ -1,0 +1,479 @@
+// MXFP8 blockwise expert GEMMs for gfx950, large-tile version.
+//
+// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 256 consecutive
+// slots of one expert (two 128-token blocks) and 256 output columns:
+//   gate/up: 32 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w
+//   down:    256 hidden columns; wave w owns 64 of them
+// so every weight byte that enters the CU is used by 256 rows.  Each wave keeps a 256 x 64
+// accumulator tile (16 x 4 MFMA 16x16 tiles, 256 accumulator registers).
+//
+// Operand traffic:
+//   * expert weights (B operand) go global -> registers, never through LDS.  In the reference
+//     layout a weight column's K runs over partitions p (4 K-bytes per 4-byte element), and lane
+//     group g of v_mfma_scale_f32_16x16x128_f8f6f4 needs K bytes [16g,16g+16) and [64+16g,
+//     64+16g+16) of the 128-byte K slice, i.e. partitions 4g..4g+3 and 16+4g..16+4g+3 of the 32
+//     partitions of the slice: eight loads per lane, each fetching 2 (gate/up) or 4 (down)
+//     adjacent columns = 2 or 4 MFMA column tiles at once.  One load instruction reads four
+//     full 128/256-byte row segments; every byte is loaded exactly once per workgroup.
+//   * activations (A operand, rows gathered through token_position_to_id) are staged through a
+//     double-buffered LDS tile of 256 rows x 128 K-bytes, read by all four waves.
+//   * E8M0 scales ride along: A scales sit in LDS transposed to [g][row%16][row/16] so that one
+//     16-byte read gives a lane the scales of all 16 row tiles (selected with op_sel); B scales
+//     are 2-4 bytes per lane per K slice straight from global.
+// The gate/up epilogue exchanges act(gate)*up through LDS so that the MX re-quantisation sees the
+// reference's blocks (8 partitions x 4 q) and writes K-contiguous rows for the down GEMM.
+//
+// Reference semantics: test/integration/nkilib/core/mlp/test_mlp_common.py:550-682 (layouts,
+// re-quantisation), test/integration/nkilib/core/moe/moe_cte/test_utils.py:474-735 (block loop).
+#include <type_traits>
+
+#include "bwmm.hpp"
+
+namespace moe {
+
+constexpr int MXT = 256;                       // threads
+constexpr int MXM = CHUNK_ROWS;                // 256 rows per workgroup
+constexpr int MXROW = 144;                     // LDS pitch of one staged row (128 + 16 pad)
+constexpr int MX_SA = MXM * MXROW;             // one A buffer
+constexpr int MX_SS = 4 * 16 * 16;             // one A-scale buffer, [g][c][mt] bytes
+constexpr int MX_LDS = 2 * MX_SA + 2 * MX_SS;  // 75776 bytes of dynamic LDS
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+struct BFrag {
+  v8i f[4];   // four column tiles
+  int sc[2];  // E8M0 scale bytes: gate/up stage: sc[0] = gate tiles 0,1 (bytes 0,1), sc[1] = up tiles;
+              // down stage: sc[0] = all four tiles (bytes 0..3)
+};
+
+__device__ __forceinline__ v8i frag_from_lds(const uint8_t* row, int g) {
+  const v4i lo = *(const v4i*)(row + 16 * g);
+  const v4i hi = *(const v4i*)(row + 64 + 16 * g);
+  v8i r;
+  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+  return r;
+}
+
+// One MFMA of row-tile fragment `af` (scale byte OA of `sa`) with column tile NT of `b`.
+template <int STAGE, int OA, int NT>
+__device__ __forceinline__ v4f mfma_tile(const v8i& af, const BFrag& b, const v4f& c, int sa) {
+  if constexpr (STAGE == 1)
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, b.f[NT], c, 0, 0, OA, sa, NT & 1, b.sc[NT >> 1]);
+  else
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, b.f[NT], c, 0, 0, OA, sa, NT, b.sc[0]);
+}
+
+// Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
+// wave-uniform 32-bit byte offset (SGPR), which is exactly the shape of every address in this
+// kernel, so no 64-bit per-lane pointer is ever formed.
+// (The descriptor and the uniform offsets are passed through readfirstlane: 64-bit address
+// arithmetic on uniform values is done by the vector ALU, and without the hint the compiler wraps
+// every load in a loop that checks whether all lanes agree on the descriptor.)
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int uni(int64_t v) { return __builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  const uint64_t addr = (uint64_t)p;
+  const uint32_t lo = (uint32_t)uni((int)(uint32_t)addr), hi = (uint32_t)uni((int)(uint32_t)(addr >> 32));
+  void* q = (void*)(((uint64_t)hi << 32) | lo);
+  return __builtin_amdgcn_make_buffer_rsrc(q, 0, uni((int)bytes), 0x00020000);
+}
+
+// NMT = number of 16-row tiles this instantiation multiplies (the chunk has at most NMT*16 rows).
+// Keeping it a compile-time constant keeps the K loop free of branches around the MFMAs.
+template <int STAGE, int NMT>
+__device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
+                                             int64_t slot0) {
+  uint8_t* sA = smem;
+  uint8_t* sS = smem + 2 * MX_SA;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
+  const int c = lane & 15, g = lane >> 4;
+  const int64_t nH = a.H / 512;
+
+  // ---- column tile ---------------------------------------------------------------------------
+  int tI = 0, p0 = 0, Pt = 128;
+  int64_t h0 = 0;
+  if (STAGE == 1) {
+    tI = blockIdx.x >> 2;
+    p0 = (blockIdx.x & 3) * 32;
+    const int64_t rows_t = (a.I - (int64_t)tI * 512 < 512) ? (a.I - (int64_t)tI * 512) : 512;
+    Pt = (int)(rows_t / 4);
+    if (p0 >= Pt) return;
+  } else {
+    h0 = (int64_t)blockIdx.x * 256;
+  }
+
+  // ---- rows: token ids, affinities ---------------------------------------------------------------
+  {
+    int id = -1;
+    if (tid < nrows) {
+      id = a.tp2id[slot0 + tid];
+      if (id < 0 || id >= a.n_real) id = -1;
+    }
+    s_tok[tid] = id;
+    if (STAGE == 2) {
+      float af = 0.f;
+      if (id >= 0 && a.aff)
+        af = (a.aff_dtype == MOE_DT_BF16) ? bf16_bits_to_f32(((const uint16_t*)a.aff)[(int64_t)id * a.E + e])
+                                          : ((const float*)a.aff)[(int64_t)id * a.E + e];
+      s_aff[tid] = af;
+    }
+  }
+  __syncthreads();
+
+  // A staging: thread covers rows (tid>>3) + 32 j, 16-byte chunk tid&7
+  const int arow0 = tid >> 3, ach = tid & 7;
+  constexpr int NAJ = NMT / 2;  // 32-row groups that hold rows of the NMT tiles
+  // Per-lane 32-bit byte offsets (row * stride + chunk); the K offset is wave-uniform and is added
+  // to the scalar base, so a load needs one VGPR of address.  Rows without a token (padding
+  // slots, rows past the end of the chunk) read some valid row instead of being zeroed: rows are
+  // independent in a GEMM and the results of such rows are never written out, so what they hold
+  // does not matter -- and the loads stay free of branches.
+  uint32_t a_voff[NAJ];
+#pragma unroll
+  for (int j = 0; j < NAJ; ++j) {
+    const int row = arow0 + 32 * j;
+    uint32_t r;
+    if (STAGE == 1) {
+      const int tok = s_tok[row];
+      r = (tok >= 0) ? (uint32_t)tok : 0u;
+    } else {
+      r = (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1)));
+    }
+    a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)(ach * 16);
+  }
+  // A scales: thread covers row tid
+  uint32_t as_voff;
+  if (STAGE == 1) {
+    const int tok = s_tok[tid];
+    as_voff = ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
+  } else {
+    as_voff = (uint32_t)(slot0 + ((tid < nrows) ? tid : (nrows - 1))) * (uint32_t)a.a_scale_stride;
+  }
+
+  // ---- K schedule -----------------------------------------------------------------------------------
+  // stage 1: ks -> (H tile ks>>2, partition group ks&3), all slices full.
+  // stage 2: slices of intermediate tile t are the first Pt(t)/32 partition groups.
+  int nks;
+  if (STAGE == 1) {
+    nks = (int)(a.H / 128);
+  } else {
+    const int64_t tail = a.I % 512;
+    nks = (int)((a.I / 512) * 4 + (tail / 128));
+  }
+  auto slice_of = [&](int ks, int& kt, int& pb) {
+    kt = ks >> 2;
+    pb = ks & 3;  // valid for both stages: only the last tile can be short and its slices come last
+  };
+
+  // ---- B operand addressing ---------------------------------------------------------------------------
+  // byte address inside the expert's weights = uniform part (gate/up, K tile, partition
+  // 32*pb + {r | 16 + r}, first column of the wave) + per-lane part (partition 4g, lane's columns).
+  int64_t w_pstride, w_tstride;  // element strides (4-byte weights; scales use the same counts in bytes)
+  __amdgpu_buffer_rsrc_t rw, rs;
+  uint32_t w_voff, s_voff;
+  int64_t colu;
+  if (STAGE == 1) {
+    w_pstride = 2 * nH * a.I;
+    w_tstride = a.I;
+    colu = (int64_t)tI * 512 + (int64_t)w * Pt + p0;
+    rw = make_rsrc(a.W + (int64_t)e * 128 * w_pstride, (uint32_t)(128 * w_pstride * 4));
+    rs = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
+    w_voff = (uint32_t)((4 * g * w_pstride + 2 * c) * 4);
+    s_voff = (uint32_t)(g * w_pstride + 2 * c);
+  } else {
+    w_pstride = (int64_t)a.nI * a.H;
+    w_tstride = a.H;
+    colu = h0 + 64 * w;
+    const int64_t sp = (a.pI + 7) / 8;
+    rw = make_rsrc(a.W + (int64_t)e * a.pI * w_pstride, (uint32_t)(a.pI * w_pstride * 4));
+    rs = make_rsrc(a.W_scale + (int64_t)e * sp * w_pstride, (uint32_t)(sp * w_pstride));
+    w_voff = (uint32_t)((4 * g * w_pstride + 4 * c) * 4);
+    s_voff = (uint32_t)(g * w_pstride + 4 * c);
+  }
+
+  auto load_b = [&](int ks, BFrag& b) {
+    int kt, pb;
+    slice_of(ks, kt, pb);
+    if (STAGE == 1) {
+#pragma unroll
+      for (int gu = 0; gu < 2; ++gu) {
+        const int64_t u0 = (int64_t)(pb * 32) * w_pstride + gu * nH * a.I + (int64_t)kt * w_tstride + colu;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const int pr = (r < 4) ? r : (16 + r - 4);
+          const v2i v = __builtin_amdgcn_raw_buffer_load_b64(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
+          b.f[gu * 2 + 0][r] = v[0];
+          b.f[gu * 2 + 1][r] = v[1];
+        }
+      }
+      const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu;
+      b.sc[0] = (int)__builtin_amdgcn_raw_buffer_load_b16(rs, s_voff, uni(us), 0);
+      b.sc[1] = (int)__builtin_amdgcn_raw_buffer_load_b16(rs, s_voff, uni(us + nH * a.I), 0);
+    } else {
+      const int64_t u0 = (int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride + colu;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int pr = (r < 4) ? r : (16 + r - 4);
+        const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
+        b.f[0][r] = v[0];
+        b.f[1][r] = v[1];
+        b.f[2][r] = v[2];
+        b.f[3][r] = v[3];
+      }
+      const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu;
+      b.sc[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, s_voff, uni(us), 0);
+      b.sc[1] = 0;
+    }
+  };
+
+  // ---- A operand staging ------------------------------------------------------------------------------
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a.A, 0xffffffffu);
+  const __amdgpu_buffer_rsrc_t ras = make_rsrc(a.A_scale, 0xffffffffu);
+  v4i areg[NAJ];
+  uint32_t asreg = 0;
+  auto load_a = [&](int ks) {
+    int kt, pb;
+    slice_of(ks, kt, pb);
+#pragma unroll
+    for (int j = 0; j < NAJ; ++j) areg[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[j], kt * 512 + pb * 128, 0);
+    asreg = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
+  };
+  auto store_a = [&](int buf) {
+    uint8_t* dst = sA + buf * MX_SA;
+#pragma unroll
+    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ach * 16) = areg[j];
+    // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
+    uint8_t* sd = sS + buf * MX_SS;
+    const int mt = tid >> 4, cc = tid & 15;
+#pragma unroll
+    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 16 + mt] = (uint8_t)((asreg >> (8 * gg)) & 0xffu);
+  };
+
+  v4f acc[NMT][4];
+  static_for<0, NMT>([&](auto mt) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = (v4f){0.f, 0.f, 0.f, 0.f};
+  });
+
+  // Row tiles are multiplied in groups of two; the fragments of the next group are read from LDS
+  // while the current group's eight MFMAs run.  The scheduling barriers keep the compiler from
+  // hoisting all sixteen fragment reads to the top (which would not fit the register file).
+  auto compute = [&](int buf, const BFrag& b) {
+    const uint8_t* src = sA + buf * MX_SA;
+    const v4i asc = *(const v4i*)(sS + buf * MX_SS + (g * 16 + c) * 16);
+    v8i af[2][2];
+    af[0][0] = frag_from_lds(src + (0 * 16 + c) * MXROW, g);
+    af[0][1] = frag_from_lds(src + (1 * 16 + c) * MXROW, g);
+    static_for<0, NMT / 2>([&](auto gi_) {
+      constexpr int gi = decltype(gi_)::value;
+      constexpr int cur = gi & 1, nxt = cur ^ 1;
+      if constexpr (gi + 1 < NMT / 2) {
+        af[nxt][0] = frag_from_lds(src + ((2 * gi + 2) * 16 + c) * MXROW, g);
+        af[nxt][1] = frag_from_lds(src + ((2 * gi + 3) * 16 + c) * MXROW, g);
+      }
+      {
+        constexpr int mt = 2 * gi;
+        const int sa = asc[mt / 4];
+        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][0], b, acc[mt][0], sa);
+        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][0], b, acc[mt][1], sa);
+        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][0], b, acc[mt][2], sa);
+        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][0], b, acc[mt][3], sa);
+      }
+      {
+        constexpr int mt = 2 * gi + 1;
+        const int sa = asc[mt / 4];
+        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][1], b, acc[mt][0], sa);
+        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][1], b, acc[mt][1], sa);
+        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][1], b, acc[mt][2], sa);
+        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][1], b, acc[mt][3], sa);
+      }
+      // Pin the eight results here, in accumulation registers.  Without a fixed point the
+      // compiler sinks the (side-effect free) MFMAs towards the end of the K step and hoists
+      // every fragment read to its top, which does not fit the register file; the memory clobber
+      // keeps the next group's LDS reads behind this point.
+      asm volatile("" : "+a"(acc[2 * gi][0]), "+a"(acc[2 * gi][1]), "+a"(acc[2 * gi][2]), "+a"(acc[2 * gi][3]),
+                        "+a"(acc[2 * gi + 1][0]), "+a"(acc[2 * gi + 1][1]), "+a"(acc[2 * gi + 1][2]),
+                        "+a"(acc[2 * gi + 1][3])
+                   :
+                   : "memory");
+    });
+  };
+
+  // ---- main loop: slice ks+1 is in flight (B in registers, A towards LDS) while slice ks multiplies ----
+  BFrag bc, bn;
+  load_a(0);
+  load_b(0, bc);
+  store_a(0);
+  __syncthreads();
+#pragma clang loop unroll(disable)
+  for (int ks = 0; ks < nks; ++ks) {
+    const bool more = ks + 1 < nks;
+    if (more) {
+      load_a(ks + 1);
+      load_b(ks + 1, bn);
+    }
+    compute(ks & 1, bc);
+    if (more) store_a((ks + 1) & 1);
+    __syncthreads();
+    bc = bn;
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------------
+  if (STAGE == 1) {
+    // Raw gate and up accumulators go through LDS, 64 rows at a time, as [row][p_local 32][q 4] fp32
+    // (gate at E, up 32 KB further); then one thread per MX block (8 partitions x 4 q) applies bias,
+    // clamps and act(gate)*up, quantises and writes 32 K-contiguous bytes plus the scale byte.
+    float* E = (float*)smem;
+    const int q = w;
+    static_for<0, NMT / 4>([&](auto ps_) {
+      constexpr int ps = decltype(ps_)::value;
+      if (ps * 64 < nrows) {
+        __syncthreads();
+        static_for<0, 4>([&](auto m_) {
+          constexpr int ml = decltype(m_)::value;
+          constexpr int mt = ps * 4 + ml;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int rl = ml * 16 + 4 * g + r;
+              E[(rl * 32 + 2 * c + t) * 4 + q] = acc[mt][t][r];
+              E[8192 + (rl * 32 + 2 * c + t) * 4 + q] = acc[mt][2 + t][r];
+            }
+          }
+        });
+        __syncthreads();
+        // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions p0+8j .. p0+8j+7 (x 4 q)
+        const int rl = tid >> 2, j = tid & 3;
+        const int row = ps * 64 + rl;
+        if (row < nrows) {
+          float* sg = E + (rl * 32 + 8 * j) * 4;
+          const float* su = E + 8192 + (rl * 32 + 8 * j) * 4;
+          float am = 0.f;
+#pragma unroll 1
+          for (int k = 0; k < 8; ++k) {
+            const float4 g4 = *(const float4*)(sg + 4 * k), u4 = *(const float4*)(su + 4 * k);
+            float gv[4] = {g4.x, g4.y, g4.z, g4.w};
+            float uv[4] = {u4.x, u4.y, u4.z, u4.w};
+            if (a.bias) {
+              const int64_t p = p0 + 8 * j + k;
+              const int64_t ig = ((((int64_t)e * a.pI + p) * 2 + 0) * a.nI + tI) * 4;
+              const int64_t iu = ((((int64_t)e * a.pI + p) * 2 + 1) * a.nI + tI) * 4;
+#pragma unroll
+              for (int qq = 0; qq < 4; ++qq) {
+                if (a.bias_dtype == MOE_DT_BF16) {
+                  gv[qq] += bf16_bits_to_f32(((const uint16_t*)a.bias)[ig + qq]);
+                  uv[qq] += bf16_bits_to_f32(((const uint16_t*)a.bias)[iu + qq]);
+                } else {
+                  gv[qq] += ((const float*)a.bias)[ig + qq];
+                  uv[qq] += ((const float*)a.bias)[iu + qq];
+                }
+              }
+            }
+            float yv[4];
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq) {
+              float gg = gv[qq], uu = uv[qq];
+              if (a.clamp_mask & MOE_CLAMP_GATE_LO) gg = fmaxf(gg, a.clamp[1]);
+              if (a.clamp_mask & MOE_CLAMP_GATE_HI) gg = fminf(gg, a.clamp[0]);
+              if (a.clamp_mask & MOE_CLAMP_UP_LO) uu = fmaxf(uu, a.clamp[3]);
+              if (a.clamp_mask & MOE_CLAMP_UP_HI) uu = fminf(uu, a.clamp[2]);
+              yv[qq] = act_apply(gg, a.act_fn) * uu;
+              am = fmaxf(am, fabsf(yv[qq]));
+            }
+            *(float4*)(sg + 4 * k) = make_float4(yv[0], yv[1], yv[2], yv[3]);  // in place: only this thread reads it
+          }
+          const uint32_t sb = mx_scale_byte(am);
+          const float is = mx_inv_scale(sb);
+          uint32_t d[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const float4 y4 = *(const float4*)(sg + 4 * k);
+            d[k] = pack4_e4m3(clip448(y4.x * is), clip448(y4.y * is), clip448(y4.z * is), clip448(y4.w * is));
+          }
+          const int64_t slot = slot0 + row;
+          uint4* o = (uint4*)(a.Yq + slot * a.y_stride + tI * 512 + (p0 + 8 * j) * 4);
+          o[0] = make_uint4(d[0], d[1], d[2], d[3]);
+          o[1] = make_uint4(d[4], d[5], d[6], d[7]);
+          a.Ys[slot * a.ys_stride + tI * 16 + (p0 >> 3) + j] = (uint8_t)sb;
+        }
+      }
+    });
+  } else {
+    const int64_t col0 = h0 + 64 * w + 4 * c;
+    float bd[4] = {0.f, 0.f, 0.f, 0.f};
+    if (a.bias) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int64_t ib = (int64_t)e * a.H + col0 + t;
+        bd[t] = (a.bias_dtype == MOE_DT_BF16) ? bf16_bits_to_f32(((const uint16_t*)a.bias)[ib]) : ((const float*)a.bias)[ib];
+      }
+    }
+    const bool post = a.scaling_mode == MOE_SCALE_POST;
+    static_for<0, NMT>([&](auto mt_) {
+      constexpr int mt = decltype(mt_)::value;
+      {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = mt * 16 + 4 * g + r;
+          if (row < nrows && s_tok[row] >= 0) {
+            const float af = post ? s_aff[row] : 1.f;
+            uint32_t o[2];
+#pragma unroll
+            for (int t = 0; t < 4; t += 2) {
+              const float d0 = (acc[mt][t][r] + bd[t]) * af;
+              const float d1 = (acc[mt][t + 1][r] + bd[t + 1]) * af;
+              o[t >> 1] = (uint32_t)f32_to_bf16_bits(d0) | ((uint32_t)f32_to_bf16_bits(d1) << 16);
+            }
+            *(uint2*)(a.D + (slot0 + row) * a.H + col0) = make_uint2(o[0], o[1]);
+          }
+        }
+      }
+    });
+  }
+}
+
+template <int STAGE>
+__global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  __shared__ int s_tok[MXM];
+  __shared__ float s_aff[MXM];
+  const int chunk = blockIdx.y;
+  if (chunk >= *a.n_chunks) return;
+  // values read from memory at a uniform address are uniform; say so, so that everything derived
+  // from them (buffer descriptors, scalar offsets) stays in scalar registers
+  const int nrows = __builtin_amdgcn_readfirstlane(a.chunk_rows[chunk]);
+  const int e = __builtin_amdgcn_readfirstlane(a.chunk_expert[chunk]);
+  const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
+  if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0);
+  else if (nrows <= 128) mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0);
+  else mx_gemm_body<STAGE, 16>(a, smem, s_tok, s_aff, nrows, e, slot0);
+}
+
+int launch_mx_gemm(int stage, const MxArgs& m, unsigned gx, unsigned gy, hipStream_t s) {
+  if (gx == 0 || gy == 0) return MOE_OK;
+  hipError_t err;
+  if (stage == 1) {
+    err = hipFuncSetAttribute((const void*)mx_gemm_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
+    if (err != hipSuccess) return MOE_E_LAUNCH;
+    hipLaunchKernelGGL(mx_gemm_kernel<1>, dim3(gx, gy), dim3(MXT), MX_LDS, s, m);
+  } else {
+    err = hipFuncSetAttribute((const void*)mx_gemm_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
+    if (err != hipSuccess) return MOE_E_LAUNCH;
+    hipLaunchKernelGGL(mx_gemm_kernel<2>, dim3(gx, gy), dim3(MXT), MX_LDS, s, m);
+  }
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+}  // namespace moe

@@ -207,8 +207,39 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     gx1 = (unsigned)((a->I + 127) / 128);
   }
 
+  const bool mx_fast = a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I);
+  MxArgs m;
+  memset(&m, 0, sizeof(m));
+  if (mx_fast) {
+    m.bias_dtype = a->bias_dtype;
+    m.aff = g.aff;
+    m.aff_dtype = a->affinity_dtype;
+    m.tp2id = a->token_position_to_id;
+    m.n_chunks = bk.n_chunks;
+    m.chunk_slot = bk.chunk_slot;
+    m.chunk_rows = bk.chunk_rows;
+    m.chunk_expert = bk.chunk_expert;
+    m.Yq = ws + p.yq;
+    m.Ys = ws + p.ys;
+    m.y_stride = p.Iw;
+    m.ys_stride = p.Iw / 32;
+    m.D = (uint16_t*)(ws + p.d);
+    m.H = a->H; m.I = a->I; m.E = a->E; m.n_real = n_real;
+    m.pI = (int32_t)p.pI; m.nI = (int32_t)p.nI;
+    m.act_fn = a->act_fn; m.scaling_mode = a->scaling_mode; m.clamp_mask = a->clamp_mask;
+    for (int i = 0; i < 4; ++i) m.clamp[i] = g.clamp[i];
+  }
+  const unsigned gyc = (unsigned)bk.max_chunks;
   if (stages & MOE_STAGE_GATE_UP) {
-    rc = launch_gemm_stage(a->kind, 1, g1, gx1, gy, s);
+    if (mx_fast) {
+      MxArgs m1 = m;
+      m1.A = g1.A; m1.a_stride = g1.a_stride; m1.A_scale = g1.A_scale; m1.a_scale_stride = g1.a_scale_stride;
+      m1.W = (const uint32_t*)a->gate_up_proj_weight; m1.W_scale = (const uint8_t*)a->gate_up_proj_scale;
+      m1.bias = a->gate_and_up_proj_bias;
+      rc = launch_mx_gemm(1, m1, (unsigned)(p.nI * 4), gyc, s);
+    } else {
+      rc = launch_gemm_stage(a->kind, 1, g1, gx1, gy, s);
+    }
     if (rc != MOE_OK) return rc;
   }
   if (a->kind == MOE_KIND_FP8_ROW && (stages & MOE_STAGE_REQUANT)) {
@@ -216,7 +247,15 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     if (rc != MOE_OK) return rc;
   }
   if (stages & MOE_STAGE_DOWN) {
-    rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);
+    if (mx_fast) {
+      MxArgs m2 = m;
+      m2.A = ws + p.yq; m2.a_stride = p.Iw; m2.A_scale = ws + p.ys; m2.a_scale_stride = p.Iw / 32;
+      m2.W = (const uint32_t*)a->down_proj_weight; m2.W_scale = (const uint8_t*)a->down_proj_scale;
+      m2.bias = a->down_proj_bias;
+      rc = launch_mx_gemm(2, m2, (unsigned)(a->H / 256), gyc, s);
+    } else {
+      rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);
+    }
     if (rc != MOE_OK) return rc;
   }
   if (stages & MOE_STAGE_COMBINE) return launch_combine(bk, a, ws + p.d, n_real, s);

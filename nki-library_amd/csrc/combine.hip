@@ -50,6 +50,39 @@ __global__ __launch_bounds__(256) void prep_blocks_kernel(const int32_t* __restr
   }
 }
 
+// Single workgroup, run after prep_blocks_kernel.  Thread 0 walks the blocks once (N is a few
+// thousand at most) and emits the expert chunks.
+__global__ __launch_bounds__(64) void build_chunks_kernel(const int32_t* __restrict__ b2e,
+                                                          const int32_t* __restrict__ n_active,
+                                                          const int32_t* __restrict__ valid_rows, int64_t N, int64_t B,
+                                                          int64_t E, int32_t* __restrict__ n_chunks,
+                                                          int32_t* __restrict__ chunk_slot,
+                                                          int32_t* __restrict__ chunk_rows,
+                                                          int32_t* __restrict__ chunk_expert, int64_t max_chunks) {
+  if (threadIdx.x != 0) return;
+  const int64_t na = *n_active;
+  int64_t nc = 0;
+  int64_t b = 0;
+  while (b < na) {
+    const int e = b2e[b];
+    int64_t j = b, last_end = -1;
+    while (j < na && b2e[j] == e) {
+      if (valid_rows[j] > 0) last_end = j * B + valid_rows[j];
+      ++j;
+    }
+    if (e >= 0 && e < E && last_end > b * B) {
+      for (int64_t s0 = b * B; s0 < last_end && nc < max_chunks; s0 += CHUNK_ROWS) {
+        chunk_slot[nc] = (int32_t)s0;
+        chunk_rows[nc] = (int32_t)((last_end - s0 < CHUNK_ROWS) ? (last_end - s0) : CHUNK_ROWS);
+        chunk_expert[nc] = e;
+        ++nc;
+      }
+    }
+    b = j;
+  }
+  *n_chunks = (int32_t)nc;
+}
+
 __global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* __restrict__ p, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -160,9 +193,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
 // ---- host-side orchestration used by moe_blockwise() -------------------------------------
 
 size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B) {
-  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B], each region 256-byte aligned
+  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B] | n_chunks[4] | 3 x chunk[max_chunks],
+  // each region 256-byte aligned
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
-  return al(16) + al((size_t)N * 4) + 2 * al((size_t)T1 * 4) + al((size_t)(T1 + 1) * 4) + al((size_t)N * B * 4);
+  return al(16) + al((size_t)N * 4) + 2 * al((size_t)T1 * 4) + al((size_t)(T1 + 1) * 4) + al((size_t)N * B * 4) +
+         al(16) + 3 * al((size_t)max_chunks_for(N, B) * 4);
 }
 
 Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
@@ -174,7 +209,12 @@ Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
   k.cnt = (int32_t*)p; p += al((size_t)T1 * 4);
   k.cursor = (int32_t*)p; p += al((size_t)T1 * 4);
   k.off = (int32_t*)p; p += al((size_t)(T1 + 1) * 4);
-  k.list = (int32_t*)p;
+  k.list = (int32_t*)p; p += al((size_t)N * B * 4);
+  k.max_chunks = max_chunks_for(N, B);
+  k.n_chunks = (int32_t*)p; p += al(16);
+  k.chunk_slot = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
+  k.chunk_rows = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
+  k.chunk_expert = (int32_t*)p;
   return k;
 }
 
@@ -188,6 +228,9 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
   const unsigned g = (unsigned)(a->N < 1024 ? a->N : 1024);
   hipLaunchKernelGGL(prep_blocks_kernel, dim3(g), dim3(256), 0, s, a->token_position_to_id, a->block_to_expert,
                      a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows);
+  MOE_CHECK_LAUNCH();
+  hipLaunchKernelGGL(build_chunks_kernel, dim3(1), dim3(64), 0, s, a->block_to_expert, k.n_active, k.valid_rows, a->N,
+                     a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.max_chunks);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
   const unsigned gs = (unsigned)((slots + 255) / 256);
