@@ -37,10 +37,13 @@ def parse_args():
     ap.add_argument("--workload", default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-blocks", type=int, default=6, help="blocks of the workload timed on the CPU oracle")
+    ap.add_argument("--routing", default="router", choices=["router", "balanced"],
+                    help="router: top-k of synthetic scores (the reported workload); balanced: every expert gets "
+                         "exactly T*k/E rows (diagnostic, shows the cost of ragged expert loads)")
     return ap.parse_args()
 
 
-def build_workload(name, dev):
+def build_workload(name, dev, routing="router"):
     import torch
     from nkilib import synthetic as syn
 
@@ -56,6 +59,13 @@ def build_workload(name, dev):
     t0 = time.time()
     gu_q, gu_s, d_q, d_s = syn.mx_expert_weights(E, H, I, 0.02, dev, seed=0)
     ids, aff = syn.route(T, E, k, dev, seed=0, **router_kw)
+    if routing == "balanced":
+        tt = torch.arange(T, device=dev).reshape(T, 1)
+        jj = torch.arange(k, device=dev).reshape(1, k)
+        ids = ((tt + jj * (E // k)) % E).to(torch.int32).contiguous()
+        aff = torch.zeros((T + 1, E), dtype=torch.float32, device=dev)
+        aff[:T].scatter_(1, ids.long(), torch.full((T, k), 1.0 / k, device=dev))
+        aff = aff.to(torch.bfloat16)
     x = syn.hidden_states(T, H, dev, seed=0)
     gamma = torch.ones((1, H), dtype=torch.bfloat16, device=dev)
     torch.cuda.synchronize()
@@ -125,7 +135,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     dev = torch.device("cuda:0")
     nv.check(nv.lib().moe_check_device(), "device check")
-    cfg, t = build_workload(args.workload, dev)
+    cfg, t = build_workload(args.workload, dev, args.routing)
     T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
     N = get_n_blocks(T, k, E, B, n_block_per_iter=2)
     spec = MoECTESpec(implementation=MoECTEImplementation.shard_on_block_mx)

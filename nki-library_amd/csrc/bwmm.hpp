@@ -62,6 +62,7 @@ struct MxArgs {
   int32_t pI, nI;
   int32_t act_fn, scaling_mode, clamp_mask;
   float clamp[4];
+  int32_t col_tiles;       // column tiles per chunk (set by the launcher)
 };
 
 // True when the large-tile kernels cover the shape: every intermediate tile holds a multiple

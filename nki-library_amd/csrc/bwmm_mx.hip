@@ -33,10 +33,12 @@ namespace moe {
 
 constexpr int MXT = 256;                       // threads
 constexpr int MXM = CHUNK_ROWS;                // 256 rows per workgroup
-constexpr int MXROW = 144;                     // LDS pitch of one staged row (128 + 16 pad)
+constexpr int MXROW = 128;                     // LDS pitch of one staged row; 16-byte chunk ch of row r sits in
+                                               // slot ch ^ (r & 7), which makes the fragment reads (16 rows x 4
+                                               // chunks per instruction) and the staging writes conflict free
 constexpr int MX_SA = MXM * MXROW;             // one A buffer
 constexpr int MX_SS = 4 * 16 * 16;             // one A-scale buffer, [g][c][mt] bytes
-constexpr int MX_LDS = 2 * MX_SA + 2 * MX_SS;  // 75776 bytes of dynamic LDS
+constexpr int MX_LDS = 2 * MX_SA + 2 * MX_SS;  // 67584 bytes of dynamic LDS (the gate/up epilogue needs 65536)
 
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -52,9 +54,9 @@ struct BFrag {
               // down stage: sc[0] = all four tiles (bytes 0..3)
 };
 
-__device__ __forceinline__ v8i frag_from_lds(const uint8_t* row, int g) {
-  const v4i lo = *(const v4i*)(row + 16 * g);
-  const v4i hi = *(const v4i*)(row + 64 + 16 * g);
+__device__ __forceinline__ v8i frag_from_lds(const uint8_t* plo, const uint8_t* phi) {
+  const v4i lo = *(const v4i*)plo;
+  const v4i hi = *(const v4i*)phi;
   v8i r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
   r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
@@ -89,7 +91,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 // Keeping it a compile-time constant keeps the K loop free of branches around the MFMAs.
 template <int STAGE, int NMT>
 __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
-                                             int64_t slot0) {
+                                             int64_t slot0, int xt) {
   uint8_t* sA = smem;
   uint8_t* sS = smem + 2 * MX_SA;
 
@@ -103,13 +105,13 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   int tI = 0, p0 = 0, Pt = 128;
   int64_t h0 = 0;
   if (STAGE == 1) {
-    tI = blockIdx.x >> 2;
-    p0 = (blockIdx.x & 3) * 32;
+    tI = xt >> 2;
+    p0 = (xt & 3) * 32;
     const int64_t rows_t = (a.I - (int64_t)tI * 512 < 512) ? (a.I - (int64_t)tI * 512) : 512;
     Pt = (int)(rows_t / 4);
     if (p0 >= Pt) return;
   } else {
-    h0 = (int64_t)blockIdx.x * 256;
+    h0 = (int64_t)xt * 256;
   }
 
   // ---- rows: token ids, affinities ---------------------------------------------------------------
@@ -239,19 +241,22 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // ---- A operand staging ------------------------------------------------------------------------------
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(a.A, 0xffffffffu);
   const __amdgpu_buffer_rsrc_t ras = make_rsrc(a.A_scale, 0xffffffffu);
-  v4i areg[NAJ];
-  uint32_t asreg = 0;
-  auto load_a = [&](int ks) {
+  struct AStage {
+    v4i d[NAJ];
+    uint32_t sc;
+  };
+  auto load_a = [&](int ks, AStage& r) {
     int kt, pb;
     slice_of(ks, kt, pb);
 #pragma unroll
-    for (int j = 0; j < NAJ; ++j) areg[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[j], kt * 512 + pb * 128, 0);
-    asreg = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
+    for (int j = 0; j < NAJ; ++j) r.d[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[j], kt * 512 + pb * 128, 0);
+    r.sc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
   };
-  auto store_a = [&](int buf) {
+  auto store_a = [&](int buf, const AStage& r) {
+    const uint32_t asreg = r.sc;
     uint8_t* dst = sA + buf * MX_SA;
 #pragma unroll
-    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ach * 16) = areg[j];
+    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
     // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
     uint8_t* sd = sS + buf * MX_SS;
     const int mt = tid >> 4, cc = tid & 15;
@@ -268,19 +273,26 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // Row tiles are multiplied in groups of two; the fragments of the next group are read from LDS
   // while the current group's eight MFMAs run.  The scheduling barriers keep the compiler from
   // hoisting all sixteen fragment reads to the top (which would not fit the register file).
+  const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   auto compute = [&](int buf, const BFrag& b) {
-    const uint8_t* src = sA + buf * MX_SA;
+    const uint8_t* plo = sA + buf * MX_SA + rd_lo;
+    const uint8_t* phi = sA + buf * MX_SA + rd_hi;
     const v4i asc = *(const v4i*)(sS + buf * MX_SS + (g * 16 + c) * 16);
     v8i af[2][2];
-    af[0][0] = frag_from_lds(src + (0 * 16 + c) * MXROW, g);
-    af[0][1] = frag_from_lds(src + (1 * 16 + c) * MXROW, g);
+    af[0][0] = frag_from_lds(plo, phi);
+    af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
     static_for<0, NMT / 2>([&](auto gi_) {
       constexpr int gi = decltype(gi_)::value;
       constexpr int cur = gi & 1, nxt = cur ^ 1;
       if constexpr (gi + 1 < NMT / 2) {
-        af[nxt][0] = frag_from_lds(src + ((2 * gi + 2) * 16 + c) * MXROW, g);
-        af[nxt][1] = frag_from_lds(src + ((2 * gi + 3) * 16 + c) * MXROW, g);
+        af[nxt][0] = frag_from_lds(plo + (2 * gi + 2) * 16 * MXROW, phi + (2 * gi + 2) * 16 * MXROW);
+        af[nxt][1] = frag_from_lds(plo + (2 * gi + 3) * 16 * MXROW, phi + (2 * gi + 3) * 16 * MXROW);
       }
+      // Fixed point between "next group's reads issued" and "this group's MFMAs": the reads above
+      // cannot sink below it (memory clobber) and the MFMAs below cannot rise above it (they use the
+      // fragments it returns), so the two fragment sets stay live together and the LDS latency of
+      // the next group is covered by this group's eight MFMAs.
+      asm volatile("" : "+v"(af[cur][0]), "+v"(af[cur][1]) : : "memory");
       {
         constexpr int mt = 2 * gi;
         const int sa = asc[mt / 4];
@@ -299,8 +311,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       }
       // Pin the eight results here, in accumulation registers.  Without a fixed point the
       // compiler sinks the (side-effect free) MFMAs towards the end of the K step and hoists
-      // every fragment read to its top, which does not fit the register file; the memory clobber
-      // keeps the next group's LDS reads behind this point.
+      // every fragment read to its top, which does not fit the register file.
       asm volatile("" : "+a"(acc[2 * gi][0]), "+a"(acc[2 * gi][1]), "+a"(acc[2 * gi][2]), "+a"(acc[2 * gi][3]),
                         "+a"(acc[2 * gi + 1][0]), "+a"(acc[2 * gi + 1][1]), "+a"(acc[2 * gi + 1][2]),
                         "+a"(acc[2 * gi + 1][3])
@@ -310,22 +321,32 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   };
 
   // ---- main loop: slice ks+1 is in flight (B in registers, A towards LDS) while slice ks multiplies ----
-  BFrag bc, bn;
-  load_a(0);
+  // Software pipeline, two K slices deep for both operands: while slice ks multiplies, the loads
+  // of slice ks+2 (A into registers, B into registers) are being issued and those of slice ks+1,
+  // issued a full slice earlier, are stored to LDS (A) / rotated into place (B).  Every load
+  // therefore has at least one whole slice of MFMA work to complete.
+  BFrag bc, b1, b2;
+  AStage a1, a2;
+  load_a(0, a1);
   load_b(0, bc);
-  store_a(0);
+  store_a(0, a1);
+  if (nks > 1) {
+    load_a(1, a1);
+    load_b(1, b1);
+  }
   __syncthreads();
 #pragma clang loop unroll(disable)
   for (int ks = 0; ks < nks; ++ks) {
-    const bool more = ks + 1 < nks;
-    if (more) {
-      load_a(ks + 1);
-      load_b(ks + 1, bn);
+    if (ks + 2 < nks) {
+      load_a(ks + 2, a2);
+      load_b(ks + 2, b2);
     }
     compute(ks & 1, bc);
-    if (more) store_a((ks + 1) & 1);
+    if (ks + 1 < nks) store_a((ks + 1) & 1, a1);
     __syncthreads();
-    bc = bn;
+    bc = b1;
+    b1 = b2;
+    a1 = a2;
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
@@ -448,29 +469,41 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_tok[MXM];
   __shared__ float s_aff[MXM];
-  const int chunk = blockIdx.y;
-  if (chunk >= *a.n_chunks) return;
+  // Workgroups are handed to the 8 XCDs round-robin by linear index, and each XCD has its own L2.
+  // XCD x therefore takes the x-th contiguous eighth of the chunk list (chunks are ordered by
+  // expert), and walks it chunk by chunk with the column tiles innermost: the workgroups that share
+  // an activation tile, and the chunks that share an expert's weights, then run at the same time
+  // behind the same L2, so each operand crosses the fabric about once.
+  const int n_chunks = __builtin_amdgcn_readfirstlane(*a.n_chunks);
+  const int per_xcd = (n_chunks + 7) >> 3;
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const int local = j / a.col_tiles, xt = j - local * a.col_tiles;
+  const int chunk = xcd * per_xcd + local;
+  if (local >= per_xcd || chunk >= n_chunks) return;
   // values read from memory at a uniform address are uniform; say so, so that everything derived
   // from them (buffer descriptors, scalar offsets) stays in scalar registers
   const int nrows = __builtin_amdgcn_readfirstlane(a.chunk_rows[chunk]);
   const int e = __builtin_amdgcn_readfirstlane(a.chunk_expert[chunk]);
   const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
-  if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0);
-  else if (nrows <= 128) mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0);
-  else mx_gemm_body<STAGE, 16>(a, smem, s_tok, s_aff, nrows, e, slot0);
+  if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  else if (nrows <= 128) mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  else mx_gemm_body<STAGE, 16>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
 }
 
-int launch_mx_gemm(int stage, const MxArgs& m, unsigned gx, unsigned gy, hipStream_t s) {
+int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {
   if (gx == 0 || gy == 0) return MOE_OK;
+  MxArgs m = m0;
+  m.col_tiles = (int32_t)gx;
+  const unsigned grid = 8u * ((gy + 7u) / 8u) * gx;  // gy = upper bound on the number of chunks
   hipError_t err;
   if (stage == 1) {
     err = hipFuncSetAttribute((const void*)mx_gemm_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
     if (err != hipSuccess) return MOE_E_LAUNCH;
-    hipLaunchKernelGGL(mx_gemm_kernel<1>, dim3(gx, gy), dim3(MXT), MX_LDS, s, m);
+    hipLaunchKernelGGL(mx_gemm_kernel<1>, dim3(grid), dim3(MXT), MX_LDS, s, m);
   } else {
     err = hipFuncSetAttribute((const void*)mx_gemm_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
     if (err != hipSuccess) return MOE_E_LAUNCH;
-    hipLaunchKernelGGL(mx_gemm_kernel<2>, dim3(gx, gy), dim3(MXT), MX_LDS, s, m);
+    hipLaunchKernelGGL(mx_gemm_kernel<2>, dim3(grid), dim3(MXT), MX_LDS, s, m);
   }
   MOE_CHECK_LAUNCH();
   return MOE_OK;

@@ -50,37 +50,58 @@ __global__ __launch_bounds__(256) void prep_blocks_kernel(const int32_t* __restr
   }
 }
 
-// Single workgroup, run after prep_blocks_kernel.  Thread 0 walks the blocks once (N is a few
-// thousand at most) and emits the expert chunks.
-__global__ __launch_bounds__(64) void build_chunks_kernel(const int32_t* __restrict__ b2e,
-                                                          const int32_t* __restrict__ n_active,
-                                                          const int32_t* __restrict__ valid_rows, int64_t N, int64_t B,
-                                                          int64_t E, int32_t* __restrict__ n_chunks,
-                                                          int32_t* __restrict__ chunk_slot,
-                                                          int32_t* __restrict__ chunk_rows,
-                                                          int32_t* __restrict__ chunk_expert, int64_t max_chunks) {
-  if (threadIdx.x != 0) return;
+// Single workgroup of 1024 threads, run after prep_blocks_kernel.  A "run" is a maximal sequence of
+// consecutive active blocks of one expert; the thread that owns a run's first block measures the
+// run (slots up to its last real token) and, after a block-wide scan of the chunk counts, writes
+// the run's chunks.  Chunk order follows block order.
+__global__ __launch_bounds__(1024) void build_chunks_kernel(const int32_t* __restrict__ b2e,
+                                                            const int32_t* __restrict__ n_active,
+                                                            const int32_t* __restrict__ valid_rows, int64_t N,
+                                                            int64_t B, int64_t E, int32_t* __restrict__ n_chunks,
+                                                            int32_t* __restrict__ chunk_slot,
+                                                            int32_t* __restrict__ chunk_rows,
+                                                            int32_t* __restrict__ chunk_expert, int64_t max_chunks) {
+  __shared__ int s_scan[1024];
+  __shared__ int s_carry;
   const int64_t na = *n_active;
-  int64_t nc = 0;
-  int64_t b = 0;
-  while (b < na) {
-    const int e = b2e[b];
-    int64_t j = b, last_end = -1;
-    while (j < na && b2e[j] == e) {
-      if (valid_rows[j] > 0) last_end = j * B + valid_rows[j];
-      ++j;
-    }
-    if (e >= 0 && e < E && last_end > b * B) {
-      for (int64_t s0 = b * B; s0 < last_end && nc < max_chunks; s0 += CHUNK_ROWS) {
-        chunk_slot[nc] = (int32_t)s0;
-        chunk_rows[nc] = (int32_t)((last_end - s0 < CHUNK_ROWS) ? (last_end - s0) : CHUNK_ROWS);
-        chunk_expert[nc] = e;
-        ++nc;
+  if (threadIdx.x == 0) s_carry = 0;
+  __syncthreads();
+  for (int64_t b0 = 0; b0 < na; b0 += 1024) {
+    const int64_t b = b0 + threadIdx.x;
+    int nch = 0;
+    int64_t last_end = -1;
+    int e = -1;
+    if (b < na) {
+      e = b2e[b];
+      const bool start = (b == 0) || (b2e[b - 1] != e);
+      if (start && e >= 0 && e < E) {
+        for (int64_t j = b; j < na && b2e[j] == e; ++j)
+          if (valid_rows[j] > 0) last_end = j * B + valid_rows[j];
+        if (last_end > b * B) nch = (int)((last_end - b * B + CHUNK_ROWS - 1) / CHUNK_ROWS);
       }
     }
-    b = j;
+    s_scan[threadIdx.x] = nch;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+      const int v = (threadIdx.x >= (unsigned)o) ? s_scan[threadIdx.x - o] : 0;
+      __syncthreads();
+      s_scan[threadIdx.x] += v;
+      __syncthreads();
+    }
+    const int base = s_carry + s_scan[threadIdx.x] - nch;
+    for (int k = 0; k < nch; ++k) {
+      const int64_t s0 = b * B + (int64_t)k * CHUNK_ROWS;
+      if (base + k < max_chunks) {
+        chunk_slot[base + k] = (int32_t)s0;
+        chunk_rows[base + k] = (int32_t)((last_end - s0 < CHUNK_ROWS) ? (last_end - s0) : CHUNK_ROWS);
+        chunk_expert[base + k] = e;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) s_carry += s_scan[1023];
+    __syncthreads();
   }
-  *n_chunks = (int32_t)nc;
+  if (threadIdx.x == 0) *n_chunks = (int32_t)((s_carry < max_chunks) ? s_carry : max_chunks);
 }
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* __restrict__ p, int64_t n) {
@@ -229,7 +250,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
   hipLaunchKernelGGL(prep_blocks_kernel, dim3(g), dim3(256), 0, s, a->token_position_to_id, a->block_to_expert,
                      a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows);
   MOE_CHECK_LAUNCH();
-  hipLaunchKernelGGL(build_chunks_kernel, dim3(1), dim3(64), 0, s, a->block_to_expert, k.n_active, k.valid_rows, a->N,
+  hipLaunchKernelGGL(build_chunks_kernel, dim3(1), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows, a->N,
                      a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.max_chunks);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
