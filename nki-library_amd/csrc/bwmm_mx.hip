@@ -1,11 +1,14 @@
 // MXFP8 blockwise expert GEMMs for gfx950, large-tile version.
 //
-// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 256 consecutive
-// slots of one expert (two 128-token blocks) and 256 output columns:
-//   gate/up: 32 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w
-//   down:    256 hidden columns; wave w owns 64 of them
-// so every weight byte that enters the CU is used by 256 rows.  Each wave keeps a 256 x 64
-// accumulator tile (16 x 4 MFMA 16x16 tiles, 256 accumulator registers).
+// A 512-thread workgroup (8 waves, two per SIMD) owns an "expert chunk" of up to 128 consecutive
+// slots of one expert and 512 output columns:
+//   gate/up: 64 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w & 3 and
+//            the 32 partitions of half w >> 2
+//   down:    512 hidden columns; wave w owns 64 of them
+// Each wave keeps a 128 x 64 accumulator tile (8 x 4 MFMA 16x16 tiles, 128 accumulator
+// registers), which leaves room for two waves per SIMD: a CU's load throughput grows with the
+// number of waves that issue loads (measured: 4 waves pull ~15 B/clk from L2, 8 waves ~30), and
+// at one wave per SIMD every stalled load issue also stalls that SIMD's MFMA stream.
 //
 // Operand traffic:
 //   * expert weights (B operand) go global -> registers, never through LDS.  In the reference
@@ -16,11 +19,12 @@
 //     adjacent columns = 2 or 4 MFMA column tiles at once.  One load instruction reads four
 //     full 128/256-byte row segments; every byte is loaded exactly once per workgroup.
 //   * activations (A operand, rows gathered through token_position_to_id) are staged through a
-//     double-buffered LDS tile of 256 rows x 128 K-bytes, read by all four waves.
+//     three-deep LDS ring of 128 rows x 128 K-bytes, read by all eight waves.
 //   * E8M0 scales ride along: A scales sit in LDS transposed to [g][row%16][row/16] so that one
-//     16-byte read gives a lane the scales of all 16 row tiles (selected with op_sel); B scales
+//     8-byte read gives a lane the scales of all 8 row tiles (selected with op_sel); B scales
 //     are 2-4 bytes per lane per K slice straight from global.
-// The gate/up epilogue exchanges act(gate)*up through LDS so that the MX re-quantisation sees the
+// The gate/up epilogue computes act(gate)*up in registers (a lane holds gate and up of the same
+// element) and exchanges the products through LDS so that the MX re-quantisation sees the
 // reference's blocks (8 partitions x 4 q) and writes K-contiguous rows for the down GEMM.
 //
 // Reference semantics: test/integration/nkilib/core/mlp/test_mlp_common.py:550-682 (layouts,
@@ -31,14 +35,19 @@
 
 namespace moe {
 
-constexpr int MXT = 256;                       // threads
-constexpr int MXM = CHUNK_ROWS;                // 256 rows per workgroup
+constexpr int MXT = 512;                       // threads
+constexpr int MXM = CHUNK_ROWS;                // 128 rows per workgroup
 constexpr int MXROW = 128;                     // LDS pitch of one staged row; 16-byte chunk ch of row r sits in
                                                // slot ch ^ (r & 7), which makes the fragment reads (16 rows x 4
                                                // chunks per instruction) and the staging writes conflict free
-constexpr int MX_SA = MXM * MXROW;             // one A buffer
-constexpr int MX_SS = 4 * 16 * 16;             // one A-scale buffer, [g][c][mt] bytes
-constexpr int MX_LDS = 2 * MX_SA + 2 * MX_SS;  // 67584 bytes of dynamic LDS (the gate/up epilogue needs 65536)
+constexpr int MX_NST = 3;                      // depth of the activation ring
+constexpr int MX_SA = MXM * MXROW;             // one A buffer (16 KB)
+constexpr int MX_SS = 4 * 16 * 8;              // one A-scale buffer, [g][c][mt] bytes
+constexpr int MX_EP = 256 + 8;                 // epilogue exchange: floats per row ([q][64 partitions] + pad)
+constexpr int MX_LDS_LOOP = MX_NST * (MX_SA + MX_SS);
+constexpr int MX_LDS_EPI = 64 * MX_EP * 4;
+constexpr int MX_LDS = MX_LDS_EPI > MX_LDS_LOOP ? MX_LDS_EPI : MX_LDS_LOOP;
+static_assert(MXM == 128, "the kernel is written for 128-row chunks");
 
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -93,7 +102,7 @@ template <int STAGE, int NMT>
 __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
                                              int64_t slot0, int xt) {
   uint8_t* sA = smem;
-  uint8_t* sS = smem + 2 * MX_SA;
+  uint8_t* sS = smem + MX_NST * MX_SA;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -105,17 +114,18 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   int tI = 0, p0 = 0, Pt = 128;
   int64_t h0 = 0;
   if (STAGE == 1) {
-    tI = xt >> 2;
-    p0 = (xt & 3) * 32;
+    tI = xt >> 1;
+    p0 = (xt & 1) * 64 + (w >> 2) * 32;
     const int64_t rows_t = (a.I - (int64_t)tI * 512 < 512) ? (a.I - (int64_t)tI * 512) : 512;
     Pt = (int)(rows_t / 4);
-    if (p0 >= Pt) return;
+    if ((xt & 1) * 64 >= Pt) return;  // whole workgroup: Pt is a multiple of 64 on this path
   } else {
-    h0 = (int64_t)xt * 256;
+    h0 = (int64_t)xt * 512;
   }
+  const int q = w & 3;
 
   // ---- rows: token ids, affinities ---------------------------------------------------------------
-  {
+  if (tid < MXM) {
     int id = -1;
     if (tid < nrows) {
       id = a.tp2id[slot0 + tid];
@@ -132,9 +142,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   }
   __syncthreads();
 
-  // A staging: thread covers rows (tid>>3) + 32 j, 16-byte chunk tid&7
+  // A staging: thread covers rows (tid>>3) + 64 j, 16-byte chunk tid&7
   const int arow0 = tid >> 3, ach = tid & 7;
-  constexpr int NAJ = NMT / 2;  // 32-row groups that hold rows of the NMT tiles
+  constexpr int NAJ = (NMT + 3) / 4;  // 64-row groups that hold rows of the NMT tiles
   // Per-lane 32-bit byte offsets (row * stride + chunk); the K offset is wave-uniform and is added
   // to the scalar base, so a load needs one VGPR of address.  Rows without a token (padding
   // slots, rows past the end of the chunk) read some valid row instead of being zeroed: rows are
@@ -143,7 +153,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   uint32_t a_voff[NAJ];
 #pragma unroll
   for (int j = 0; j < NAJ; ++j) {
-    const int row = arow0 + 32 * j;
+    const int row = arow0 + 64 * j;
     uint32_t r;
     if (STAGE == 1) {
       const int tok = s_tok[row];
@@ -153,13 +163,16 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     }
     a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)(ach * 16);
   }
-  // A scales: thread covers row tid
+  // A scales: waves 0 and 1, thread covers row tid
   uint32_t as_voff;
-  if (STAGE == 1) {
-    const int tok = s_tok[tid];
-    as_voff = ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
-  } else {
-    as_voff = (uint32_t)(slot0 + ((tid < nrows) ? tid : (nrows - 1))) * (uint32_t)a.a_scale_stride;
+  {
+    const int row = tid & (MXM - 1);
+    if (STAGE == 1) {
+      const int tok = s_tok[row];
+      as_voff = ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
+    } else {
+      as_voff = (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1))) * (uint32_t)a.a_scale_stride;
+    }
   }
 
   // ---- K schedule -----------------------------------------------------------------------------------
@@ -187,7 +200,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   if (STAGE == 1) {
     w_pstride = 2 * nH * a.I;
     w_tstride = a.I;
-    colu = (int64_t)tI * 512 + (int64_t)w * Pt + p0;
+    colu = (int64_t)tI * 512 + (int64_t)q * Pt + p0;
     rw = make_rsrc(a.W + (int64_t)e * 128 * w_pstride, (uint32_t)(128 * w_pstride * 4));
     rs = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
     w_voff = (uint32_t)((4 * g * w_pstride + 2 * c) * 4);
@@ -203,19 +216,26 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     s_voff = (uint32_t)(g * w_pstride + 4 * c);
   }
 
-  auto load_b = [&](int ks, BFrag& b) {
+  // Weight loads land in a "raw" register set exactly as the load instructions return them: one
+  // 8/16-byte load gives a lane the same K row of 2 (gate/up) or 4 (down) column tiles, while an
+  // MFMA wants the 8 K rows of one tile in consecutive registers.  The transposition into a BFrag
+  // is 32 register moves, done after the multiply of the previous slice, so that the loads have a
+  // whole slice of MFMA work to complete.
+  struct BRaw {
+    typename std::conditional<STAGE == 1, v2i, v4i>::type d[STAGE == 1 ? 16 : 8];
+    int sc[2];
+  };
+  auto load_b = [&](int ks, BRaw& b) {
     int kt, pb;
     slice_of(ks, kt, pb);
-    if (STAGE == 1) {
+    if constexpr (STAGE == 1) {
 #pragma unroll
       for (int gu = 0; gu < 2; ++gu) {
         const int64_t u0 = (int64_t)(pb * 32) * w_pstride + gu * nH * a.I + (int64_t)kt * w_tstride + colu;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
           const int pr = (r < 4) ? r : (16 + r - 4);
-          const v2i v = __builtin_amdgcn_raw_buffer_load_b64(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
-          b.f[gu * 2 + 0][r] = v[0];
-          b.f[gu * 2 + 1][r] = v[1];
+          b.d[gu * 8 + r] = __builtin_amdgcn_raw_buffer_load_b64(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
         }
       }
       const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu;
@@ -226,16 +246,33 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         const int pr = (r < 4) ? r : (16 + r - 4);
-        const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
-        b.f[0][r] = v[0];
-        b.f[1][r] = v[1];
-        b.f[2][r] = v[2];
-        b.f[3][r] = v[3];
+        b.d[r] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
       }
       const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu;
       b.sc[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, s_voff, uni(us), 0);
       b.sc[1] = 0;
     }
+  };
+  auto unpack_b = [&](const BRaw& b, BFrag& f) {
+    if constexpr (STAGE == 1) {
+#pragma unroll
+      for (int gu = 0; gu < 2; ++gu)
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          f.f[gu * 2 + 0][r] = b.d[gu * 8 + r][0];
+          f.f[gu * 2 + 1][r] = b.d[gu * 8 + r][1];
+        }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        f.f[0][r] = b.d[r][0];
+        f.f[1][r] = b.d[r][1];
+        f.f[2][r] = b.d[r][2];
+        f.f[3][r] = b.d[r][3];
+      }
+    }
+    f.sc[0] = b.sc[0];
+    f.sc[1] = b.sc[1];
   };
 
   // ---- A operand staging ------------------------------------------------------------------------------
@@ -250,18 +287,20 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     slice_of(ks, kt, pb);
 #pragma unroll
     for (int j = 0; j < NAJ; ++j) r.d[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[j], kt * 512 + pb * 128, 0);
-    r.sc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
+    if (w < 2) r.sc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
   };
-  auto store_a = [&](int buf, const AStage& r) {
-    const uint32_t asreg = r.sc;
-    uint8_t* dst = sA + buf * MX_SA;
+  auto store_a = [&](int st, const AStage& r) {
+    uint8_t* dst = sA + st * MX_SA;
 #pragma unroll
-    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
+    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 64 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
     // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
-    uint8_t* sd = sS + buf * MX_SS;
-    const int mt = tid >> 4, cc = tid & 15;
+    if (w < 2) {
+      const uint32_t asreg = r.sc;
+      uint8_t* sd = sS + st * MX_SS;
+      const int mt = tid >> 4, cc = tid & 15;
 #pragma unroll
-    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 16 + mt] = (uint8_t)((asreg >> (8 * gg)) & 0xffu);
+      for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 8 + mt] = (uint8_t)((asreg >> (8 * gg)) & 0xffu);
+    }
   };
 
   v4f acc[NMT][4];
@@ -271,13 +310,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   });
 
   // Row tiles are multiplied in groups of two; the fragments of the next group are read from LDS
-  // while the current group's eight MFMAs run.  The scheduling barriers keep the compiler from
-  // hoisting all sixteen fragment reads to the top (which would not fit the register file).
+  // while the current group's eight MFMAs run.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
-  auto compute = [&](int buf, const BFrag& b) {
-    const uint8_t* plo = sA + buf * MX_SA + rd_lo;
-    const uint8_t* phi = sA + buf * MX_SA + rd_hi;
-    const v4i asc = *(const v4i*)(sS + buf * MX_SS + (g * 16 + c) * 16);
+  auto compute = [&](int st, const BFrag& b) {
+    const uint8_t* plo = sA + st * MX_SA + rd_lo;
+    const uint8_t* phi = sA + st * MX_SA + rd_hi;
+    const v2i asc = *(const v2i*)(sS + st * MX_SS + (g * 16 + c) * 8);
     v8i af[2][2];
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
@@ -320,113 +358,112 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     });
   };
 
-  // ---- main loop: slice ks+1 is in flight (B in registers, A towards LDS) while slice ks multiplies ----
-  // Software pipeline, two K slices deep for both operands: while slice ks multiplies, the loads
-  // of slice ks+2 (A into registers, B into registers) are being issued and those of slice ks+1,
-  // issued a full slice earlier, are stored to LDS (A) / rotated into place (B).  Every load
-  // therefore has at least one whole slice of MFMA work to complete.
-  BFrag bc, b1, b2;
-  AStage a1, a2;
-  load_a(0, a1);
-  load_b(0, bc);
-  store_a(0, a1);
+  // ---- main loop ------------------------------------------------------------------------------------
+  // Slice ks multiplies out of ring stage ks % 3 with the weights in `bc`.  Around it: the
+  // activations of slice ks+2 are loaded into registers before the multiply and stored to ring
+  // stage (ks+2) % 3 after it (that stage was last read in slice ks-1, which every wave left
+  // before the barrier that ended it); the weights of slice ks+1 are loaded before the multiply
+  // and transposed into `bc` after it.  One barrier per slice publishes the stores.
+  BRaw br;
+  AStage as;
+  BFrag bc;
+  load_a(0, as);
+  load_b(0, br);
+  store_a(0, as);
   if (nks > 1) {
-    load_a(1, a1);
-    load_b(1, b1);
+    load_a(1, as);
+    store_a(1, as);
   }
+  unpack_b(br, bc);
   __syncthreads();
+  int st = 0;
 #pragma clang loop unroll(disable)
   for (int ks = 0; ks < nks; ++ks) {
-    if (ks + 2 < nks) {
-      load_a(ks + 2, a2);
-      load_b(ks + 2, b2);
-    }
-    compute(ks & 1, bc);
-    if (ks + 1 < nks) store_a((ks + 1) & 1, a1);
+    if (ks + 2 < nks) load_a(ks + 2, as);
+    if (ks + 1 < nks) load_b(ks + 1, br);
+    compute(st, bc);
+    const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
+    if (ks + 2 < nks) store_a(st2, as);
+    unpack_b(br, bc);
     __syncthreads();
-    bc = b1;
-    b1 = b2;
-    a1 = a2;
+    st = (st == 2) ? 0 : st + 1;
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
-    // Raw gate and up accumulators go through LDS, 64 rows at a time, as [row][p_local 32][q 4] fp32
-    // (gate at E, up 32 KB further); then one thread per MX block (8 partitions x 4 q) applies bias,
-    // clamps and act(gate)*up, quantises and writes 32 K-contiguous bytes plus the scale byte.
+    // act(gate + bias) * (up + bias) in registers, then through LDS, 64 rows at a time, as
+    // [row][q][64 partitions] fp32; then one thread per MX block (8 partitions x 4 q) quantises and
+    // writes 32 K-contiguous bytes plus the scale byte.
     float* E = (float*)smem;
-    const int q = w;
-    static_for<0, NMT / 4>([&](auto ps_) {
+    float bg[2] = {0.f, 0.f}, bu[2] = {0.f, 0.f};
+    if (a.bias) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int64_t p = p0 + 2 * c + t;
+        const int64_t ig = ((((int64_t)e * a.pI + p) * 2 + 0) * a.nI + tI) * 4 + q;
+        const int64_t iu = ((((int64_t)e * a.pI + p) * 2 + 1) * a.nI + tI) * 4 + q;
+        if (a.bias_dtype == MOE_DT_BF16) {
+          bg[t] = bf16_bits_to_f32(((const uint16_t*)a.bias)[ig]);
+          bu[t] = bf16_bits_to_f32(((const uint16_t*)a.bias)[iu]);
+        } else {
+          bg[t] = ((const float*)a.bias)[ig];
+          bu[t] = ((const float*)a.bias)[iu];
+        }
+      }
+    }
+    const int pl0 = (w >> 2) * 32 + 2 * c;  // first of the lane's two partitions within the workgroup's 64
+    constexpr int NPS = (NMT + 3) / 4;
+    static_for<0, NPS>([&](auto ps_) {
       constexpr int ps = decltype(ps_)::value;
       if (ps * 64 < nrows) {
         __syncthreads();
-        static_for<0, 4>([&](auto m_) {
+        static_for<0, (NMT - ps * 4 < 4 ? NMT - ps * 4 : 4)>([&](auto m_) {
           constexpr int ml = decltype(m_)::value;
           constexpr int mt = ps * 4 + ml;
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
+          for (int r = 0; r < 4; ++r) {
+            float y[2];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int rl = ml * 16 + 4 * g + r;
-              E[(rl * 32 + 2 * c + t) * 4 + q] = acc[mt][t][r];
-              E[8192 + (rl * 32 + 2 * c + t) * 4 + q] = acc[mt][2 + t][r];
-            }
-          }
-        });
-        __syncthreads();
-        // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions p0+8j .. p0+8j+7 (x 4 q)
-        const int rl = tid >> 2, j = tid & 3;
-        const int row = ps * 64 + rl;
-        if (row < nrows) {
-          float* sg = E + (rl * 32 + 8 * j) * 4;
-          const float* su = E + 8192 + (rl * 32 + 8 * j) * 4;
-          float am = 0.f;
-#pragma unroll 1
-          for (int k = 0; k < 8; ++k) {
-            const float4 g4 = *(const float4*)(sg + 4 * k), u4 = *(const float4*)(su + 4 * k);
-            float gv[4] = {g4.x, g4.y, g4.z, g4.w};
-            float uv[4] = {u4.x, u4.y, u4.z, u4.w};
-            if (a.bias) {
-              const int64_t p = p0 + 8 * j + k;
-              const int64_t ig = ((((int64_t)e * a.pI + p) * 2 + 0) * a.nI + tI) * 4;
-              const int64_t iu = ((((int64_t)e * a.pI + p) * 2 + 1) * a.nI + tI) * 4;
-#pragma unroll
-              for (int qq = 0; qq < 4; ++qq) {
-                if (a.bias_dtype == MOE_DT_BF16) {
-                  gv[qq] += bf16_bits_to_f32(((const uint16_t*)a.bias)[ig + qq]);
-                  uv[qq] += bf16_bits_to_f32(((const uint16_t*)a.bias)[iu + qq]);
-                } else {
-                  gv[qq] += ((const float*)a.bias)[ig + qq];
-                  uv[qq] += ((const float*)a.bias)[iu + qq];
-                }
-              }
-            }
-            float yv[4];
-#pragma unroll
-            for (int qq = 0; qq < 4; ++qq) {
-              float gg = gv[qq], uu = uv[qq];
+            for (int t = 0; t < 2; ++t) {
+              float gg = acc[mt][t][r] + bg[t], uu = acc[mt][2 + t][r] + bu[t];
               if (a.clamp_mask & MOE_CLAMP_GATE_LO) gg = fmaxf(gg, a.clamp[1]);
               if (a.clamp_mask & MOE_CLAMP_GATE_HI) gg = fminf(gg, a.clamp[0]);
               if (a.clamp_mask & MOE_CLAMP_UP_LO) uu = fmaxf(uu, a.clamp[3]);
               if (a.clamp_mask & MOE_CLAMP_UP_HI) uu = fminf(uu, a.clamp[2]);
-              yv[qq] = act_apply(gg, a.act_fn) * uu;
-              am = fmaxf(am, fabsf(yv[qq]));
+              y[t] = act_apply(gg, a.act_fn) * uu;
             }
-            *(float4*)(sg + 4 * k) = make_float4(yv[0], yv[1], yv[2], yv[3]);  // in place: only this thread reads it
+            const int rl = ml * 16 + 4 * g + r;
+            *(float2*)(E + rl * MX_EP + q * 64 + pl0) = make_float2(y[0], y[1]);
+          }
+        });
+        __syncthreads();
+        // thread (rl = tid/8, j = tid%8): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 64 (x 4 q)
+        const int rl = tid >> 3, j = tid & 7;
+        const int row = ps * 64 + rl;
+        if (row < nrows) {
+          const float* src = E + rl * MX_EP + 8 * j;
+          float yv[4][8];
+          float am = 0.f;
+#pragma unroll
+          for (int qq = 0; qq < 4; ++qq) {
+            const float4 lo = *(const float4*)(src + qq * 64), hi = *(const float4*)(src + qq * 64 + 4);
+            yv[qq][0] = lo.x; yv[qq][1] = lo.y; yv[qq][2] = lo.z; yv[qq][3] = lo.w;
+            yv[qq][4] = hi.x; yv[qq][5] = hi.y; yv[qq][6] = hi.z; yv[qq][7] = hi.w;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) am = fmaxf(am, fabsf(yv[qq][k]));
           }
           const uint32_t sb = mx_scale_byte(am);
           const float is = mx_inv_scale(sb);
           uint32_t d[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) {
-            const float4 y4 = *(const float4*)(sg + 4 * k);
-            d[k] = pack4_e4m3(clip448(y4.x * is), clip448(y4.y * is), clip448(y4.z * is), clip448(y4.w * is));
-          }
+          for (int k = 0; k < 8; ++k)
+            d[k] = pack4_e4m3(clip448(yv[0][k] * is), clip448(yv[1][k] * is), clip448(yv[2][k] * is), clip448(yv[3][k] * is));
           const int64_t slot = slot0 + row;
-          uint4* o = (uint4*)(a.Yq + slot * a.y_stride + tI * 512 + (p0 + 8 * j) * 4);
+          const int pw = (xt & 1) * 64 + 8 * j;  // first partition of the block within the intermediate tile
+          uint4* o = (uint4*)(a.Yq + slot * a.y_stride + tI * 512 + pw * 4);
           o[0] = make_uint4(d[0], d[1], d[2], d[3]);
           o[1] = make_uint4(d[4], d[5], d[6], d[7]);
-          a.Ys[slot * a.ys_stride + tI * 16 + (p0 >> 3) + j] = (uint8_t)sb;
+          a.Ys[slot * a.ys_stride + tI * 16 + (pw >> 3)] = (uint8_t)sb;
         }
       }
     });
@@ -465,7 +502,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 }
 
 template <int STAGE>
-__global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
+__global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(2, 2))) void mx_gemm_kernel(const MxArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_tok[MXM];
   __shared__ float s_aff[MXM];
@@ -485,9 +522,9 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int nrows = __builtin_amdgcn_readfirstlane(a.chunk_rows[chunk]);
   const int e = __builtin_amdgcn_readfirstlane(a.chunk_expert[chunk]);
   const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
-  if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  else if (nrows <= 128) mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  else mx_gemm_body<STAGE, 16>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  if (nrows <= 32) mx_gemm_body<STAGE, 2>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  else if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  else mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
 }
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {
