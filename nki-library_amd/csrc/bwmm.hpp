@@ -65,10 +65,9 @@ struct MxArgs {
   int32_t col_tiles;       // column tiles per chunk (set by the launcher)
 };
 
-// True when the large-tile kernels cover the shape: 512 hidden columns per workgroup in the down
-// stage and, in the gate/up stage, 64 partitions per workgroup out of every intermediate tile
-// (I % 256 == 0); other shapes run the general kernel.
-inline bool mx_fast_path_ok(int64_t H, int64_t I) { return H % 512 == 0 && I % 256 == 0; }
+// True when the large-tile kernels cover the shape: every intermediate tile holds a multiple
+// of 32 partitions (I % 128 == 0); other shapes run the general kernel.
+inline bool mx_fast_path_ok(int64_t H, int64_t I) { return H % 512 == 0 && I % 128 == 0; }
 int launch_mx_gemm(int stage, const MxArgs& m, unsigned gx, unsigned gy, hipStream_t s);
 
 int launch_gemm_stage(int kind, int stage, const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s);

@@ -1,14 +1,14 @@
 // MXFP8 blockwise expert GEMMs for gfx950, large-tile version.
 //
-// A 512-thread workgroup (8 waves, two per SIMD) owns an "expert chunk" of up to 128 consecutive
-// slots of one expert and 512 output columns:
-//   gate/up: 64 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w & 3 and
-//            the 32 partitions of half w >> 2
-//   down:    512 hidden columns; wave w owns 64 of them
+// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 128 consecutive
+// slots of one expert and 256 output columns:
+//   gate/up: 32 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w
+//   down:    256 hidden columns; wave w owns 64 of them
 // Each wave keeps a 128 x 64 accumulator tile (8 x 4 MFMA 16x16 tiles, 128 accumulator
-// registers), which leaves room for two waves per SIMD: a CU's load throughput grows with the
-// number of waves that issue loads (measured: 4 waves pull ~15 B/clk from L2, 8 waves ~30), and
-// at one wave per SIMD every stalled load issue also stalls that SIMD's MFMA stream.
+// registers), which leaves room for two workgroups per CU, i.e. two waves per SIMD that are not
+// tied to each other by a barrier: while one workgroup issues loads, waits for them or runs its
+// epilogue, the other one's MFMAs keep the SIMD busy.  (A CU's load throughput also grows with
+// the number of waves that issue loads: measured ~15 B/clk from L2 with 4 waves, ~30 with 8.)
 //
 // Operand traffic:
 //   * expert weights (B operand) go global -> registers, never through LDS.  In the reference
@@ -19,7 +19,7 @@
 //     adjacent columns = 2 or 4 MFMA column tiles at once.  One load instruction reads four
 //     full 128/256-byte row segments; every byte is loaded exactly once per workgroup.
 //   * activations (A operand, rows gathered through token_position_to_id) are staged through a
-//     three-deep LDS ring of 128 rows x 128 K-bytes, read by all eight waves.
+//     three-deep LDS ring of 128 rows x 128 K-bytes, read by all four waves.
 //   * E8M0 scales ride along: A scales sit in LDS transposed to [g][row%16][row/16] so that one
 //     8-byte read gives a lane the scales of all 8 row tiles (selected with op_sel); B scales
 //     are 2-4 bytes per lane per K slice straight from global.
@@ -35,7 +35,7 @@
 
 namespace moe {
 
-constexpr int MXT = 512;                       // threads
+constexpr int MXT = 256;                       // threads
 constexpr int MXM = CHUNK_ROWS;                // 128 rows per workgroup
 constexpr int MXROW = 128;                     // LDS pitch of one staged row; 16-byte chunk ch of row r sits in
                                                // slot ch ^ (r & 7), which makes the fragment reads (16 rows x 4
@@ -43,7 +43,7 @@ constexpr int MXROW = 128;                     // LDS pitch of one staged row; 1
 constexpr int MX_NST = 3;                      // depth of the activation ring
 constexpr int MX_SA = MXM * MXROW;             // one A buffer (16 KB)
 constexpr int MX_SS = 4 * 16 * 8;              // one A-scale buffer, [g][c][mt] bytes
-constexpr int MX_EP = 256 + 8;                 // epilogue exchange: floats per row ([q][64 partitions] + pad)
+constexpr int MX_EP = 128 + 8;                 // epilogue exchange: floats per row ([q][32 partitions] + pad)
 constexpr int MX_LDS_LOOP = MX_NST * (MX_SA + MX_SS);
 constexpr int MX_LDS_EPI = 64 * MX_EP * 4;
 constexpr int MX_LDS = MX_LDS_EPI > MX_LDS_LOOP ? MX_LDS_EPI : MX_LDS_LOOP;
@@ -114,15 +114,15 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   int tI = 0, p0 = 0, Pt = 128;
   int64_t h0 = 0;
   if (STAGE == 1) {
-    tI = xt >> 1;
-    p0 = (xt & 1) * 64 + (w >> 2) * 32;
+    tI = xt >> 2;
+    p0 = (xt & 3) * 32;
     const int64_t rows_t = (a.I - (int64_t)tI * 512 < 512) ? (a.I - (int64_t)tI * 512) : 512;
     Pt = (int)(rows_t / 4);
-    if ((xt & 1) * 64 >= Pt) return;  // whole workgroup: Pt is a multiple of 64 on this path
+    if (p0 >= Pt) return;  // whole workgroup: Pt is a multiple of 32 on this path
   } else {
-    h0 = (int64_t)xt * 512;
+    h0 = (int64_t)xt * 256;
   }
-  const int q = w & 3;
+  const int q = w;
 
   // ---- rows: token ids, affinities ---------------------------------------------------------------
   if (tid < MXM) {
@@ -142,9 +142,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   }
   __syncthreads();
 
-  // A staging: thread covers rows (tid>>3) + 64 j, 16-byte chunk tid&7
+  // A staging: thread covers rows (tid>>3) + 32 j, 16-byte chunk tid&7
   const int arow0 = tid >> 3, ach = tid & 7;
-  constexpr int NAJ = (NMT + 3) / 4;  // 64-row groups that hold rows of the NMT tiles
+  constexpr int NAJ = NMT / 2;  // 32-row groups that hold rows of the NMT tiles
   // Per-lane 32-bit byte offsets (row * stride + chunk); the K offset is wave-uniform and is added
   // to the scalar base, so a load needs one VGPR of address.  Rows without a token (padding
   // slots, rows past the end of the chunk) read some valid row instead of being zeroed: rows are
@@ -153,7 +153,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   uint32_t a_voff[NAJ];
 #pragma unroll
   for (int j = 0; j < NAJ; ++j) {
-    const int row = arow0 + 64 * j;
+    const int row = arow0 + 32 * j;
     uint32_t r;
     if (STAGE == 1) {
       const int tok = s_tok[row];
@@ -292,7 +292,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   auto store_a = [&](int st, const AStage& r) {
     uint8_t* dst = sA + st * MX_SA;
 #pragma unroll
-    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 64 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
+    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
     // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
     if (w < 2) {
       const uint32_t asreg = r.sc;
@@ -309,52 +309,33 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = (v4f){0.f, 0.f, 0.f, 0.f};
   });
 
-  // Row tiles are multiplied in groups of two; the fragments of the next group are read from LDS
-  // while the current group's eight MFMAs run.
+  // Row tiles are multiplied one at a time; the fragment of the next tile is read from LDS while
+  // the current tile's four MFMAs run.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   auto compute = [&](int st, const BFrag& b) {
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
     const v2i asc = *(const v2i*)(sS + st * MX_SS + (g * 16 + c) * 8);
-    v8i af[2][2];
-    af[0][0] = frag_from_lds(plo, phi);
-    af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
-    static_for<0, NMT / 2>([&](auto gi_) {
-      constexpr int gi = decltype(gi_)::value;
-      constexpr int cur = gi & 1, nxt = cur ^ 1;
-      if constexpr (gi + 1 < NMT / 2) {
-        af[nxt][0] = frag_from_lds(plo + (2 * gi + 2) * 16 * MXROW, phi + (2 * gi + 2) * 16 * MXROW);
-        af[nxt][1] = frag_from_lds(plo + (2 * gi + 3) * 16 * MXROW, phi + (2 * gi + 3) * 16 * MXROW);
-      }
-      // Fixed point between "next group's reads issued" and "this group's MFMAs": the reads above
+    v8i af[2];
+    af[0] = frag_from_lds(plo, phi);
+    static_for<0, NMT>([&](auto mt_) {
+      constexpr int mt = decltype(mt_)::value;
+      constexpr int cur = mt & 1, nxt = cur ^ 1;
+      if constexpr (mt + 1 < NMT) af[nxt] = frag_from_lds(plo + (mt + 1) * 16 * MXROW, phi + (mt + 1) * 16 * MXROW);
+      // Fixed point between "next tile's reads issued" and "this tile's MFMAs": the reads above
       // cannot sink below it (memory clobber) and the MFMAs below cannot rise above it (they use the
-      // fragments it returns), so the two fragment sets stay live together and the LDS latency of
-      // the next group is covered by this group's eight MFMAs.
-      asm volatile("" : "+v"(af[cur][0]), "+v"(af[cur][1]) : : "memory");
-      {
-        constexpr int mt = 2 * gi;
-        const int sa = asc[mt / 4];
-        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][0], b, acc[mt][0], sa);
-        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][0], b, acc[mt][1], sa);
-        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][0], b, acc[mt][2], sa);
-        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][0], b, acc[mt][3], sa);
-      }
-      {
-        constexpr int mt = 2 * gi + 1;
-        const int sa = asc[mt / 4];
-        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][1], b, acc[mt][0], sa);
-        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][1], b, acc[mt][1], sa);
-        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][1], b, acc[mt][2], sa);
-        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][1], b, acc[mt][3], sa);
-      }
-      // Pin the eight results here, in accumulation registers.  Without a fixed point the
-      // compiler sinks the (side-effect free) MFMAs towards the end of the K step and hoists
-      // every fragment read to its top, which does not fit the register file.
-      asm volatile("" : "+a"(acc[2 * gi][0]), "+a"(acc[2 * gi][1]), "+a"(acc[2 * gi][2]), "+a"(acc[2 * gi][3]),
-                        "+a"(acc[2 * gi + 1][0]), "+a"(acc[2 * gi + 1][1]), "+a"(acc[2 * gi + 1][2]),
-                        "+a"(acc[2 * gi + 1][3])
-                   :
-                   : "memory");
+      // fragment it returns), so both fragments stay live together and the LDS latency of the next
+      // tile is covered by this tile's MFMAs.
+      asm volatile("" : "+v"(af[cur]) : : "memory");
+      const int sa = asc[mt / 4];
+      acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur], b, acc[mt][0], sa);
+      acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur], b, acc[mt][1], sa);
+      acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur], b, acc[mt][2], sa);
+      acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur], b, acc[mt][3], sa);
+      // Pin the four results here, in accumulation registers.  Without a fixed point the compiler
+      // sinks the (side-effect free) MFMAs towards the end of the K step and hoists every fragment
+      // read to its top, which does not fit the register file.
+      asm volatile("" : "+a"(acc[mt][0]), "+a"(acc[mt][1]), "+a"(acc[mt][2]), "+a"(acc[mt][3]) : : "memory");
     });
   };
 
@@ -392,7 +373,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
     // act(gate + bias) * (up + bias) in registers, then through LDS, 64 rows at a time, as
-    // [row][q][64 partitions] fp32; then one thread per MX block (8 partitions x 4 q) quantises and
+    // [row][q][32 partitions] fp32; then one thread per MX block (8 partitions x 4 q) quantises and
     // writes 32 K-contiguous bytes plus the scale byte.
     float* E = (float*)smem;
     float bg[2] = {0.f, 0.f}, bu[2] = {0.f, 0.f};
@@ -411,7 +392,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         }
       }
     }
-    const int pl0 = (w >> 2) * 32 + 2 * c;  // first of the lane's two partitions within the workgroup's 64
+    const int pl0 = 2 * c;  // first of the lane's two partitions within the workgroup's 32
     constexpr int NPS = (NMT + 3) / 4;
     static_for<0, NPS>([&](auto ps_) {
       constexpr int ps = decltype(ps_)::value;
@@ -433,12 +414,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
               y[t] = act_apply(gg, a.act_fn) * uu;
             }
             const int rl = ml * 16 + 4 * g + r;
-            *(float2*)(E + rl * MX_EP + q * 64 + pl0) = make_float2(y[0], y[1]);
+            *(float2*)(E + rl * MX_EP + q * 32 + pl0) = make_float2(y[0], y[1]);
           }
         });
         __syncthreads();
-        // thread (rl = tid/8, j = tid%8): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 64 (x 4 q)
-        const int rl = tid >> 3, j = tid & 7;
+        // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 32 (x 4 q)
+        const int rl = tid >> 2, j = tid & 3;
         const int row = ps * 64 + rl;
         if (row < nrows) {
           const float* src = E + rl * MX_EP + 8 * j;
@@ -446,7 +427,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           float am = 0.f;
 #pragma unroll
           for (int qq = 0; qq < 4; ++qq) {
-            const float4 lo = *(const float4*)(src + qq * 64), hi = *(const float4*)(src + qq * 64 + 4);
+            const float4 lo = *(const float4*)(src + qq * 32), hi = *(const float4*)(src + qq * 32 + 4);
             yv[qq][0] = lo.x; yv[qq][1] = lo.y; yv[qq][2] = lo.z; yv[qq][3] = lo.w;
             yv[qq][4] = hi.x; yv[qq][5] = hi.y; yv[qq][6] = hi.z; yv[qq][7] = hi.w;
 #pragma unroll
@@ -459,7 +440,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           for (int k = 0; k < 8; ++k)
             d[k] = pack4_e4m3(clip448(yv[0][k] * is), clip448(yv[1][k] * is), clip448(yv[2][k] * is), clip448(yv[3][k] * is));
           const int64_t slot = slot0 + row;
-          const int pw = (xt & 1) * 64 + 8 * j;  // first partition of the block within the intermediate tile
+          const int pw = p0 + 8 * j;  // first partition of the block within the intermediate tile
           uint4* o = (uint4*)(a.Yq + slot * a.y_stride + tI * 512 + pw * 4);
           o[0] = make_uint4(d[0], d[1], d[2], d[3]);
           o[1] = make_uint4(d[4], d[5], d[6], d[7]);
