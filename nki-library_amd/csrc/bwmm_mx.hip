@@ -1,27 +1,33 @@
 // MXFP8 blockwise expert GEMMs for gfx950, large-tile version.
 //
-// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 128 consecutive
-// slots of one expert and 256 output columns:
+// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 256 consecutive
+// slots of one expert (two 128-token blocks) and 256 output columns:
 //   gate/up: 32 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w
 //   down:    256 hidden columns; wave w owns 64 of them
-// Each wave keeps a 128 x 64 accumulator tile (8 x 4 MFMA 16x16 tiles, 128 accumulator
-// registers), which leaves room for two workgroups per CU, i.e. two waves per SIMD that are not
-// tied to each other by a barrier: while one workgroup issues loads, waits for them or runs its
-// epilogue, the other one's MFMAs keep the SIMD busy.  (A CU's load throughput also grows with
-// the number of waves that issue loads: measured ~15 B/clk from L2 with 4 waves, ~30 with 8.)
+// so every weight byte that enters the CU is used by 256 rows, and both operands enter the CU
+// exactly once per workgroup: the bytes a CU pulls through its L1 per flop are what bounds this
+// kernel (smaller or split tiles were measured: 128-row workgroups double the traffic into the
+// CU and, because sibling workgroups drift apart by more K slices than the L2 holds, the traffic
+// over the fabric as well).  Each wave keeps a 256 x 64 accumulator tile (16 x 4 MFMA 16x16
+// tiles, 256 accumulator registers).
 //
-// Operand traffic:
+// With one wave per SIMD nothing overlaps unless the instruction stream says so:
+//   * the loads of the coming K slices are issued a few at a time between the MFMA groups of slice ks
+//     (a burst of loads blocks the wave at the issue stage for thousands of cycles while the
+//     matrix pipe drains);
 //   * expert weights (B operand) go global -> registers, never through LDS.  In the reference
 //     layout a weight column's K runs over partitions p (4 K-bytes per 4-byte element), and lane
 //     group g of v_mfma_scale_f32_16x16x128_f8f6f4 needs K bytes [16g,16g+16) and [64+16g,
 //     64+16g+16) of the 128-byte K slice, i.e. partitions 4g..4g+3 and 16+4g..16+4g+3 of the 32
 //     partitions of the slice: eight loads per lane, each fetching 2 (gate/up) or 4 (down)
 //     adjacent columns = 2 or 4 MFMA column tiles at once.  One load instruction reads four
-//     full 128/256-byte row segments; every byte is loaded exactly once per workgroup.
+//     full 128/256-byte row segments.  The loads land in a "raw" register set, which is
+//     transposed into MFMA operand order at the top of the slice that uses it;
 //   * activations (A operand, rows gathered through token_position_to_id) are staged through a
-//     three-deep LDS ring of 128 rows x 128 K-bytes, read by all four waves.
+//     three-deep LDS ring of 256 rows x 128 K-bytes, read by all four waves; the fragments of the
+//     next two row tiles are read while the current two multiply;
 //   * E8M0 scales ride along: A scales sit in LDS transposed to [g][row%16][row/16] so that one
-//     8-byte read gives a lane the scales of all 8 row tiles (selected with op_sel); B scales
+//     16-byte read gives a lane the scales of all 16 row tiles (selected with op_sel); B scales
 //     are 2-4 bytes per lane per K slice straight from global.
 // The gate/up epilogue computes act(gate)*up in registers (a lane holds gate and up of the same
 // element) and exchanges the products through LDS so that the MX re-quantisation sees the
@@ -36,18 +42,18 @@
 namespace moe {
 
 constexpr int MXT = 256;                       // threads
-constexpr int MXM = CHUNK_ROWS;                // 128 rows per workgroup
+constexpr int MXM = CHUNK_ROWS;                // 256 rows per workgroup
 constexpr int MXROW = 128;                     // LDS pitch of one staged row; 16-byte chunk ch of row r sits in
                                                // slot ch ^ (r & 7), which makes the fragment reads (16 rows x 4
                                                // chunks per instruction) and the staging writes conflict free
 constexpr int MX_NST = 3;                      // depth of the activation ring
-constexpr int MX_SA = MXM * MXROW;             // one A buffer (16 KB)
-constexpr int MX_SS = 4 * 16 * 8;              // one A-scale buffer, [g][c][mt] bytes
+constexpr int MX_SA = MXM * MXROW;             // one A buffer (32 KB)
+constexpr int MX_SS = 4 * 16 * 16;             // one A-scale buffer, [g][c][mt] bytes
 constexpr int MX_EP = 128 + 8;                 // epilogue exchange: floats per row ([q][32 partitions] + pad)
 constexpr int MX_LDS_LOOP = MX_NST * (MX_SA + MX_SS);
 constexpr int MX_LDS_EPI = 64 * MX_EP * 4;
 constexpr int MX_LDS = MX_LDS_EPI > MX_LDS_LOOP ? MX_LDS_EPI : MX_LDS_LOOP;
-static_assert(MXM == 128, "the kernel is written for 128-row chunks");
+static_assert(MXM == 256, "the kernel is written for 256-row chunks");
 
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -125,7 +131,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   const int q = w;
 
   // ---- rows: token ids, affinities ---------------------------------------------------------------
-  if (tid < MXM) {
+  {
     int id = -1;
     if (tid < nrows) {
       id = a.tp2id[slot0 + tid];
@@ -163,21 +169,19 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     }
     a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)(ach * 16);
   }
-  // A scales: waves 0 and 1, thread covers row tid
+  // A scales: thread covers row tid
   uint32_t as_voff;
-  {
-    const int row = tid & (MXM - 1);
-    if (STAGE == 1) {
-      const int tok = s_tok[row];
-      as_voff = ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
-    } else {
-      as_voff = (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1))) * (uint32_t)a.a_scale_stride;
-    }
+  if (STAGE == 1) {
+    const int tok = s_tok[tid];
+    as_voff = ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
+  } else {
+    as_voff = (uint32_t)(slot0 + ((tid < nrows) ? tid : (nrows - 1))) * (uint32_t)a.a_scale_stride;
   }
 
   // ---- K schedule -----------------------------------------------------------------------------------
   // stage 1: ks -> (H tile ks>>2, partition group ks&3), all slices full.
-  // stage 2: slices of intermediate tile t are the first Pt(t)/32 partition groups.
+  // stage 2: slices of intermediate tile t are the first Pt(t)/32 partition groups; only the last
+  // tile can be short and its slices come last, so ks -> (ks>>2, ks&3) holds for both.
   int nks;
   if (STAGE == 1) {
     nks = (int)(a.H / 128);
@@ -185,74 +189,92 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     const int64_t tail = a.I % 512;
     nks = (int)((a.I / 512) * 4 + (tail / 128));
   }
-  auto slice_of = [&](int ks, int& kt, int& pb) {
-    kt = ks >> 2;
-    pb = ks & 3;  // valid for both stages: only the last tile can be short and its slices come last
-  };
 
   // ---- B operand addressing ---------------------------------------------------------------------------
   // byte address inside the expert's weights = uniform part (gate/up, K tile, partition
   // 32*pb + {r | 16 + r}, first column of the wave) + per-lane part (partition 4g, lane's columns).
   int64_t w_pstride, w_tstride;  // element strides (4-byte weights; scales use the same counts in bytes)
-  __amdgpu_buffer_rsrc_t rw, rs;
+  __amdgpu_buffer_rsrc_t rw_, rs_;
   uint32_t w_voff, s_voff;
   int64_t colu;
   if (STAGE == 1) {
     w_pstride = 2 * nH * a.I;
     w_tstride = a.I;
     colu = (int64_t)tI * 512 + (int64_t)q * Pt + p0;
-    rw = make_rsrc(a.W + (int64_t)e * 128 * w_pstride, (uint32_t)(128 * w_pstride * 4));
-    rs = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
+    rw_ = make_rsrc(a.W + (int64_t)e * 128 * w_pstride, (uint32_t)(128 * w_pstride * 4));
+    rs_ = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
     w_voff = (uint32_t)((4 * g * w_pstride + 2 * c) * 4);
     s_voff = (uint32_t)(g * w_pstride + 2 * c);
   } else {
     w_pstride = (int64_t)a.nI * a.H;
     w_tstride = a.H;
-    colu = h0 + 64 * w;
+    colu = h0 + 64 * q;
     const int64_t sp = (a.pI + 7) / 8;
-    rw = make_rsrc(a.W + (int64_t)e * a.pI * w_pstride, (uint32_t)(a.pI * w_pstride * 4));
-    rs = make_rsrc(a.W_scale + (int64_t)e * sp * w_pstride, (uint32_t)(sp * w_pstride));
+    rw_ = make_rsrc(a.W + (int64_t)e * a.pI * w_pstride, (uint32_t)(a.pI * w_pstride * 4));
+    rs_ = make_rsrc(a.W_scale + (int64_t)e * sp * w_pstride, (uint32_t)(sp * w_pstride));
     w_voff = (uint32_t)((4 * g * w_pstride + 4 * c) * 4);
     s_voff = (uint32_t)(g * w_pstride + 4 * c);
   }
 
-  // Weight loads land in a "raw" register set exactly as the load instructions return them: one
-  // 8/16-byte load gives a lane the same K row of 2 (gate/up) or 4 (down) column tiles, while an
-  // MFMA wants the 8 K rows of one tile in consecutive registers.  The transposition into a BFrag
-  // is 32 register moves, done after the multiply of the previous slice, so that the loads have a
-  // whole slice of MFMA work to complete.
+  // A K slice's loads, numbered so that they can be issued a few at a time:
+  //   0 .. NAJ-1            activation rows (16 bytes per lane each)
+  //   NAJ                   activation scales
+  //   NAJ+1 .. NAJ+NBL      weights
+  //   NAJ+NBL+1 ..          weight scales
+  constexpr int NBL = (STAGE == 1) ? 16 : 8;
+  constexpr int NBS = (STAGE == 1) ? 2 : 1;
+  constexpr int NLOADS = NAJ + 1 + NBL + NBS;
   struct BRaw {
-    typename std::conditional<STAGE == 1, v2i, v4i>::type d[STAGE == 1 ? 16 : 8];
+    typename std::conditional<STAGE == 1, v2i, v4i>::type d[NBL];
     int sc[2];
   };
-  auto load_b = [&](int ks, BRaw& b) {
-    int kt, pb;
-    slice_of(ks, kt, pb);
-    if constexpr (STAGE == 1) {
-#pragma unroll
-      for (int gu = 0; gu < 2; ++gu) {
-        const int64_t u0 = (int64_t)(pb * 32) * w_pstride + gu * nH * a.I + (int64_t)kt * w_tstride + colu;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          const int pr = (r < 4) ? r : (16 + r - 4);
-          b.d[gu * 8 + r] = __builtin_amdgcn_raw_buffer_load_b64(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
-        }
-      }
-      const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu;
-      b.sc[0] = (int)__builtin_amdgcn_raw_buffer_load_b16(rs, s_voff, uni(us), 0);
-      b.sc[1] = (int)__builtin_amdgcn_raw_buffer_load_b16(rs, s_voff, uni(us + nH * a.I), 0);
+  struct AStage {
+    v4i d[NAJ];
+    uint32_t sc;
+  };
+  const __amdgpu_buffer_rsrc_t ra_ = make_rsrc(a.A, 0xffffffffu);
+  const __amdgpu_buffer_rsrc_t ras_ = make_rsrc(a.A_scale, 0xffffffffu);
+  // Loads of a slice past the end go through descriptors of zero records: such a load is out of
+  // range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads.
+  const __amdgpu_buffer_rsrc_t ra0 = make_rsrc(a.A, 0u), ras0 = make_rsrc(a.A_scale, 0u);
+  const __amdgpu_buffer_rsrc_t rw0 = make_rsrc(a.W, 0u), rs0 = make_rsrc(a.W_scale, 0u);
+  auto issue_load = [&](auto idx_, int ks, AStage& as, BRaw& b) {
+    constexpr int idx = decltype(idx_)::value;
+    const bool live = ks < nks;
+    const __amdgpu_buffer_rsrc_t ra = live ? ra_ : ra0, ras = live ? ras_ : ras0, rw = live ? rw_ : rw0, rs = live ? rs_ : rs0;
+    const int kt = ks >> 2, pb = ks & 3;
+    if constexpr (idx < NAJ) {
+      as.d[idx] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[idx], kt * 512 + pb * 128, 0);
+    } else if constexpr (idx == NAJ) {
+      as.sc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
+    } else if constexpr (idx < NAJ + 1 + NBL) {
+      constexpr int i = idx - NAJ - 1;
+      constexpr int r = i % 8, gu = i / 8;  // gu is 0 in the down stage
+      constexpr int pr = (r < 4) ? r : (16 + r - 4);
+      const int64_t u0 = (int64_t)(pb * 32) * w_pstride + (int64_t)gu * nH * a.I + (int64_t)kt * w_tstride + colu;
+      if constexpr (STAGE == 1)
+        b.d[i] = __builtin_amdgcn_raw_buffer_load_b64(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
+      else
+        b.d[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
     } else {
-      const int64_t u0 = (int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride + colu;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const int pr = (r < 4) ? r : (16 + r - 4);
-        b.d[r] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
-      }
-      const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu;
-      b.sc[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, s_voff, uni(us), 0);
-      b.sc[1] = 0;
+      constexpr int i = idx - NAJ - 1 - NBL;
+      const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu + (int64_t)i * nH * a.I;
+      if constexpr (STAGE == 1)
+        b.sc[i] = (int)__builtin_amdgcn_raw_buffer_load_b16(rs, s_voff, uni(us), 0);
+      else
+        b.sc[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, s_voff, uni(us), 0);
     }
   };
+  constexpr int NLA = NAJ + 1;  // activation loads come first in the numbering
+  auto issue_a = [&](int ks, AStage& as, BRaw& b) {
+    static_for<0, NLA>([&](auto i_) { issue_load(i_, ks, as, b); });
+  };
+  auto issue_b = [&](int ks, AStage& as, BRaw& b) {
+    static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, ks, as, b); });
+  };
+  // Transposition of a raw set into MFMA operand order: one 8/16-byte load gives a lane the same
+  // K row of 2 (gate/up) or 4 (down) column tiles, while an MFMA wants the 8 K rows of one tile
+  // in consecutive registers.
   auto unpack_b = [&](const BRaw& b, BFrag& f) {
     if constexpr (STAGE == 1) {
 #pragma unroll
@@ -262,6 +284,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           f.f[gu * 2 + 0][r] = b.d[gu * 8 + r][0];
           f.f[gu * 2 + 1][r] = b.d[gu * 8 + r][1];
         }
+      f.sc[0] = b.sc[0];
+      f.sc[1] = b.sc[1];
     } else {
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
@@ -270,37 +294,20 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         f.f[2][r] = b.d[r][2];
         f.f[3][r] = b.d[r][3];
       }
+      f.sc[0] = b.sc[0];
+      f.sc[1] = 0;
     }
-    f.sc[0] = b.sc[0];
-    f.sc[1] = b.sc[1];
-  };
-
-  // ---- A operand staging ------------------------------------------------------------------------------
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(a.A, 0xffffffffu);
-  const __amdgpu_buffer_rsrc_t ras = make_rsrc(a.A_scale, 0xffffffffu);
-  struct AStage {
-    v4i d[NAJ];
-    uint32_t sc;
-  };
-  auto load_a = [&](int ks, AStage& r) {
-    int kt, pb;
-    slice_of(ks, kt, pb);
-#pragma unroll
-    for (int j = 0; j < NAJ; ++j) r.d[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[j], kt * 512 + pb * 128, 0);
-    if (w < 2) r.sc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
   };
   auto store_a = [&](int st, const AStage& r) {
+    const uint32_t asreg = r.sc;
     uint8_t* dst = sA + st * MX_SA;
 #pragma unroll
     for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
     // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
-    if (w < 2) {
-      const uint32_t asreg = r.sc;
-      uint8_t* sd = sS + st * MX_SS;
-      const int mt = tid >> 4, cc = tid & 15;
+    uint8_t* sd = sS + st * MX_SS;
+    const int mt = tid >> 4, cc = tid & 15;
 #pragma unroll
-      for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 8 + mt] = (uint8_t)((asreg >> (8 * gg)) & 0xffu);
-    }
+    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 16 + mt] = (uint8_t)((asreg >> (8 * gg)) & 0xffu);
   };
 
   v4f acc[NMT][4];
@@ -309,63 +316,100 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = (v4f){0.f, 0.f, 0.f, 0.f};
   });
 
-  // Row tiles are multiplied one at a time; the fragment of the next tile is read from LDS while
-  // the current tile's four MFMAs run.
+  // One K slice: row tiles are multiplied in groups of two; the fragments of the next group are
+  // read from LDS while the current group's eight MFMAs run.  The groups of the first half are each
+  // followed by a share of the weight loads of slice ks+1 (if LB) and then of the activation loads
+  // of slice ks+2 (if LA).
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
-  auto compute = [&](int st, const BFrag& b) {
+  constexpr int NG = NMT / 2;
+  auto compute = [&](auto lb_, auto la_, int st, const BFrag& b, int ks, AStage& as, BRaw& braw) {
+    constexpr bool LB = decltype(lb_)::value, LA = decltype(la_)::value;
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
-    const v2i asc = *(const v2i*)(sS + st * MX_SS + (g * 16 + c) * 8);
-    v8i af[2];
-    af[0] = frag_from_lds(plo, phi);
-    static_for<0, NMT>([&](auto mt_) {
-      constexpr int mt = decltype(mt_)::value;
-      constexpr int cur = mt & 1, nxt = cur ^ 1;
-      if constexpr (mt + 1 < NMT) af[nxt] = frag_from_lds(plo + (mt + 1) * 16 * MXROW, phi + (mt + 1) * 16 * MXROW);
-      // Fixed point between "next tile's reads issued" and "this tile's MFMAs": the reads above
+    const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
+    v8i af[2][2];
+    af[0][0] = frag_from_lds(plo, phi);
+    af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
+    static_for<0, NG>([&](auto gi_) {
+      constexpr int gi = decltype(gi_)::value;
+      constexpr int cur = gi & 1, nxt = cur ^ 1;
+      if constexpr (gi + 1 < NG) {
+        af[nxt][0] = frag_from_lds(plo + (2 * gi + 2) * 16 * MXROW, phi + (2 * gi + 2) * 16 * MXROW);
+        af[nxt][1] = frag_from_lds(plo + (2 * gi + 3) * 16 * MXROW, phi + (2 * gi + 3) * 16 * MXROW);
+      }
+      // Fixed point between "next group's reads issued" and "this group's MFMAs": the reads above
       // cannot sink below it (memory clobber) and the MFMAs below cannot rise above it (they use the
-      // fragment it returns), so both fragments stay live together and the LDS latency of the next
-      // tile is covered by this tile's MFMAs.
-      asm volatile("" : "+v"(af[cur]) : : "memory");
-      const int sa = asc[mt / 4];
-      acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur], b, acc[mt][0], sa);
-      acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur], b, acc[mt][1], sa);
-      acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur], b, acc[mt][2], sa);
-      acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur], b, acc[mt][3], sa);
-      // Pin the four results here, in accumulation registers.  Without a fixed point the compiler
-      // sinks the (side-effect free) MFMAs towards the end of the K step and hoists every fragment
-      // read to its top, which does not fit the register file.
-      asm volatile("" : "+a"(acc[mt][0]), "+a"(acc[mt][1]), "+a"(acc[mt][2]), "+a"(acc[mt][3]) : : "memory");
+      // fragments it returns), so the two fragment sets stay live together and the LDS latency of
+      // the next group is covered by this group's eight MFMAs.
+      asm volatile("" : "+v"(af[cur][0]), "+v"(af[cur][1]) : : "memory");
+      {
+        constexpr int mt = 2 * gi;
+        const int sa = asc[mt / 4];
+        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][0], b, acc[mt][0], sa);
+        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][0], b, acc[mt][1], sa);
+        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][0], b, acc[mt][2], sa);
+        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][0], b, acc[mt][3], sa);
+      }
+      {
+        constexpr int mt = 2 * gi + 1;
+        const int sa = asc[mt / 4];
+        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][1], b, acc[mt][0], sa);
+        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][1], b, acc[mt][1], sa);
+        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][1], b, acc[mt][2], sa);
+        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][1], b, acc[mt][3], sa);
+      }
+      // Pin the eight results here, in accumulation registers.  Without a fixed point the
+      // compiler sinks the (side-effect free) MFMAs towards the end of the K step and hoists
+      // every fragment read to its top, which does not fit the register file.  The memory clobber
+      // also keeps this group's share of the loads behind the MFMAs.
+      asm volatile("" : "+a"(acc[2 * gi][0]), "+a"(acc[2 * gi][1]), "+a"(acc[2 * gi][2]), "+a"(acc[2 * gi][3]),
+                        "+a"(acc[2 * gi + 1][0]), "+a"(acc[2 * gi + 1][1]), "+a"(acc[2 * gi + 1][2]),
+                        "+a"(acc[2 * gi + 1][3])
+                   :
+                   : "memory");
+      // Loads are spread over the first NGL groups, weights (the longer latency) first; the rest of
+      // the slice is the time they have to arrive before the end of the slice needs them.
+      constexpr int NGL = (NG + 1) / 2;
+      if constexpr (gi < NGL) {
+        constexpr int lo = gi * NLOADS / NGL, hi = (gi + 1) * NLOADS / NGL;
+        static_for<lo, hi>([&](auto i_) {
+          constexpr int i = decltype(i_)::value;
+          constexpr int nb = NLOADS - NLA;
+          if constexpr (i < nb) {
+            if constexpr (LB) issue_load(std::integral_constant<int, NLA + i>{}, ks + 1, as, braw);
+          } else {
+            if constexpr (LA) issue_load(std::integral_constant<int, i - nb>{}, ks + 2, as, braw);
+          }
+        });
+      }
     });
   };
 
   // ---- main loop ------------------------------------------------------------------------------------
-  // Slice ks multiplies out of ring stage ks % 3 with the weights in `bc`.  Around it: the
-  // activations of slice ks+2 are loaded into registers before the multiply and stored to ring
-  // stage (ks+2) % 3 after it (that stage was last read in slice ks-1, which every wave left
-  // before the barrier that ended it); the weights of slice ks+1 are loaded before the multiply
-  // and transposed into `bc` after it.  One barrier per slice publishes the stores.
+  // Slice ks multiplies out of ring stage ks % 3 with the weights in `bc`, transposed at its top
+  // from the raw set.  During its first half the weight loads of slice ks+1 refill the raw set
+  // and the activation loads of slice ks+2 fill the staging registers, which go to ring stage
+  // (ks+2) % 3 at the end of the slice (that stage was last read in slice ks-1,
+  // which every wave left before the barrier that ended it).  One barrier per slice publishes the
+  // stores.
   BRaw br;
   AStage as;
   BFrag bc;
-  load_a(0, as);
-  load_b(0, br);
+  issue_a(0, as, br);
+  issue_b(0, as, br);
   store_a(0, as);
   if (nks > 1) {
-    load_a(1, as);
+    issue_a(1, as, br);
     store_a(1, as);
   }
-  unpack_b(br, bc);
   __syncthreads();
   int st = 0;
 #pragma clang loop unroll(disable)
   for (int ks = 0; ks < nks; ++ks) {
-    if (ks + 2 < nks) load_a(ks + 2, as);
-    if (ks + 1 < nks) load_b(ks + 1, br);
-    compute(st, bc);
-    const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
-    if (ks + 2 < nks) store_a(st2, as);
     unpack_b(br, bc);
+    compute(std::true_type{}, std::true_type{}, st, bc, ks, as, br);
+    const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
+    store_a(st2, as);  // past the end: zeros into a stage that nobody reads any more
     __syncthreads();
     st = (st == 2) ? 0 : st + 1;
   }
@@ -393,12 +437,22 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       }
     }
     const int pl0 = 2 * c;  // first of the lane's two partitions within the workgroup's 32
-    constexpr int NPS = (NMT + 3) / 4;
+    constexpr int NPS = NMT / 4;
+    // Clamps as unconditional min/max against +-inf, and the activation kind as a compile-time
+    // constant of the pass: a lane evaluates 128 elements here, and per-element decisions made this
+    // code longer (and slower) than the K loop.
+    const float inf = __builtin_inff();
+    const float g_lo = (a.clamp_mask & MOE_CLAMP_GATE_LO) ? a.clamp[1] : -inf;
+    const float g_hi = (a.clamp_mask & MOE_CLAMP_GATE_HI) ? a.clamp[0] : inf;
+    const float u_lo = (a.clamp_mask & MOE_CLAMP_UP_LO) ? a.clamp[3] : -inf;
+    const float u_hi = (a.clamp_mask & MOE_CLAMP_UP_HI) ? a.clamp[2] : inf;
+    auto passes = [&](auto act_) {
+    constexpr int ACT = decltype(act_)::value;
     static_for<0, NPS>([&](auto ps_) {
       constexpr int ps = decltype(ps_)::value;
       if (ps * 64 < nrows) {
         __syncthreads();
-        static_for<0, (NMT - ps * 4 < 4 ? NMT - ps * 4 : 4)>([&](auto m_) {
+        static_for<0, 4>([&](auto m_) {
           constexpr int ml = decltype(m_)::value;
           constexpr int mt = ps * 4 + ml;
 #pragma unroll
@@ -406,12 +460,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
             float y[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-              float gg = acc[mt][t][r] + bg[t], uu = acc[mt][2 + t][r] + bu[t];
-              if (a.clamp_mask & MOE_CLAMP_GATE_LO) gg = fmaxf(gg, a.clamp[1]);
-              if (a.clamp_mask & MOE_CLAMP_GATE_HI) gg = fminf(gg, a.clamp[0]);
-              if (a.clamp_mask & MOE_CLAMP_UP_LO) uu = fmaxf(uu, a.clamp[3]);
-              if (a.clamp_mask & MOE_CLAMP_UP_HI) uu = fminf(uu, a.clamp[2]);
-              y[t] = act_apply(gg, a.act_fn) * uu;
+              const float gg = fminf(fmaxf(acc[mt][t][r] + bg[t], g_lo), g_hi);
+              const float uu = fminf(fmaxf(acc[mt][2 + t][r] + bu[t], u_lo), u_hi);
+              y[t] = act_apply(gg, ACT) * uu;
             }
             const int rl = ml * 16 + 4 * g + r;
             *(float2*)(E + rl * MX_EP + q * 32 + pl0) = make_float2(y[0], y[1]);
@@ -448,8 +499,15 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         }
       }
     });
+    };
+    switch (a.act_fn) {
+      case MOE_ACT_SILU: passes(std::integral_constant<int, MOE_ACT_SILU>{}); break;
+      case MOE_ACT_GELU: passes(std::integral_constant<int, MOE_ACT_GELU>{}); break;
+      case MOE_ACT_GELU_TANH: passes(std::integral_constant<int, MOE_ACT_GELU_TANH>{}); break;
+      default: passes(std::integral_constant<int, MOE_ACT_SWISH>{}); break;
+    }
   } else {
-    const int64_t col0 = h0 + 64 * w + 4 * c;
+    const int64_t col0 = h0 + 64 * q + 4 * c;
     float bd[4] = {0.f, 0.f, 0.f, 0.f};
     if (a.bias) {
 #pragma unroll
@@ -483,7 +541,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 }
 
 template <int STAGE>
-__global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(2, 2))) void mx_gemm_kernel(const MxArgs a) {
+__global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_tok[MXM];
   __shared__ float s_aff[MXM];
@@ -503,9 +561,9 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int nrows = __builtin_amdgcn_readfirstlane(a.chunk_rows[chunk]);
   const int e = __builtin_amdgcn_readfirstlane(a.chunk_expert[chunk]);
   const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
-  if (nrows <= 32) mx_gemm_body<STAGE, 2>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  else if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  else mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  else if (nrows <= 128) mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  else mx_gemm_body<STAGE, 16>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
 }
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {

@@ -23,7 +23,7 @@ struct Bookkeeping {
   int64_t max_chunks;
 };
 
-constexpr int CHUNK_ROWS = 128;
+constexpr int CHUNK_ROWS = 256;
 inline int64_t max_chunks_for(int64_t N, int64_t B) { return N * ((B + CHUNK_ROWS - 1) / CHUNK_ROWS); }
 
 size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B);

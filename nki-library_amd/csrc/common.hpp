@@ -115,10 +115,17 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 }
 
 // ---- activation functions (ActFnType, common_types.py:32-36) ---------------------------
+// x * sigmoid(k x) with the hardware exp2 and reciprocal (about 1 ulp each): the library expf and
+// the IEEE division cost ~100 instructions per element, which made the gate/up epilogue as long
+// as half its K loop.  Saturates correctly: exp2 -> inf gives x * 0, exp2 -> 0 gives x.
+__device__ __forceinline__ float x_sigmoid(float x, float k) {
+  const float e = __builtin_amdgcn_exp2f(x * (-1.44269504088896340736f * k));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
 __device__ __forceinline__ float act_apply(float x, int kind) {
   switch (kind) {
     case MOE_ACT_SILU:
-      return x / (1.0f + expf(-x));
+      return x_sigmoid(x, 1.0f);
     case MOE_ACT_GELU:
       return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
     case MOE_ACT_GELU_TANH: {
@@ -126,7 +133,7 @@ __device__ __forceinline__ float act_apply(float x, int kind) {
       return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
     }
     default:  // MOE_ACT_SWISH: x * sigmoid(1.702 x)
-      return x / (1.0f + expf(-1.702f * x));
+      return x_sigmoid(x, 1.702f);
   }
 }
 
