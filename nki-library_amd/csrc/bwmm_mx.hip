@@ -21,8 +21,9 @@
 //     64+16g+16) of the 128-byte K slice, i.e. partitions 4g..4g+3 and 16+4g..16+4g+3 of the 32
 //     partitions of the slice: eight loads per lane, each fetching 2 (gate/up) or 4 (down)
 //     adjacent columns = 2 or 4 MFMA column tiles at once.  One load instruction reads four
-//     full 128/256-byte row segments.  The loads land in a "raw" register set, which is
-//     transposed into MFMA operand order at the top of the slice that uses it;
+//     full 128/256-byte row segments.  The loads land in one of two "raw" register sets, two
+//     slices ahead; a set is transposed into MFMA operand order at the top of the slice that uses
+//     it;
 //   * activations (A operand, rows gathered through token_position_to_id) are staged through a
 //     three-deep LDS ring of 256 rows x 128 K-bytes, read by all four waves; the fragments of the
 //     next two row tiles are read while the current two multiply;
@@ -39,6 +40,9 @@
 
 #include "bwmm.hpp"
 
+#ifndef MX_DBG_WAIT0
+#define MX_DBG_WAIT0 0
+#endif
 namespace moe {
 
 constexpr int MXT = 256;                       // threads
@@ -95,11 +99,59 @@ __device__ __forceinline__ v4f mfma_tile(const v8i& af, const BFrag& b, const v4
 // every load in a loop that checks whether all lanes agree on the descriptor.)
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ int uni(int64_t v) { return __builtin_amdgcn_readfirstlane((int)v); }
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+__device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
   const uint64_t addr = (uint64_t)p;
-  const uint32_t lo = (uint32_t)uni((int)(uint32_t)addr), hi = (uint32_t)uni((int)(uint32_t)(addr >> 32));
-  void* q = (void*)(((uint64_t)hi << 32) | lo);
-  return __builtin_amdgcn_make_buffer_rsrc(q, 0, uni((int)bytes), 0x00020000);
+  v4i d;
+  d[0] = uni((int)(uint32_t)addr);
+  d[1] = uni((int)(uint32_t)(addr >> 32)) & 0xffff;  // stride 0: raw buffer
+  d[2] = uni((int)bytes);
+  d[3] = 0x00020000;
+  return d;
+}
+// The K loop's loads are written as instructions, not builtins: the compiler orders the results of
+// its own loads with a counter that completes in order, and places those waits as if every load it
+// can see on any path had just been issued -- which with two alternating weight sets means waiting
+// for the set that was only just requested.  Loads the compiler cannot see get no waits from it;
+// the waits are placed by hand where the data is first used (vm_wait).  The destination is an
+// in/out operand so that the load updates the variable's register in place.
+__device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+__device__ __forceinline__ void ld_b64(v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+// One load into d1 if sel != 0, else into d0.  The choice is made inside the statement, so the
+// compiler sees straight-line code that updates both variables in place (a branch of its own would
+// end in copies of registers whose loads are still in flight).
+__device__ __forceinline__ void ld2_b128(v4i& d0, v4i& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile(
+      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dwordx4 %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
+      ".Lmx%=_1:\n\tbuffer_load_dwordx4 %1, %2, %3, %4 offen\n.Lmx%=_2:"
+      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
+}
+__device__ __forceinline__ void ld2_b64(v2i& d0, v2i& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile(
+      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dwordx2 %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
+      ".Lmx%=_1:\n\tbuffer_load_dwordx2 %1, %2, %3, %4 offen\n.Lmx%=_2:"
+      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
+}
+__device__ __forceinline__ void ld2_b32(int& d0, int& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile(
+      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dword %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
+      ".Lmx%=_1:\n\tbuffer_load_dword %1, %2, %3, %4 offen\n.Lmx%=_2:"
+      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
+}
+__device__ __forceinline__ void ld2_u16(int& d0, int& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile(
+      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_ushort %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
+      ".Lmx%=_1:\n\tbuffer_load_ushort %1, %2, %3, %4 offen\n.Lmx%=_2:"
+      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
+}
+__device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+__device__ __forceinline__ void ld_u16(int& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 // NMT = number of 16-row tiles this instantiation multiplies (the chunk has at most NMT*16 rows).
@@ -194,7 +246,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // byte address inside the expert's weights = uniform part (gate/up, K tile, partition
   // 32*pb + {r | 16 + r}, first column of the wave) + per-lane part (partition 4g, lane's columns).
   int64_t w_pstride, w_tstride;  // element strides (4-byte weights; scales use the same counts in bytes)
-  __amdgpu_buffer_rsrc_t rw_, rs_;
+  v4i rw_, rs_;
   uint32_t w_voff, s_voff;
   int64_t colu;
   if (STAGE == 1) {
@@ -230,47 +282,70 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   };
   struct AStage {
     v4i d[NAJ];
-    uint32_t sc;
+    int sc;
   };
-  const __amdgpu_buffer_rsrc_t ra_ = make_rsrc(a.A, 0xffffffffu);
-  const __amdgpu_buffer_rsrc_t ras_ = make_rsrc(a.A_scale, 0xffffffffu);
+  const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, 0xffffffffu);
   // Loads of a slice past the end go through descriptors of zero records: such a load is out of
   // range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads.
-  const __amdgpu_buffer_rsrc_t ra0 = make_rsrc(a.A, 0u), ras0 = make_rsrc(a.A_scale, 0u);
-  const __amdgpu_buffer_rsrc_t rw0 = make_rsrc(a.W, 0u), rs0 = make_rsrc(a.W_scale, 0u);
-  auto issue_load = [&](auto idx_, int ks, AStage& as, BRaw& b) {
+  auto desc = [&](const v4i& d, int ks) {
+    v4i r;
+    r[0] = uni(d[0]);
+    r[1] = uni(d[1]);
+    r[2] = uni((ks < nks) ? d[2] : 0);
+    r[3] = uni(d[3]);
+    return r;
+  };
+  auto issue_load = [&](auto idx_, int ks, AStage& as, BRaw& b, BRaw& b1, int sel) {
     constexpr int idx = decltype(idx_)::value;
-    const bool live = ks < nks;
-    const __amdgpu_buffer_rsrc_t ra = live ? ra_ : ra0, ras = live ? ras_ : ras0, rw = live ? rw_ : rw0, rs = live ? rs_ : rs0;
     const int kt = ks >> 2, pb = ks & 3;
     if constexpr (idx < NAJ) {
-      as.d[idx] = __builtin_amdgcn_raw_buffer_load_b128(ra, a_voff[idx], kt * 512 + pb * 128, 0);
+      ld_b128(as.d[idx], a_voff[idx], desc(ra_, ks), kt * 512 + pb * 128);
     } else if constexpr (idx == NAJ) {
-      as.sc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, kt * 16 + pb * 4, 0);
+      ld_b32(as.sc, as_voff, desc(ras_, ks), kt * 16 + pb * 4);
     } else if constexpr (idx < NAJ + 1 + NBL) {
       constexpr int i = idx - NAJ - 1;
       constexpr int r = i % 8, gu = i / 8;  // gu is 0 in the down stage
       constexpr int pr = (r < 4) ? r : (16 + r - 4);
       const int64_t u0 = (int64_t)(pb * 32) * w_pstride + (int64_t)gu * nH * a.I + (int64_t)kt * w_tstride + colu;
       if constexpr (STAGE == 1)
-        b.d[i] = __builtin_amdgcn_raw_buffer_load_b64(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
+        ld2_b64(b.d[i], b1.d[i], sel, w_voff, desc(rw_, ks), uni((u0 + pr * w_pstride) * 4));
       else
-        b.d[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, uni((u0 + pr * w_pstride) * 4), 0);
+        ld2_b128(b.d[i], b1.d[i], sel, w_voff, desc(rw_, ks), uni((u0 + pr * w_pstride) * 4));
     } else {
       constexpr int i = idx - NAJ - 1 - NBL;
       const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu + (int64_t)i * nH * a.I;
       if constexpr (STAGE == 1)
-        b.sc[i] = (int)__builtin_amdgcn_raw_buffer_load_b16(rs, s_voff, uni(us), 0);
+        ld2_u16(b.sc[i], b1.sc[i], sel, s_voff, desc(rs_, ks), uni(us));
       else
-        b.sc[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, s_voff, uni(us), 0);
+        ld2_b32(b.sc[0], b1.sc[0], sel, s_voff, desc(rs_, ks), uni(us));
     }
   };
-  constexpr int NLA = NAJ + 1;  // activation loads come first in the numbering
-  auto issue_a = [&](int ks, AStage& as, BRaw& b) {
-    static_for<0, NLA>([&](auto i_) { issue_load(i_, ks, as, b); });
+  constexpr int NLA = NAJ + 1;        // activation loads come first in the numbering and in issue order
+  constexpr int NLB = NLOADS - NLA;   // weight loads of a slice
+  auto issue_a = [&](int ks, AStage& as, BRaw& b0, BRaw& b1) {
+    static_for<0, NLA>([&](auto i_) { issue_load(i_, ks, as, b0, b1, 0); });
   };
-  auto issue_b = [&](int ks, AStage& as, BRaw& b) {
-    static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, ks, as, b); });
+  auto issue_b = [&](int ks, AStage& as, BRaw& b0, BRaw& b1, int sel) {
+    static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, ks, as, b0, b1, sel); });
+  };
+  // Waits until at most N of this wave's loads are outstanding (they complete in issue order), and
+  // ties the registers that the oldest of them fill to that point.
+  // (The wait itself names no register: an in/out operand may be copied into place before the
+  // statement, i.e. read while its load is still in flight.)
+  auto wait_a = [&](auto n_, AStage& as) {
+    constexpr int N = decltype(n_)::value;
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : N) : "memory");
+    asm volatile("" : "+v"(as.sc));
+#pragma unroll
+    for (int j = 0; j < NAJ; ++j) asm volatile("" : "+v"(as.d[j]));
+  };
+  auto wait_b = [&](auto n_, BRaw& b) {
+    constexpr int N = decltype(n_)::value;
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : N) : "memory");
+#pragma unroll
+    for (int j = 0; j < NBL; ++j) asm volatile("" : "+v"(b.d[j]));
+    asm volatile("" : "+v"(b.sc[0]));
+    if constexpr (STAGE == 1) asm volatile("" : "+v"(b.sc[1]));
   };
   // Transposition of a raw set into MFMA operand order: one 8/16-byte load gives a lane the same
   // K row of 2 (gate/up) or 4 (down) column tiles, while an MFMA wants the 8 K rows of one tile
@@ -299,7 +374,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     }
   };
   auto store_a = [&](int st, const AStage& r) {
-    const uint32_t asreg = r.sc;
+    const uint32_t asreg = (uint32_t)r.sc;
     uint8_t* dst = sA + st * MX_SA;
 #pragma unroll
     for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
@@ -318,12 +393,10 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 
   // One K slice: row tiles are multiplied in groups of two; the fragments of the next group are
   // read from LDS while the current group's eight MFMAs run.  The groups of the first half are each
-  // followed by a share of the weight loads of slice ks+1 (if LB) and then of the activation loads
-  // of slice ks+2 (if LA).
+  // followed by a share of the loads of slice ks+2.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
-  auto compute = [&](auto lb_, auto la_, int st, const BFrag& b, int ks, AStage& as, BRaw& braw) {
-    constexpr bool LB = decltype(lb_)::value, LA = decltype(la_)::value;
+  auto compute = [&](int st, const BFrag& b, int ks, int ph, AStage& as, BRaw& b0, BRaw& b1) {
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
     const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
@@ -367,52 +440,67 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
                         "+a"(acc[2 * gi + 1][3])
                    :
                    : "memory");
-      // Loads are spread over the first NGL groups, weights (the longer latency) first; the rest of
-      // the slice is the time they have to arrive before the end of the slice needs them.
+      // The loads of slice ks+2 are spread over the first NGL groups, activations first; the rest of
+      // the slice is the time the activations have to arrive before the end of the slice stores
+      // them, while the weights have until the top of slice ks+2.  The weights go to the raw set
+      // that was transposed at the top of this slice (a uniform branch picks it).
       constexpr int NGL = (NG + 1) / 2;
       if constexpr (gi < NGL) {
         constexpr int lo = gi * NLOADS / NGL, hi = (gi + 1) * NLOADS / NGL;
-        static_for<lo, hi>([&](auto i_) {
-          constexpr int i = decltype(i_)::value;
-          constexpr int nb = NLOADS - NLA;
-          if constexpr (i < nb) {
-            if constexpr (LB) issue_load(std::integral_constant<int, NLA + i>{}, ks + 1, as, braw);
-          } else {
-            if constexpr (LA) issue_load(std::integral_constant<int, i - nb>{}, ks + 2, as, braw);
-          }
-        });
+        static_for<lo, hi>([&](auto i_) { issue_load(i_, ks + 2, as, b0, b1, ph); });
       }
     });
   };
 
   // ---- main loop ------------------------------------------------------------------------------------
   // Slice ks multiplies out of ring stage ks % 3 with the weights in `bc`, transposed at its top
-  // from the raw set.  During its first half the weight loads of slice ks+1 refill the raw set
-  // and the activation loads of slice ks+2 fill the staging registers, which go to ring stage
-  // (ks+2) % 3 at the end of the slice (that stage was last read in slice ks-1,
-  // which every wave left before the barrier that ended it).  One barrier per slice publishes the
-  // stores.
-  BRaw br;
+  // from raw set ks % 2.  During its first half the loads of slice ks+2 are issued: the weights
+  // refill that raw set, the activations fill the staging registers, which go to ring stage
+  // (ks+2) % 3 at the end of the slice (that stage was last read in slice ks-1, which every wave
+  // left before the barrier that ended it).  One barrier per slice publishes the stores.  The MFMA
+  // code exists once; only the few instructions that touch a raw set are selected by the parity of
+  // ks (two copies of the MFMA sequence do not survive register allocation).
+  BRaw br0, br1;
   AStage as;
   BFrag bc;
-  issue_a(0, as, br);
-  issue_b(0, as, br);
+  static_for<0, NBL>([&](auto j_) {
+    constexpr int j = decltype(j_)::value;
+    br0.d[j] = 0;
+    br1.d[j] = 0;
+  });
+  br0.sc[0] = br0.sc[1] = br1.sc[0] = br1.sc[1] = 0;
+  static_for<0, NAJ>([&](auto j_) { as.d[decltype(j_)::value] = 0; });
+  as.sc = 0;
+  issue_b(0, as, br0, br1, 0);
+  issue_b(1, as, br0, br1, 1);
+  issue_a(0, as, br0, br1);
+  wait_a(std::integral_constant<int, 0>{}, as);
   store_a(0, as);
-  if (nks > 1) {
-    issue_a(1, as, br);
-    store_a(1, as);
-  }
+  issue_a(1, as, br0, br1);
+  wait_a(std::integral_constant<int, 0>{}, as);
+  store_a(1, as);
   __syncthreads();
   int st = 0;
 #pragma clang loop unroll(disable)
   for (int ks = 0; ks < nks; ++ks) {
-    unpack_b(br, bc);
-    compute(std::true_type{}, std::true_type{}, st, bc, ks, as, br);
+    const int ph = ks & 1;
+    // weights of this slice: requested two slices ago; everything issued since is one slice's loads
+    if (ph) {
+      wait_b(std::integral_constant<int, NLOADS>{}, br1);
+      unpack_b(br1, bc);
+    } else {
+      wait_b(std::integral_constant<int, NLOADS>{}, br0);
+      unpack_b(br0, bc);
+    }
+    compute(st, bc, ks, ph, as, br0, br1);
     const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
+    // activations of slice ks+2: requested in this slice, before its NLB weight loads
+    wait_a(std::integral_constant<int, NLB>{}, as);
     store_a(st2, as);  // past the end: zeros into a stage that nobody reads any more
     __syncthreads();
     st = (st == 2) ? 0 : st + 1;
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
