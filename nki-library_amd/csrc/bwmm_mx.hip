@@ -285,48 +285,74 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     int sc;
   };
   const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, 0xffffffffu);
-  // Loads of a slice past the end go through descriptors of zero records: such a load is out of
-  // range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads.
-  auto desc = [&](const v4i& d, int ks) {
-    v4i r;
-    r[0] = uni(d[0]);
-    r[1] = uni(d[1]);
-    r[2] = uni((ks < nks) ? d[2] : 0);
-    r[3] = uni(d[3]);
+  // Scalar byte offset of a weight load = (offset of its row and column within the slice, fixed per
+  // load and kept in scalar registers) + (offset of the slice, computed once per slice): one scalar
+  // add per load.  Address arithmetic done per load costs more issue cycles than the MFMAs between
+  // two loads take.
+  int w_soff[NBL], s_soff[NBS];
+#pragma unroll
+  for (int i = 0; i < NBL; ++i) {
+    const int r = i % 8, gu = i / 8;  // gu is 0 in the down stage
+    const int pr = (r < 4) ? r : (16 + r - 4);
+    w_soff[i] = uni(((int64_t)gu * nH * a.I + (int64_t)pr * w_pstride + colu) * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < NBS; ++i) s_soff[i] = uni((int64_t)i * nH * a.I + colu);
+  // Everything a slice's loads share: descriptors (of zero records past the end: such a load is out
+  // of range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads)
+  // and the slice's scalar offsets.
+  struct SliceAddr {
+    v4i ra, ras, rw, rs;
+    int a_off, as_off, w_off, s_off;
+  };
+  auto slice_addr = [&](int ks) {
+    SliceAddr r;
+    const int live = (ks < nks) ? -1 : 0;
+    auto sel = [&](const v4i& d) {
+      v4i x;
+      x[0] = uni(d[0]);
+      x[1] = uni(d[1]);
+      x[2] = uni(d[2] & live);
+      x[3] = uni(d[3]);
+      return x;
+    };
+    r.ra = sel(ra_); r.ras = sel(ras_); r.rw = sel(rw_); r.rs = sel(rs_);
+    const int kt = ks >> 2, pb = ks & 3;
+    r.a_off = ks * 128;
+    r.as_off = ks * 4;
+    r.w_off = uni(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * 4);
+    r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
-  auto issue_load = [&](auto idx_, int ks, AStage& as, BRaw& b, BRaw& b1, int sel) {
+  auto issue_load = [&](auto idx_, const SliceAddr& sa, AStage& as, BRaw& b, BRaw& b1, int sel) {
     constexpr int idx = decltype(idx_)::value;
-    const int kt = ks >> 2, pb = ks & 3;
     if constexpr (idx < NAJ) {
-      ld_b128(as.d[idx], a_voff[idx], desc(ra_, ks), kt * 512 + pb * 128);
+      ld_b128(as.d[idx], a_voff[idx], sa.ra, sa.a_off);
     } else if constexpr (idx == NAJ) {
-      ld_b32(as.sc, as_voff, desc(ras_, ks), kt * 16 + pb * 4);
+      ld_b32(as.sc, as_voff, sa.ras, sa.as_off);
     } else if constexpr (idx < NAJ + 1 + NBL) {
       constexpr int i = idx - NAJ - 1;
-      constexpr int r = i % 8, gu = i / 8;  // gu is 0 in the down stage
-      constexpr int pr = (r < 4) ? r : (16 + r - 4);
-      const int64_t u0 = (int64_t)(pb * 32) * w_pstride + (int64_t)gu * nH * a.I + (int64_t)kt * w_tstride + colu;
       if constexpr (STAGE == 1)
-        ld2_b64(b.d[i], b1.d[i], sel, w_voff, desc(rw_, ks), uni((u0 + pr * w_pstride) * 4));
+        ld2_b64(b.d[i], b1.d[i], sel, w_voff, sa.rw, w_soff[i] + sa.w_off);
       else
-        ld2_b128(b.d[i], b1.d[i], sel, w_voff, desc(rw_, ks), uni((u0 + pr * w_pstride) * 4));
+        ld2_b128(b.d[i], b1.d[i], sel, w_voff, sa.rw, w_soff[i] + sa.w_off);
     } else {
       constexpr int i = idx - NAJ - 1 - NBL;
-      const int64_t us = (int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride + colu + (int64_t)i * nH * a.I;
       if constexpr (STAGE == 1)
-        ld2_u16(b.sc[i], b1.sc[i], sel, s_voff, desc(rs_, ks), uni(us));
+        ld2_u16(b.sc[i], b1.sc[i], sel, s_voff, sa.rs, s_soff[i] + sa.s_off);
       else
-        ld2_b32(b.sc[0], b1.sc[0], sel, s_voff, desc(rs_, ks), uni(us));
+        ld2_b32(b.sc[0], b1.sc[0], sel, s_voff, sa.rs, s_soff[0] + sa.s_off);
     }
   };
   constexpr int NLA = NAJ + 1;        // activation loads come first in the numbering and in issue order
   constexpr int NLB = NLOADS - NLA;   // weight loads of a slice
   auto issue_a = [&](int ks, AStage& as, BRaw& b0, BRaw& b1) {
-    static_for<0, NLA>([&](auto i_) { issue_load(i_, ks, as, b0, b1, 0); });
+    const SliceAddr sa = slice_addr(ks);
+    static_for<0, NLA>([&](auto i_) { issue_load(i_, sa, as, b0, b1, 0); });
   };
   auto issue_b = [&](int ks, AStage& as, BRaw& b0, BRaw& b1, int sel) {
-    static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, ks, as, b0, b1, sel); });
+    const SliceAddr sa = slice_addr(ks);
+    static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, sa, as, b0, b1, sel); });
   };
   // Waits until at most N of this wave's loads are outstanding (they complete in issue order), and
   // ties the registers that the oldest of them fill to that point.
@@ -400,6 +426,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
     const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
+    const SliceAddr sad = slice_addr(ks + 2);
     v8i af[2][2];
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
@@ -447,7 +474,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       constexpr int NGL = (NG + 1) / 2;
       if constexpr (gi < NGL) {
         constexpr int lo = gi * NLOADS / NGL, hi = (gi + 1) * NLOADS / NGL;
-        static_for<lo, hi>([&](auto i_) { issue_load(i_, ks + 2, as, b0, b1, ph); });
+        static_for<lo, hi>([&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
       }
     });
   };
