@@ -147,6 +147,9 @@ __device__ __forceinline__ void ld2_u16(int& d0, int& d1, int sel, uint32_t voff
       ".Lmx%=_1:\n\tbuffer_load_ushort %1, %2, %3, %4 offen\n.Lmx%=_2:"
       : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
 }
+__device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
 __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
@@ -422,6 +425,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // followed by a share of the loads of slice ks+2.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
+  constexpr int GA = (NG + 3) / 4;  // groups that carry activation loads
+  // weight loads issued after the last activation load of a slice
+  constexpr int NB_AFTER_A = NLB - ((GA - 1) * NLB) / NG;
   auto compute = [&](int st, const BFrag& b, int ks, int ph, AStage& as, BRaw& b0, BRaw& b1) {
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
@@ -467,15 +473,15 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
                         "+a"(acc[2 * gi + 1][3])
                    :
                    : "memory");
-      // The loads of slice ks+2 are spread over the first NGL groups, activations first; the rest of
-      // the slice is the time the activations have to arrive before the end of the slice stores
-      // them, while the weights have until the top of slice ks+2.  The weights go to the raw set
-      // that was transposed at the top of this slice (a uniform branch picks it).
-      constexpr int NGL = (NG + 1) / 2;
-      if constexpr (gi < NGL) {
-        constexpr int lo = gi * NLOADS / NGL, hi = (gi + 1) * NLOADS / NGL;
-        static_for<lo, hi>([&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
+      // The loads of slice ks+2: the activations after the first GA groups (they must have arrived
+      // by the end of this slice), the weights spread evenly over all groups (they have until the
+      // top of slice ks+2, and a burst of loads blocks the wave at the issue stage while the memory
+      // pipeline drains at HBM speed).  The weights go to the raw set that was transposed at the top
+      // of this slice.
+      if constexpr (gi < GA) {
+        static_for<gi * NLA / GA, (gi + 1) * NLA / GA>([&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
       }
+      static_for<NLA + gi * NLB / NG, NLA + (gi + 1) * NLB / NG>([&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
     });
   };
 
@@ -521,8 +527,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     }
     compute(st, bc, ks, ph, as, br0, br1);
     const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
-    // activations of slice ks+2: requested in this slice, before its NLB weight loads
-    wait_a(std::integral_constant<int, NLB>{}, as);
+    // activations of slice ks+2: requested in this slice, NB_AFTER_A weight loads ago
+    wait_a(std::integral_constant<int, NB_AFTER_A>{}, as);
     store_a(st2, as);  // past the end: zeros into a stage that nobody reads any more
     __syncthreads();
     st = (st == 2) ? 0 : st + 1;
@@ -632,24 +638,27 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       }
     }
     const bool post = a.scaling_mode == MOE_SCALE_POST;
+    // Rows go out through a descriptor that ends after the chunk's last row, so rows past the end
+    // are dropped by the range check and the stores need no branches.  (Rows of padding slots
+    // inside the chunk are written too: nothing reads the contributions of such slots.)
+    const v4i rd = make_rsrc(a.D + slot0 * a.H, (uint32_t)((int64_t)nrows * a.H * 2));
+    const uint32_t d_voff = (uint32_t)((4 * g * a.H + col0) * 2);
+    const int rowb = uni(a.H * 2);
+    typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+    typedef float v2f __attribute__((ext_vector_type(2)));
     static_for<0, NMT>([&](auto mt_) {
       constexpr int mt = decltype(mt_)::value;
-      {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = mt * 16 + 4 * g + r;
-          if (row < nrows && s_tok[row] >= 0) {
-            const float af = post ? s_aff[row] : 1.f;
-            uint32_t o[2];
+      for (int r = 0; r < 4; ++r) {
+        const int row = mt * 16 + 4 * g + r;
+        const float af = post ? s_aff[row] : 1.f;
+        v2i o;
 #pragma unroll
-            for (int t = 0; t < 4; t += 2) {
-              const float d0 = (acc[mt][t][r] + bd[t]) * af;
-              const float d1 = (acc[mt][t + 1][r] + bd[t + 1]) * af;
-              o[t >> 1] = (uint32_t)f32_to_bf16_bits(d0) | ((uint32_t)f32_to_bf16_bits(d1) << 16);
-            }
-            *(uint2*)(a.D + (slot0 + row) * a.H + col0) = make_uint2(o[0], o[1]);
-          }
+        for (int t = 0; t < 4; t += 2) {
+          const v2f d = {(acc[mt][t][r] + bd[t]) * af, (acc[mt][t + 1][r] + bd[t + 1]) * af};
+          o[t >> 1] = __builtin_bit_cast(int, __builtin_convertvector(d, v2bf));
         }
+        st_b64(o, d_voff, rd, (mt * 16 + r) * rowb);
       }
     });
   }
