@@ -3,10 +3,11 @@
 // test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:199-264).
 //
 // A stable counting sort of the routed (token, expert) pairs by expert:
-//   1. count_kernel    one workgroup per expert counts the tokens that selected it
+//   1. count_kernel    one workgroup per expert counts the tokens that selected it; the grid also
+//                      fills token_position_to_id with the pad id
 //   2. layout_kernel   one workgroup: blocks per expert, padding blocks to the last expert (or
 //                      split), exclusive scan -> first slot of every expert, block_to_expert,
-//                      conditions, and the pad fill of token_position_to_id
+//                      conditions
 //   3. scatter_kernel  one workgroup per expert ranks its tokens in ascending token id with a
 //                      block-wide scan and writes their ids
 // The work is latency bound (a few hundred KB of int32), so each step is a single small launch.
@@ -16,20 +17,31 @@ namespace moe {
 
 constexpr int BB_THREADS = 256;
 
+// 1 if token t lists expert e among its k choices.  k == 8 (two 16-byte loads) is the common case.
 __device__ __forceinline__ int token_selects(const int32_t* ids, int64_t t, int64_t k, int e) {
+  if (k == 8) {
+    const int4 a = ((const int4*)(ids + t * 8))[0], b = ((const int4*)(ids + t * 8))[1];
+    return (a.x == e) | (a.y == e) | (a.z == e) | (a.w == e) | (b.x == e) | (b.y == e) | (b.z == e) | (b.w == e);
+  }
   int hit = 0;
   for (int64_t j = 0; j < k; ++j) hit |= (ids[t * k + j] == e);
   return hit;
 }
 
+// One workgroup per expert counts its tokens (a ballot and a population count per 64 tokens); all
+// workgroups together also fill token_position_to_id with the pad id, which the scatter overwrites
+// where tokens sit.
 __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
-                                                             int32_t* __restrict__ counts) {
+                                                             int32_t* __restrict__ counts,
+                                                             int32_t* __restrict__ tp2id, int64_t NB, int pad_id) {
   __shared__ int red[BB_THREADS / 64];
   const int e = blockIdx.x;
   int c = 0;
-  for (int64_t t = threadIdx.x; t < T; t += BB_THREADS) c += token_selects(ids, t, k, e);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+  for (int64_t t0 = 0; t0 < T; t0 += BB_THREADS) {
+    const int64_t t = t0 + threadIdx.x;
+    const int hit = (t < T) ? token_selects(ids, t, k, e) : 0;
+    c += __popcll(__ballot(hit));
+  }
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -37,86 +49,87 @@ __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __r
     for (int i = 0; i < BB_THREADS / 64; ++i) s += red[i];
     counts[e] = s;
   }
+  for (int64_t i = (int64_t)blockIdx.x * BB_THREADS + threadIdx.x; i < NB; i += (int64_t)gridDim.x * BB_THREADS)
+    tp2id[i] = pad_id;
 }
 
 // ws layout: counts[E] | first_slot[E] | n_padding[1]
+// One workgroup: blocks per expert (padding blocks to the last expert, or split), exclusive scan ->
+// first slot of every expert, block_to_expert, conditions.  The scan over experts is serial (E is a
+// few hundred) but runs out of LDS; everything else is spread over the threads.
 __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ counts,
                                                               int32_t* __restrict__ first_slot,
                                                               int32_t* __restrict__ block_to_expert,
                                                               int32_t* __restrict__ conditions, int64_t n_conditions,
-                                                              int32_t* __restrict__ tp2id, int64_t E, int64_t B,
-                                                              int64_t N, int pad_id, int use_split_padding,
+                                                              int64_t E, int64_t B, int64_t N, int use_split_padding,
                                                               int32_t* __restrict__ status) {
+  extern __shared__ int s_nb[];  // [E] blocks per expert, then [E] first block of every expert
+  int* s_first = s_nb + E;
   __shared__ int s_npad;
-  __shared__ int s_bad;
-  // Serial part: E is at most a few hundred.
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) s_nb[e] = (int)((counts[e] + B - 1) / B);
+  __syncthreads();
   if (threadIdx.x == 0) {
     int64_t used = 0;
-    for (int64_t e = 0; e < E; ++e) used += (counts[e] + B - 1) / B;
+    for (int64_t e = 0; e < E; ++e) used += s_nb[e];
     int64_t npad = N - used;
-    s_bad = npad < 0;
+    if (status) *status = npad < 0;
     if (npad < 0) npad = 0;
     s_npad = (int)npad;
+    if (use_split_padding) {
+      s_nb[(E - 1) / 2] += (int)(npad / 2);
+      s_nb[E - 1] += (int)(npad - npad / 2);
+    } else {
+      s_nb[E - 1] += (int)npad;
+    }
     int64_t blk = 0;
     for (int64_t e = 0; e < E; ++e) {
-      int64_t nb = (counts[e] + B - 1) / B;
-      if (use_split_padding) {
-        if (e == (E - 1) / 2) nb += npad / 2;
-        if (e == E - 1) nb += npad - npad / 2;
-      } else if (e == E - 1) {
-        nb += npad;
-      }
-      first_slot[e] = (int32_t)(blk * B);
-      for (int64_t j = 0; j < nb && blk + j < N; ++j) block_to_expert[blk + j] = (int32_t)e;
-      blk += nb;
+      s_first[e] = (int)blk;
+      blk += s_nb[e];
     }
-    if (status) *status = s_bad;
   }
   __syncthreads();
-  const int64_t npad = s_npad;
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
+    const int64_t blk = s_first[e];
+    first_slot[e] = (int32_t)(blk * B);
+    for (int64_t j = 0; j < s_nb[e] && blk + j < N; ++j) block_to_expert[blk + j] = (int32_t)e;
+  }
   if (conditions) {
     // ones, then zeros over the trailing (npad + n_conditions - N) entries
-    const int64_t n_zero = npad + (n_conditions - N);
+    const int64_t n_zero = s_npad + (n_conditions - N);
     for (int64_t i = threadIdx.x; i < n_conditions; i += BB_THREADS)
       conditions[i] = (i < n_conditions - n_zero) ? 1 : 0;
   }
-  for (int64_t i = threadIdx.x; i < N * B; i += BB_THREADS) tp2id[i] = pad_id;
 }
 
+// One workgroup per expert ranks its tokens in ascending token id (ballot + population count below
+// the lane, plus the counts of the waves before) and writes their ids.
 __global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
                                                                const int32_t* __restrict__ first_slot,
                                                                int32_t* __restrict__ tp2id, int64_t NB) {
-  __shared__ int wsum[BB_THREADS / 64];
-  __shared__ int s_base;
+  __shared__ int wsum[2][BB_THREADS / 64];
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  if (threadIdx.x == 0) s_base = first_slot[e];
-  __syncthreads();
-  for (int64_t t0 = 0; t0 < T; t0 += BB_THREADS) {
+  int base = first_slot[e];
+  int buf = 0;
+  for (int64_t t0 = 0; t0 < T; t0 += BB_THREADS, buf ^= 1) {
     const int64_t t = t0 + threadIdx.x;
     const int hit = (t < T) ? token_selects(ids, t, k, e) : 0;
-    // inclusive scan of hit inside the wave
-    int inc = hit;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      int n = __shfl_up(inc, o, 64);
-      if (lane >= o) inc += n;
-    }
-    if (lane == 63) wsum[w] = inc;
-    __syncthreads();
+    const unsigned long long m = __ballot(hit);
+    const int below = __popcll(m & ((1ull << lane) - 1ull));
+    if (lane == 0) wsum[buf][w] = __popcll(m);
+    __syncthreads();  // wsum[buf] is rewritten two iterations later, after the next barrier
     int before = 0, total = 0;
+#pragma unroll
     for (int i = 0; i < BB_THREADS / 64; ++i) {
-      if (i < w) before += wsum[i];
-      total += wsum[i];
+      const int v = wsum[buf][i];
+      before += (i < w) ? v : 0;
+      total += v;
     }
-    const int base = s_base;
     if (hit) {
-      const int64_t pos = (int64_t)base + before + inc - 1;
+      const int64_t pos = (int64_t)base + before + below;
       if (pos < NB) tp2id[pos] = (int32_t)t;
     }
-    __syncthreads();
-    if (threadIdx.x == 0) s_base = base + total;
-    __syncthreads();
+    base += total;
   }
 }
 
@@ -138,11 +151,12 @@ extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, i
   int32_t* counts = (int32_t*)workspace;
   int32_t* first_slot = counts + E;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(bb_count_kernel, dim3((unsigned)E), dim3(BB_THREADS), 0, s, topk_ids, T, k, counts);
+  hipLaunchKernelGGL(bb_count_kernel, dim3((unsigned)E), dim3(BB_THREADS), 0, s, topk_ids, T, k, counts,
+                     token_position_to_id, N * B, skip_token ? -1 : (int)T);
   MOE_CHECK_LAUNCH();
-  hipLaunchKernelGGL(bb_layout_kernel, dim3(1), dim3(BB_THREADS), 0, s, counts, first_slot, block_to_expert,
-                     conditions, n_conditions, token_position_to_id, E, B, N, skip_token ? -1 : (int)T,
-                     use_split_padding, status_out);
+  if (2 * E * sizeof(int) > 48 * 1024) return MOE_E_BAD_SHAPE;
+  hipLaunchKernelGGL(bb_layout_kernel, dim3(1), dim3(BB_THREADS), 2 * E * sizeof(int), s, counts, first_slot,
+                     block_to_expert, conditions, n_conditions, E, B, N, use_split_padding, status_out);
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(bb_scatter_kernel, dim3((unsigned)E), dim3(BB_THREADS), 0, s, topk_ids, T, k, first_slot,
                      token_position_to_id, N * B);
