@@ -150,6 +150,11 @@ __device__ __forceinline__ void ld2_u16(int& d0, int& d1, int sel, uint32_t voff
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
+// 16 bytes per lane straight into LDS at lds + 16 * lane (no destination registers).
+__device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+}
 __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
@@ -203,7 +208,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   }
   __syncthreads();
 
-  // A staging: thread covers rows (tid>>3) + 32 j, 16-byte chunk tid&7
+  // A staging: thread covers rows (tid>>3) + 32 j; its load goes straight to LDS slot tid&7 of that
+  // row and fetches the 16-byte chunk (tid&7) ^ (row&7) that belongs there
   const int arow0 = tid >> 3, ach = tid & 7;
   constexpr int NAJ = NMT / 2;  // 32-row groups that hold rows of the NMT tiles
   // Per-lane 32-bit byte offsets (row * stride + chunk); the K offset is wave-uniform and is added
@@ -222,7 +228,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     } else {
       r = (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1)));
     }
-    a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)(ach * 16);
+    a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)((ach ^ (arow0 & 7)) * 16);
   }
   // A scales: thread covers row tid
   uint32_t as_voff;
@@ -284,7 +290,6 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     int sc[2];
   };
   struct AStage {
-    v4i d[NAJ];
     int sc;
   };
   const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, 0xffffffffu);
@@ -307,9 +312,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   struct SliceAddr {
     v4i ra, ras, rw, rs;
     int a_off, as_off, w_off, s_off;
+    uint32_t lds_a;  // LDS address of the ring stage that receives this slice's activations
   };
-  auto slice_addr = [&](int ks) {
+  const uint32_t lds_ring = (uint32_t)(uintptr_t)sA;
+  auto slice_addr = [&](int ks, int st) {
     SliceAddr r;
+    r.lds_a = uni((int)(lds_ring + (uint32_t)st * MX_SA));
     const int live = (ks < nks) ? -1 : 0;
     auto sel = [&](const v4i& d) {
       v4i x;
@@ -330,7 +338,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   auto issue_load = [&](auto idx_, const SliceAddr& sa, AStage& as, BRaw& b, BRaw& b1, int sel) {
     constexpr int idx = decltype(idx_)::value;
     if constexpr (idx < NAJ) {
-      ld_b128(as.d[idx], a_voff[idx], sa.ra, sa.a_off);
+      // the wave's 64 lanes fill 8 rows x 128 bytes = 1 KB of the ring stage, in lane order
+      ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[idx], sa.ra, sa.a_off);
     } else if constexpr (idx == NAJ) {
       ld_b32(as.sc, as_voff, sa.ras, sa.as_off);
     } else if constexpr (idx < NAJ + 1 + NBL) {
@@ -349,12 +358,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   };
   constexpr int NLA = NAJ + 1;        // activation loads come first in the numbering and in issue order
   constexpr int NLB = NLOADS - NLA;   // weight loads of a slice
-  auto issue_a = [&](int ks, AStage& as, BRaw& b0, BRaw& b1) {
-    const SliceAddr sa = slice_addr(ks);
+  auto issue_a = [&](int ks, int st, AStage& as, BRaw& b0, BRaw& b1) {
+    const SliceAddr sa = slice_addr(ks, st);
     static_for<0, NLA>([&](auto i_) { issue_load(i_, sa, as, b0, b1, 0); });
   };
   auto issue_b = [&](int ks, AStage& as, BRaw& b0, BRaw& b1, int sel) {
-    const SliceAddr sa = slice_addr(ks);
+    const SliceAddr sa = slice_addr(ks, 0);
     static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, sa, as, b0, b1, sel); });
   };
   // Waits until at most N of this wave's loads are outstanding (they complete in issue order), and
@@ -365,8 +374,6 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     constexpr int N = decltype(n_)::value;
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : N) : "memory");
     asm volatile("" : "+v"(as.sc));
-#pragma unroll
-    for (int j = 0; j < NAJ; ++j) asm volatile("" : "+v"(as.d[j]));
   };
   auto wait_b = [&](auto n_, BRaw& b) {
     constexpr int N = decltype(n_)::value;
@@ -404,9 +411,6 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   };
   auto store_a = [&](int st, const AStage& r) {
     const uint32_t asreg = (uint32_t)r.sc;
-    uint8_t* dst = sA + st * MX_SA;
-#pragma unroll
-    for (int j = 0; j < NAJ; ++j) *(v4i*)(dst + (arow0 + 32 * j) * MXROW + ((ach ^ (arow0 & 7)) * 16)) = r.d[j];
     // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
     uint8_t* sd = sS + st * MX_SS;
     const int mt = tid >> 4, cc = tid & 15;
@@ -432,7 +436,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
     const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
-    const SliceAddr sad = slice_addr(ks + 2);
+    const SliceAddr sad = slice_addr(ks + 2, (st == 0) ? 2 : st - 1);
     v8i af[2][2];
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
@@ -502,14 +506,13 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     br1.d[j] = 0;
   });
   br0.sc[0] = br0.sc[1] = br1.sc[0] = br1.sc[1] = 0;
-  static_for<0, NAJ>([&](auto j_) { as.d[decltype(j_)::value] = 0; });
   as.sc = 0;
   issue_b(0, as, br0, br1, 0);
   issue_b(1, as, br0, br1, 1);
-  issue_a(0, as, br0, br1);
+  issue_a(0, 0, as, br0, br1);
   wait_a(std::integral_constant<int, 0>{}, as);
   store_a(0, as);
-  issue_a(1, as, br0, br1);
+  issue_a(1, 1, as, br0, br1);
   wait_a(std::integral_constant<int, 0>{}, as);
   store_a(1, as);
   __syncthreads();
