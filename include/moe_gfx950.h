@@ -82,6 +82,28 @@ int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* gamma, int g
                             void* out_scale, void* out_norm, int64_t rows, int64_t H, float eps,
                             int64_t hidden_actual, int do_norm, int layout, void* stream);
 
+/* ---- router top-k front end ----------------------------------------------------------- */
+
+/* Replaces router_topk (src/nkilib_src/nkilib/core/router_topk/router_topk.py:55-75; semantics
+ * router_topk_torch_ref, src/nkilib_src/nkilib/core/router_topk/router_topk_torch.py:23-135).
+ * x bf16 [T, H] (the x_hbm_layout == 1 form), w bf16 [H, E], w_bias [E] (bias_dtype) or NULL.
+ * logits = x @ w + bias in fp32; expert_index int32 [T, k] = the k largest logits per token in
+ * descending order, ties to the lower expert index (NULL to skip the store, like
+ * skip_store_expert_index); router_logits [T, E] (bf16 / fp32, NULL = skip_store_router_logits).
+ * act_fn: 0 sigmoid, 1 softmax (RouterActFnType).  router_pre_norm != 0: activation over all E
+ * experts; with norm_topk_prob the selected values divided by their sum, zero elsewhere; without
+ * it the full activation (mask_to_topk != 0 zeroes the unselected experts -- the masked table
+ * moe_cte consumes; not a reference option).  router_pre_norm == 0: activation over the k selected
+ * logits only, scattered into zeros.  expert_affinities [T (+1 if pad_row), E] bf16 / fp32; with
+ * pad_row row T (the padding token of moe_cte) is zeroed.  topk_affinities fp32 [T, k] or NULL
+ * (return_eager_affi).  k <= 8, E <= 512, H % 64 == 0.  workspace: moe_router_topk_workspace_bytes. */
+size_t moe_router_topk_workspace_bytes(int64_t H, int64_t E);
+int moe_router_topk(const void* x, const void* w, const void* w_bias, int bias_dtype, int64_t T, int64_t H,
+                    int64_t E, int k, int act_fn, int router_pre_norm, int norm_topk_prob, int mask_to_topk,
+                    int pad_row, void* router_logits, int logits_dtype, int32_t* expert_index,
+                    void* expert_affinities, int aff_dtype, float* topk_affinities, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
 /* ---- token -> block index construction ---------------------------------------------- */
 
 /* Device version of generate_token_position_to_id_and_experts

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "nkilib", "_lib")
 OUT = os.path.join(OUT_DIR, "libmoe_gfx950.so")
-SOURCES = ["rmsnorm_quant.hip", "build_blocks.hip", "combine.hip", "bwmm.hip", "bwmm_mx.hip", "capi.hip"]
+SOURCES = ["rmsnorm_quant.hip", "build_blocks.hip", "combine.hip", "bwmm.hip", "bwmm_mx.hip", "router_topk.hip", "capi.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

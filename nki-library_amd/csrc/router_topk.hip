@@ -1,0 +1,321 @@
+// Router top-k front end for gfx950: logits = x @ w (+ bias), top-k selection, affinities.
+//
+// Semantics: router_topk_torch_ref, src/nkilib_src/nkilib/core/router_topk/router_topk_torch.py:23-135
+// (kernel signature src/nkilib_src/nkilib/core/router_topk/router_topk.py:55-75).
+//
+// Two launches:
+//   1. transpose_w_kernel   w [H,E] -> wt [E,H] (a few MB), so that both GEMM operands are contiguous
+//                           along K, which is what an MFMA lane wants (8 consecutive K values);
+//   2. router_kernel<NT>    a workgroup of 4 waves owns 128 tokens and all E = 16*NT experts.  Each wave
+//                           multiplies its 32 tokens (2 row tiles, fragments straight from global) with the
+//                           K slice of wt that the workgroup stages in LDS, with
+//                           v_mfma_f32_16x16x32_bf16 into 2*NT accumulator tiles, and then selects the top
+//                           k per token without leaving registers: a token's E logits sit in 16 lanes x
+//                           NT registers, so k rounds of (local argmax, 4-step lane reduction, retire the
+//                           winner) pick them in descending order, ties to the lower expert index.
+// Everything after the GEMM is fp32: softmax over all E (or over the k selected), sigmoid, the optional
+// division by the sum of the selected values.
+#include "common.hpp"
+
+namespace moe {
+
+constexpr int RT_THREADS = 256;
+constexpr int RT_TOK = 128;      // tokens per workgroup
+constexpr int RT_K = 64;         // K elements per LDS stage
+constexpr int RT_PITCH = RT_K + 8;  // bf16 elements per staged row of wt (16-byte aligned, conflict-spreading pad)
+
+__global__ __launch_bounds__(256) void transpose_w_kernel(const uint16_t* __restrict__ w, uint16_t* __restrict__ wt,
+                                                          int64_t H, int64_t E) {
+  __shared__ uint16_t tile[32][33];
+  const int64_t h0 = (int64_t)blockIdx.x * 32, e0 = (int64_t)blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int r = ty; r < 32; r += 8) {
+    const int64_t h = h0 + r, e = e0 + tx;
+    tile[r][tx] = (h < H && e < E) ? w[h * E + e] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) {
+    const int64_t e = e0 + r, h = h0 + tx;
+    if (e < E && h < H) wt[e * H + h] = tile[tx][r];
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_bytes_kernel(uint8_t* __restrict__ p, int64_t n) {
+  for (int64_t i = threadIdx.x; i < n; i += 256) p[i] = 0;
+}
+
+struct RouterArgs {
+  const uint16_t* x;   // bf16 [T, H]
+  const uint16_t* wt;  // bf16 [E, H]
+  const void* bias;    // [E] or null
+  int bias_dtype;
+  int64_t T, H, E;
+  int k, act_fn, pre_norm, norm_topk, mask_to_topk;
+  void* logits_out;    // [T, E] or null
+  int logits_dtype;
+  int32_t* index_out;  // [T, k] or null
+  void* aff_out;       // [T (+1), E]
+  int aff_dtype;
+  float* topk_aff_out; // [T, k] or null
+};
+
+__device__ __forceinline__ void store_val(void* p, int dtype, int64_t i, float v) {
+  if (dtype == MOE_DT_BF16) ((uint16_t*)p)[i] = f32_to_bf16_bits(v);
+  else ((float*)p)[i] = v;
+}
+
+// max / sum over the 16 lanes that share a token row (lanes with equal lane >> 4)
+__device__ __forceinline__ float row16_max(float v) {
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <int NT>
+__global__ __launch_bounds__(RT_THREADS) void router_kernel(const RouterArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint16_t* sW = (uint16_t*)smem;  // [16*NT][RT_PITCH]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int64_t t0 = (int64_t)blockIdx.x * RT_TOK + w * 32;
+  constexpr int EP = 16 * NT;  // experts covered by this instantiation (>= a.E)
+
+  v4f acc[2][NT];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int n = 0; n < NT; ++n) acc[m][n] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  // A rows: lane (c, g) of row tile m reads token t0 + 16m + c, K elements 8g .. 8g+7 of each 32-wide step
+  const uint16_t* xr[2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    int64_t t = t0 + 16 * m + c;
+    if (t >= a.T) t = a.T - 1;  // rows past the end repeat the last token; nothing is written for them
+    xr[m] = a.x + t * a.H + 8 * g;
+  }
+  const int nsteps = (int)(a.H / RT_K);
+  for (int s = 0; s < nsteps; ++s) {
+    const int64_t k0 = (int64_t)s * RT_K;
+    __syncthreads();
+    // stage wt[:, k0 .. k0+63]: 16*NT rows of 128 bytes, 8 chunks of 16 bytes each
+    for (int i = tid; i < EP * 8; i += RT_THREADS) {
+      const int e = i >> 3, ch = i & 7;
+      v4i v = {0, 0, 0, 0};
+      if (e < a.E) v = *(const v4i*)(a.wt + (int64_t)e * a.H + k0 + ch * 8);
+      *(v4i*)(sW + e * RT_PITCH + ch * 8) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      v8bf af[2];
+#pragma unroll
+      for (int m = 0; m < 2; ++m) af[m] = *(const v8bf*)(xr[m] + k0 + kk * 32);
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const v8bf bf = *(const v8bf*)(sW + (n * 16 + c) * RT_PITCH + kk * 32 + 8 * g);
+        acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[0], bf, acc[0][n], 0, 0, 0);
+        acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[1], bf, acc[1][n], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- epilogue: per token (row tile m, row 4g + r); the lane's experts are n*16 + c --------------
+  float bias[NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    const int e = n * 16 + c;
+    bias[n] = (a.bias && e < a.E) ? load_as_f32(a.bias, a.bias_dtype, e) : 0.f;
+  }
+  const float NEG = -__builtin_inff();
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int64_t t = t0 + 16 * m + 4 * g + r;
+      const bool live = t < a.T;  // uniform over the 16 lanes of the row
+      float v[NT];
+#pragma unroll
+      for (int n = 0; n < NT; ++n) v[n] = (n * 16 + c < a.E) ? acc[m][n][r] + bias[n] : NEG;
+      if (a.logits_out && live) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+          if (n * 16 + c < a.E) store_val(a.logits_out, a.logits_dtype, t * a.E + n * 16 + c, v[n]);
+      }
+      // full activation (pre-norm pipeline)
+      float fullv[NT];
+      if (a.pre_norm) {
+        if (a.act_fn == 1) {  // softmax over all experts
+          float mx = NEG;
+#pragma unroll
+          for (int n = 0; n < NT; ++n) mx = fmaxf(mx, v[n]);
+          mx = row16_max(mx);
+          float sum = 0.f;
+#pragma unroll
+          for (int n = 0; n < NT; ++n) {
+            fullv[n] = (v[n] == NEG) ? 0.f : expf(v[n] - mx);
+            sum += fullv[n];
+          }
+          sum = row16_sum(sum);
+#pragma unroll
+          for (int n = 0; n < NT; ++n) fullv[n] = fullv[n] / sum;
+        } else {
+#pragma unroll
+          for (int n = 0; n < NT; ++n) fullv[n] = 1.0f / (1.0f + expf(-v[n]));
+        }
+      }
+      // k rounds of argmax, ties to the lower expert index
+      unsigned taken = 0;  // bit n: the lane's expert n*16 + c has been selected
+      float selv[8];
+      int seli[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        selv[j] = 0.f;
+        seli[j] = 0;
+      }
+      for (int j = 0; j < a.k; ++j) {
+        float bv = NEG;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          const bool free_ = !((taken >> n) & 1u) && (n * 16 + c < a.E);
+          if (free_ && v[n] > bv) {  // ascending n: the lower index wins ties inside the lane
+            bv = v[n];
+            bi = n * 16 + c;
+          }
+        }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) {
+          const float ov = __shfl_xor(bv, o, 64);
+          const int oi = __shfl_xor(bi, o, 64);
+          if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+          }
+        }
+        if ((bi & 15) == c && bi < (int)a.E) taken |= 1u << (bi >> 4);
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj)
+          if (jj == j) {
+            selv[jj] = bv;
+            seli[jj] = bi;
+          }
+      }
+      // affinities of the selected experts
+      float affk[8];
+      if (a.pre_norm) {
+        float ssum = 0.f;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) ssum += ((taken >> n) & 1u) ? fullv[n] : 0.f;
+        ssum = row16_sum(ssum);
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+          float o = fullv[n];
+          if (a.norm_topk) o = ((taken >> n) & 1u) ? fullv[n] / ssum : 0.f;
+          else if (a.mask_to_topk) o = ((taken >> n) & 1u) ? fullv[n] : 0.f;
+          fullv[n] = o;
+        }
+      } else {
+        // activate the k selected logits only
+        float mx = selv[0], sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (j < a.k) {
+            affk[j] = (a.act_fn == 1) ? expf(selv[j] - mx) : 1.0f / (1.0f + expf(-selv[j]));
+            sum += affk[j];
+          }
+#pragma unroll
+        for (int n = 0; n < NT; ++n) fullv[n] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (j < a.k) {
+            if (a.act_fn == 1) affk[j] = affk[j] / sum;
+            if ((seli[j] & 15) == c) {
+#pragma unroll
+              for (int n = 0; n < NT; ++n)
+                if (n == (seli[j] >> 4)) fullv[n] = affk[j];
+            }
+          }
+      }
+      if (live) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+          if (n * 16 + c < a.E) store_val(a.aff_out, a.aff_dtype, t * a.E + n * 16 + c, fullv[n]);
+        if (c == 0) {
+          for (int j = 0; j < a.k; ++j) {
+            if (a.index_out) a.index_out[t * a.k + j] = seli[j];
+          }
+        }
+        if (a.topk_aff_out) {
+          // the lane that owns the selected expert knows its final affinity
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (j < a.k && (seli[j] & 15) == c) {
+#pragma unroll
+              for (int n = 0; n < NT; ++n)
+                if (n == (seli[j] >> 4)) a.topk_aff_out[t * a.k + j] = fullv[n];
+            }
+        }
+      }
+    }
+  }
+}
+
+template <int NT>
+static int launch_router(const RouterArgs& a, hipStream_t s) {
+  const unsigned grid = (unsigned)((a.T + RT_TOK - 1) / RT_TOK);
+  const size_t lds = (size_t)16 * NT * RT_PITCH * 2;
+  hipError_t err = hipFuncSetAttribute((const void*)router_kernel<NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (err != hipSuccess) return MOE_E_LAUNCH;
+  hipLaunchKernelGGL(router_kernel<NT>, dim3(grid), dim3(RT_THREADS), lds, s, a);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+}  // namespace moe
+
+using namespace moe;
+
+extern "C" size_t moe_router_topk_workspace_bytes(int64_t H, int64_t E) { return (size_t)(H * E * 2 + 256); }
+
+extern "C" int moe_router_topk(const void* x, const void* w, const void* w_bias, int bias_dtype, int64_t T, int64_t H,
+                               int64_t E, int k, int act_fn, int router_pre_norm, int norm_topk_prob, int mask_to_topk,
+                               int pad_row, void* router_logits, int logits_dtype, int32_t* expert_index,
+                               void* expert_affinities, int aff_dtype, float* topk_affinities, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  if (!x || !w || !expert_affinities || !workspace) return MOE_E_BAD_ARG;
+  if (T < 0 || H <= 0 || E <= 0 || k <= 0 || k > 8 || k > E) return MOE_E_BAD_ARG;
+  if (act_fn != 0 && act_fn != 1) return MOE_E_BAD_ARG;
+  if (H % RT_K != 0 || E > 512) return MOE_E_BAD_SHAPE;
+  if (aff_dtype != MOE_DT_BF16 && aff_dtype != MOE_DT_FP32) return MOE_E_BAD_ARG;
+  if (router_logits && logits_dtype != MOE_DT_BF16 && logits_dtype != MOE_DT_FP32) return MOE_E_BAD_ARG;
+  if (w_bias && bias_dtype != MOE_DT_BF16 && bias_dtype != MOE_DT_FP32 && bias_dtype != MOE_DT_FP16) return MOE_E_BAD_ARG;
+  if (workspace_bytes < moe_router_topk_workspace_bytes(H, E)) return MOE_E_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  if (pad_row) {
+    // row T of the affinity table is the padding token's: zeros (E elements)
+    const int64_t n = E * (aff_dtype == MOE_DT_BF16 ? 2 : 4);
+    hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1), dim3(256), 0, s,
+                       (uint8_t*)expert_affinities + T * n, n);
+    MOE_CHECK_LAUNCH();
+  }
+  if (T == 0) return MOE_OK;
+  uint16_t* wt = (uint16_t*)workspace;
+  hipLaunchKernelGGL(transpose_w_kernel, dim3((unsigned)((H + 31) / 32), (unsigned)((E + 31) / 32)), dim3(256), 0, s,
+                     (const uint16_t*)w, wt, H, E);
+  MOE_CHECK_LAUNCH();
+  RouterArgs a;
+  a.x = (const uint16_t*)x; a.wt = wt; a.bias = w_bias; a.bias_dtype = bias_dtype;
+  a.T = T; a.H = H; a.E = E; a.k = k; a.act_fn = act_fn; a.pre_norm = router_pre_norm; a.norm_topk = norm_topk_prob;
+  a.mask_to_topk = mask_to_topk;
+  a.logits_out = router_logits; a.logits_dtype = logits_dtype; a.index_out = expert_index;
+  a.aff_out = expert_affinities; a.aff_dtype = aff_dtype; a.topk_aff_out = topk_affinities;
+  if (E <= 128) return launch_router<8>(a, s);
+  if (E <= 256) return launch_router<16>(a, s);
+  return launch_router<32>(a, s);
+}

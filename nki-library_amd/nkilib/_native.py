@@ -34,6 +34,8 @@ EXPORTED_SYMBOLS = (
     "moe_rmsnorm_quant_mxfp8",
     "moe_build_blocks_workspace_bytes",
     "moe_build_blocks",
+    "moe_router_topk_workspace_bytes",
+    "moe_router_topk",
     "moe_blockwise_workspace_bytes",
     "moe_blockwise",
     "moe_blockwise_stages",
@@ -123,6 +125,12 @@ def lib():
     L.moe_build_blocks.restype = c_int
     L.moe_build_blocks.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p,
                                    c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]
+    L.moe_router_topk_workspace_bytes.restype = c_size_t
+    L.moe_router_topk_workspace_bytes.argtypes = [c_int64, c_int64]
+    L.moe_router_topk.restype = c_int
+    L.moe_router_topk.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_int,
+                                  c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                  c_size_t, c_void_p]
     L.moe_blockwise_workspace_bytes.restype = c_size_t
     L.moe_blockwise_workspace_bytes.argtypes = [POINTER(BwmmArgs)]
     L.moe_blockwise.restype = c_int

@@ -32,3 +32,13 @@ class QuantizationType(Enum):
     MX = 3
     STATIC_MX = 4
     ROW_MX = 5
+
+
+class RouterActFnType(Enum):
+    """Activation of the router top-k kernel (common_types.py:39-46 of the reference)."""
+
+    SIGMOID = 0
+    SOFTMAX = 1
+
+    def __str__(self):
+        return self.name.lower()

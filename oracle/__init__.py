@@ -20,6 +20,9 @@ Parity unpinned (no source, fixture or mathematical fact fixes them):
     explicit saturating clip the goldens apply, i.e. IEEE/OCP behaviour.
   * hardware approximations of ``nisa.activation`` / ``nisa.quantize_mx``; the
     oracle follows the numpy goldens, not the hardware.
+  * router top-k: which of several experts with equal logits ``torch.argsort``
+    returns (the reference's bf16 logits tie often); the oracle selects on
+    fp32 logits and breaks ties towards the lower expert index.
 
 Modules
   numerics   bf16 / fp8-e4m3fn / E8M0 encode + decode
@@ -27,5 +30,6 @@ Modules
   blocks     token -> block index construction (bit exact, integer)
   rmsnorm    RMSNorm + fp8 ROW / STATIC quantise, RMSNorm -> MXFP8
   moe        blockwise MoE goldens (bf16, fp8-weight, fp8-row, MXFP8)
+  router     router top-k (logits, top-k selection, affinities)
   compare    the reference comparator (max-abs-rel "maxAllClose")
 """
