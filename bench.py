@@ -40,6 +40,9 @@ def parse_args():
     ap.add_argument("--workload", default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-blocks", type=int, default=6, help="blocks of the workload timed on the CPU oracle")
+    ap.add_argument("--with-router", action="store_true",
+                    help="start from hidden states: time the router top-k front end (synthetic router weights) as a "
+                         "stage of its own and route with its output; the headline metric stays the MoE layer")
     ap.add_argument("--routing", default="router", choices=["router", "balanced"],
                     help="router: top-k of synthetic scores (the reported workload); balanced: every expert gets "
                          "exactly T*k/E rows (diagnostic, shows the cost of ragged expert loads)")
@@ -146,6 +149,14 @@ def main():
     gu_x4 = t["gu_q"].view(torch.int32).reshape(t["gu_q"].shape[:-1])
 
     names = ["norm_quant", "build_blocks", "prep", "gate_up", "down", "combine"]
+    if args.with_router:
+        from nkilib.core.router_topk import route_for_moe
+        from nkilib.core.utils.common_types import RouterActFnType
+
+        names = ["router"] + names
+        g = torch.Generator(device=dev)
+        g.manual_seed(77)
+        w_router = (torch.randn((H, E), generator=g, device=dev) * 0.05).to(torch.bfloat16)
     events = []
 
     def rec():
@@ -157,6 +168,10 @@ def main():
         if timed:
             events.append([])
             rec()
+        if args.with_router:
+            t["ids"], t["aff"] = route_for_moe(t["x"], w_router, None, k, RouterActFnType.SIGMOID, norm_topk_prob=True)
+            if timed:
+                rec()
         xq, xs = rmsnorm_mx_quantize(t["x"], t["gamma"])
         if timed:
             rec()
