@@ -509,12 +509,15 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   as.sc = 0;
   issue_b(0, as, br0, br1, 0);
   issue_b(1, as, br0, br1, 1);
+  // both leading slices in one round trip
+  AStage as1;
+  as1.sc = 0;
   issue_a(0, 0, as, br0, br1);
+  issue_a(1, 1, as1, br0, br1);
   wait_a(std::integral_constant<int, 0>{}, as);
+  wait_a(std::integral_constant<int, 0>{}, as1);
   store_a(0, as);
-  issue_a(1, 1, as, br0, br1);
-  wait_a(std::integral_constant<int, 0>{}, as);
-  store_a(1, as);
+  store_a(1, as1);
   __syncthreads();
   int st = 0;
 #pragma clang loop unroll(disable)
