@@ -82,13 +82,41 @@ __device__ __forceinline__ v8i frag_from_lds(const uint8_t* plo, const uint8_t* 
   return r;
 }
 
-// One MFMA of row-tile fragment `af` (scale byte OA of `sa`) with column tile NT of `b`.
+// One MFMA of row-tile fragment `af` (scale byte OA of `sa`) with column tile NT of `b`, written as
+// an instruction: statements of this kind keep their order, so what the source puts between two
+// MFMAs (a load, an LDS read) is issued between them and runs in the shadow of the first -- with one
+// wave per SIMD nothing else hides it.  op_sel / op_sel_hi carry bit 0 / bit 1 of the two scale
+// byte selectors.
+#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)                                                              \
+  if constexpr (OA == OA_ && OB == OB_)                                                                   \
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:" SEL_ " op_sel_hi:" SELHI_ \
+                 : "+a"(c) : "v"(af), "v"(bf), "v"(sa), "v"(sb))
+template <int OA, int OB>
+__device__ __forceinline__ void mfma_asm(v4f& c, const v8i& af, const v8i& bf, int sa, int sb) {
+  MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
+  MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
+  MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
+  MX_MFMA_CASE(3, 0, "[1,0,0]", "[1,0,0]");
+  MX_MFMA_CASE(0, 1, "[0,1,0]", "[0,0,0]");
+  MX_MFMA_CASE(1, 1, "[1,1,0]", "[0,0,0]");
+  MX_MFMA_CASE(2, 1, "[0,1,0]", "[1,0,0]");
+  MX_MFMA_CASE(3, 1, "[1,1,0]", "[1,0,0]");
+  MX_MFMA_CASE(0, 2, "[0,0,0]", "[0,1,0]");
+  MX_MFMA_CASE(1, 2, "[1,0,0]", "[0,1,0]");
+  MX_MFMA_CASE(2, 2, "[0,0,0]", "[1,1,0]");
+  MX_MFMA_CASE(3, 2, "[1,0,0]", "[1,1,0]");
+  MX_MFMA_CASE(0, 3, "[0,1,0]", "[0,1,0]");
+  MX_MFMA_CASE(1, 3, "[1,1,0]", "[0,1,0]");
+  MX_MFMA_CASE(2, 3, "[0,1,0]", "[1,1,0]");
+  MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
+}
+#undef MX_MFMA_CASE
 template <int STAGE, int OA, int NT>
-__device__ __forceinline__ v4f mfma_tile(const v8i& af, const BFrag& b, const v4f& c, int sa) {
+__device__ __forceinline__ void mfma_tile(const v8i& af, const BFrag& b, v4f& c, int sa) {
   if constexpr (STAGE == 1)
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, b.f[NT], c, 0, 0, OA, sa, NT & 1, b.sc[NT >> 1]);
+    mfma_asm<OA, (NT & 1)>(c, af, b.f[NT], sa, b.sc[NT >> 1]);
   else
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, b.f[NT], c, 0, 0, OA, sa, NT, b.sc[0]);
+    mfma_asm<OA, NT>(c, af, b.f[NT], sa, b.sc[0]);
 }
 
 // Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
@@ -429,9 +457,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // followed by a share of the loads of slice ks+2.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
-  constexpr int GA = (NG + 3) / 4;  // groups that carry activation loads
-  // weight loads issued after the last activation load of a slice
-  constexpr int NB_AFTER_A = NLB - ((GA - 1) * NLB) / NG;
+  constexpr int NB_AFTER_A = NLB;  // weight loads issued after the last activation load of a slice
   auto compute = [&](int st, const BFrag& b, int ks, int ph, AStage& as, BRaw& b0, BRaw& b1) {
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
@@ -452,40 +478,18 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       // fragments it returns), so the two fragment sets stay live together and the LDS latency of
       // the next group is covered by this group's eight MFMAs.
       asm volatile("" : "+v"(af[cur][0]), "+v"(af[cur][1]) : : "memory");
-      {
-        constexpr int mt = 2 * gi;
-        const int sa = asc[mt / 4];
-        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][0], b, acc[mt][0], sa);
-        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][0], b, acc[mt][1], sa);
-        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][0], b, acc[mt][2], sa);
-        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][0], b, acc[mt][3], sa);
-      }
-      {
-        constexpr int mt = 2 * gi + 1;
-        const int sa = asc[mt / 4];
-        acc[mt][0] = mfma_tile<STAGE, mt % 4, 0>(af[cur][1], b, acc[mt][0], sa);
-        acc[mt][1] = mfma_tile<STAGE, mt % 4, 1>(af[cur][1], b, acc[mt][1], sa);
-        acc[mt][2] = mfma_tile<STAGE, mt % 4, 2>(af[cur][1], b, acc[mt][2], sa);
-        acc[mt][3] = mfma_tile<STAGE, mt % 4, 3>(af[cur][1], b, acc[mt][3], sa);
-      }
-      // Pin the eight results here, in accumulation registers.  Without a fixed point the
-      // compiler sinks the (side-effect free) MFMAs towards the end of the K step and hoists
-      // every fragment read to its top, which does not fit the register file.  The memory clobber
-      // also keeps this group's share of the loads behind the MFMAs.
-      asm volatile("" : "+a"(acc[2 * gi][0]), "+a"(acc[2 * gi][1]), "+a"(acc[2 * gi][2]), "+a"(acc[2 * gi][3]),
-                        "+a"(acc[2 * gi + 1][0]), "+a"(acc[2 * gi + 1][1]), "+a"(acc[2 * gi + 1][2]),
-                        "+a"(acc[2 * gi + 1][3])
-                   :
-                   : "memory");
-      // The loads of slice ks+2: the activations after the first GA groups (they must have arrived
-      // by the end of this slice), the weights spread evenly over all groups (they have until the
-      // top of slice ks+2, and a burst of loads blocks the wave at the issue stage while the memory
-      // pipeline drains at HBM speed).  The weights go to the raw set that was transposed at the top
-      // of this slice.
-      if constexpr (gi < GA) {
-        static_for<gi * NLA / GA, (gi + 1) * NLA / GA>([&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
-      }
-      static_for<NLA + gi * NLB / NG, NLA + (gi + 1) * NLB / NG>([&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
+      // Eight MFMAs; after each one, its share of the loads of slice ks+2 (activations first: they
+      // must have arrived by the end of this slice; the weights have until the top of slice ks+2 and
+      // go to the raw set that was transposed at the top of this slice).  One or two loads fit in
+      // the 32 cycles an MFMA occupies the matrix pipe; a burst of them does not.
+      static_for<0, 8>([&](auto j_) {
+        constexpr int j = decltype(j_)::value;
+        constexpr int mt = 2 * gi + j / 4, nt = j % 4;
+        constexpr int m = gi * 8 + j;  // MFMA number within the slice
+        mfma_tile<STAGE, mt % 4, nt>(af[cur][j / 4], b, acc[mt][nt], asc[mt / 4]);
+        static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>(
+            [&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
+      });
     });
   };
 
@@ -539,7 +543,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     __syncthreads();
     st = (st == 2) ? 0 : st + 1;
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // the last MFMAs are still in the pipe: as instructions of unknown kind to the compiler, it adds
+  // no wait between them and the first read of an accumulator
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
