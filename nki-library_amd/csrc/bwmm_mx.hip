@@ -414,28 +414,26 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // Transposition of a raw set into MFMA operand order: one 8/16-byte load gives a lane the same
   // K row of 2 (gate/up) or 4 (down) column tiles, while an MFMA wants the 8 K rows of one tile
   // in consecutive registers.
-  auto unpack_b = [&](const BRaw& b, BFrag& f) {
-    if constexpr (STAGE == 1) {
+  // `m1` (all ones or zero, uniform) picks set b1 or b0: one select per register does the choice
+  // and the transposition together, with no branch (a branch ends in a block of copies per path).
+  auto pick = [&](int& d, int x0, int x1, uint64_t m1) {
+    asm volatile("v_cndmask_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x0), "v"(x1), "s"(m1));
+  };
+  auto unpack_b = [&](const BRaw& b0, const BRaw& b1, uint64_t m1, BFrag& f) {
+    constexpr int NT_LD = (STAGE == 1) ? 2 : 4;  // column tiles per load
+    int t[4][8];
 #pragma unroll
-      for (int gu = 0; gu < 2; ++gu)
+    for (int i = 0; i < NBL; ++i)
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          f.f[gu * 2 + 0][r] = b.d[gu * 8 + r][0];
-          f.f[gu * 2 + 1][r] = b.d[gu * 8 + r][1];
-        }
-      f.sc[0] = b.sc[0];
-      f.sc[1] = b.sc[1];
-    } else {
+      for (int x = 0; x < NT_LD; ++x) pick(t[(i / 8) * NT_LD + x][i % 8], b0.d[i][x], b1.d[i][x], m1);
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        f.f[0][r] = b.d[r][0];
-        f.f[1][r] = b.d[r][1];
-        f.f[2][r] = b.d[r][2];
-        f.f[3][r] = b.d[r][3];
-      }
-      f.sc[0] = b.sc[0];
-      f.sc[1] = 0;
-    }
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int r = 0; r < 8; ++r) f.f[nt][r] = t[nt][r];
+    pick(f.sc[0], b0.sc[0], b1.sc[0], m1);
+    if constexpr (STAGE == 1) pick(f.sc[1], b0.sc[1], b1.sc[1], m1);
+    else f.sc[1] = 0;
+    asm volatile("s_nop 1");  // the selects feed the first MFMA
   };
   auto store_a = [&](int st, const AStage& r) {
     const uint32_t asreg = (uint32_t)r.sc;
@@ -458,14 +456,18 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
   constexpr int NB_AFTER_A = NLB;  // weight loads issued after the last activation load of a slice
-  auto compute = [&](int st, const BFrag& b, int ks, int ph, AStage& as, BRaw& b0, BRaw& b1) {
+  auto compute = [&](int st, BFrag& b, int ks, int ph, AStage& as, BRaw& b0, BRaw& b1) {
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
     const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
-    const SliceAddr sad = slice_addr(ks + 2, (st == 0) ? 2 : st - 1);
+    // first fragments of this slice: in flight while the weights are transposed
     v8i af[2][2];
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
+    asm volatile("" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLOADS) : "memory");
+    unpack_b(b0, b1, ph ? ~0ull : 0ull, b);
+    SliceAddr sad;
     static_for<0, NG>([&](auto gi_) {
       constexpr int gi = decltype(gi_)::value;
       constexpr int cur = gi & 1, nxt = cur ^ 1;
@@ -487,6 +489,13 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         constexpr int mt = 2 * gi + j / 4, nt = j % 4;
         constexpr int m = gi * 8 + j;  // MFMA number within the slice
         mfma_tile<STAGE, mt % 4, nt>(af[cur][j / 4], b, acc[mt][nt], asc[mt / 4]);
+        if constexpr (m == 0) {
+          // the scalar arithmetic for the addresses of slice ks+2 starts here, behind the first
+          // MFMA, instead of ahead of it
+          int ks2 = ks + 2;
+          asm volatile("" : "+s"(ks2));
+          sad = slice_addr(ks2, (st == 0) ? 2 : st - 1);
+        }
         static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>(
             [&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
       });
@@ -528,13 +537,6 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   for (int ks = 0; ks < nks; ++ks) {
     const int ph = ks & 1;
     // weights of this slice: requested two slices ago; everything issued since is one slice's loads
-    if (ph) {
-      wait_b(std::integral_constant<int, NLOADS>{}, br1);
-      unpack_b(br1, bc);
-    } else {
-      wait_b(std::integral_constant<int, NLOADS>{}, br0);
-      unpack_b(br0, bc);
-    }
     compute(st, bc, ks, ph, as, br0, br1);
     const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
     // activations of slice ks+2: requested in this slice, NB_AFTER_A weight loads ago
