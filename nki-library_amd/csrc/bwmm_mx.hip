@@ -68,9 +68,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 struct BFrag {
-  v8i f[4];   // four column tiles
-  int sc[2];  // E8M0 scale bytes: gate/up stage: sc[0] = gate tiles 0,1 (bytes 0,1), sc[1] = up tiles;
-              // down stage: sc[0] = all four tiles (bytes 0..3)
+  v8i f[4];  // four column tiles
+  int sc;    // their E8M0 scale bytes (byte t = tile t)
 };
 
 __device__ __forceinline__ v8i frag_from_lds(const uint8_t* plo, const uint8_t* phi) {
@@ -111,12 +110,9 @@ __device__ __forceinline__ void mfma_asm(v4f& c, const v8i& af, const v8i& bf, i
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
 }
 #undef MX_MFMA_CASE
-template <int STAGE, int OA, int NT>
+template <int OA, int NT>
 __device__ __forceinline__ void mfma_tile(const v8i& af, const BFrag& b, v4f& c, int sa) {
-  if constexpr (STAGE == 1)
-    mfma_asm<OA, (NT & 1)>(c, af, b.f[NT], sa, b.sc[NT >> 1]);
-  else
-    mfma_asm<OA, NT>(c, af, b.f[NT], sa, b.sc[0]);
+  mfma_asm<OA, NT>(c, af, b.f[NT], sa, b.sc);
 }
 
 // Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
@@ -145,9 +141,6 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
-__device__ __forceinline__ void ld_b64(v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-}
 // One load into d1 if sel != 0, else into d0.  The choice is made inside the statement, so the
 // compiler sees straight-line code that updates both variables in place (a branch of its own would
 // end in copies of registers whose loads are still in flight).
@@ -157,22 +150,10 @@ __device__ __forceinline__ void ld2_b128(v4i& d0, v4i& d1, int sel, uint32_t vof
       ".Lmx%=_1:\n\tbuffer_load_dwordx4 %1, %2, %3, %4 offen\n.Lmx%=_2:"
       : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
 }
-__device__ __forceinline__ void ld2_b64(v2i& d0, v2i& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile(
-      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dwordx2 %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
-      ".Lmx%=_1:\n\tbuffer_load_dwordx2 %1, %2, %3, %4 offen\n.Lmx%=_2:"
-      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
-}
 __device__ __forceinline__ void ld2_b32(int& d0, int& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile(
       "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dword %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
       ".Lmx%=_1:\n\tbuffer_load_dword %1, %2, %3, %4 offen\n.Lmx%=_2:"
-      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
-}
-__device__ __forceinline__ void ld2_u16(int& d0, int& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile(
-      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_ushort %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
-      ".Lmx%=_1:\n\tbuffer_load_ushort %1, %2, %3, %4 offen\n.Lmx%=_2:"
       : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
 }
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
@@ -185,9 +166,6 @@ __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v
 }
 __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-}
-__device__ __forceinline__ void ld_u16(int& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 // NMT = number of 16-row tiles this instantiation multiplies (the chunk has at most NMT*16 rows).
@@ -286,14 +264,20 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   v4i rw_, rs_;
   uint32_t w_voff, s_voff;
   int64_t colu;
+  // A lane loads 16 bytes = 4 adjacent columns of one K row: column 4*cl + t belongs to column tile
+  // t.  In the gate/up stage the wave's 32 gate columns take lanes c = 0..7 of each group and its 32
+  // up columns lanes c = 8..15, so every column tile is half gate, half up, and one load instruction
+  // fetches 128 contiguous bytes of gate and of up for 4 K rows.  (8-byte loads, one tile pair per
+  // load, cost the memory pipeline as much per instruction as 16-byte ones.)
+  const int hcol = (STAGE == 1) ? (c >> 3) : 0, cl = (STAGE == 1) ? (c & 7) : c;
   if (STAGE == 1) {
     w_pstride = 2 * nH * a.I;
     w_tstride = a.I;
     colu = (int64_t)tI * 512 + (int64_t)q * Pt + p0;
     rw_ = make_rsrc(a.W + (int64_t)e * 128 * w_pstride, (uint32_t)(128 * w_pstride * 4));
     rs_ = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
-    w_voff = (uint32_t)((4 * g * w_pstride + 2 * c) * 4);
-    s_voff = (uint32_t)(g * w_pstride + 2 * c);
+    w_voff = (uint32_t)((4 * g * w_pstride + hcol * nH * a.I + 4 * cl) * 4);
+    s_voff = (uint32_t)(g * w_pstride + hcol * nH * a.I + 4 * cl);
   } else {
     w_pstride = (int64_t)a.nI * a.H;
     w_tstride = a.H;
@@ -310,12 +294,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   //   NAJ                   activation scales
   //   NAJ+1 .. NAJ+NBL      weights
   //   NAJ+NBL+1 ..          weight scales
-  constexpr int NBL = (STAGE == 1) ? 16 : 8;
-  constexpr int NBS = (STAGE == 1) ? 2 : 1;
+  constexpr int NBL = 8;
+  constexpr int NBS = 1;
   constexpr int NLOADS = NAJ + 1 + NBL + NBS;
   struct BRaw {
-    typename std::conditional<STAGE == 1, v2i, v4i>::type d[NBL];
-    int sc[2];
+    v4i d[NBL];
+    int sc;
   };
   struct AStage {
     int sc;
@@ -328,12 +312,11 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   int w_soff[NBL], s_soff[NBS];
 #pragma unroll
   for (int i = 0; i < NBL; ++i) {
-    const int r = i % 8, gu = i / 8;  // gu is 0 in the down stage
-    const int pr = (r < 4) ? r : (16 + r - 4);
-    w_soff[i] = uni(((int64_t)gu * nH * a.I + (int64_t)pr * w_pstride + colu) * 4);
+    const int pr = (i < 4) ? i : (16 + i - 4);
+    w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * 4);
   }
 #pragma unroll
-  for (int i = 0; i < NBS; ++i) s_soff[i] = uni((int64_t)i * nH * a.I + colu);
+  for (int i = 0; i < NBS; ++i) s_soff[i] = uni(colu);
   // Everything a slice's loads share: descriptors (of zero records past the end: such a load is out
   // of range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads)
   // and the slice's scalar offsets.
@@ -372,16 +355,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       ld_b32(as.sc, as_voff, sa.ras, sa.as_off);
     } else if constexpr (idx < NAJ + 1 + NBL) {
       constexpr int i = idx - NAJ - 1;
-      if constexpr (STAGE == 1)
-        ld2_b64(b.d[i], b1.d[i], sel, w_voff, sa.rw, w_soff[i] + sa.w_off);
-      else
-        ld2_b128(b.d[i], b1.d[i], sel, w_voff, sa.rw, w_soff[i] + sa.w_off);
+      ld2_b128(b.d[i], b1.d[i], sel, w_voff, sa.rw, w_soff[i] + sa.w_off);
     } else {
-      constexpr int i = idx - NAJ - 1 - NBL;
-      if constexpr (STAGE == 1)
-        ld2_u16(b.sc[i], b1.sc[i], sel, s_voff, sa.rs, s_soff[i] + sa.s_off);
-      else
-        ld2_b32(b.sc[0], b1.sc[0], sel, s_voff, sa.rs, s_soff[0] + sa.s_off);
+      ld2_b32(b.sc, b1.sc, sel, s_voff, sa.rs, s_soff[0] + sa.s_off);
     }
   };
   constexpr int NLA = NAJ + 1;        // activation loads come first in the numbering and in issue order
@@ -403,36 +379,22 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : N) : "memory");
     asm volatile("" : "+v"(as.sc));
   };
-  auto wait_b = [&](auto n_, BRaw& b) {
-    constexpr int N = decltype(n_)::value;
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : N) : "memory");
-#pragma unroll
-    for (int j = 0; j < NBL; ++j) asm volatile("" : "+v"(b.d[j]));
-    asm volatile("" : "+v"(b.sc[0]));
-    if constexpr (STAGE == 1) asm volatile("" : "+v"(b.sc[1]));
-  };
-  // Transposition of a raw set into MFMA operand order: one 8/16-byte load gives a lane the same
-  // K row of 2 (gate/up) or 4 (down) column tiles, while an MFMA wants the 8 K rows of one tile
-  // in consecutive registers.
   // `m1` (all ones or zero, uniform) picks set b1 or b0: one select per register does the choice
   // and the transposition together, with no branch (a branch ends in a block of copies per path).
   auto pick = [&](int& d, int x0, int x1, uint64_t m1) {
     asm volatile("v_cndmask_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x0), "v"(x1), "s"(m1));
   };
   auto unpack_b = [&](const BRaw& b0, const BRaw& b1, uint64_t m1, BFrag& f) {
-    constexpr int NT_LD = (STAGE == 1) ? 2 : 4;  // column tiles per load
     int t[4][8];
 #pragma unroll
     for (int i = 0; i < NBL; ++i)
 #pragma unroll
-      for (int x = 0; x < NT_LD; ++x) pick(t[(i / 8) * NT_LD + x][i % 8], b0.d[i][x], b1.d[i][x], m1);
+      for (int x = 0; x < 4; ++x) pick(t[x][i], b0.d[i][x], b1.d[i][x], m1);
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
       for (int r = 0; r < 8; ++r) f.f[nt][r] = t[nt][r];
-    pick(f.sc[0], b0.sc[0], b1.sc[0], m1);
-    if constexpr (STAGE == 1) pick(f.sc[1], b0.sc[1], b1.sc[1], m1);
-    else f.sc[1] = 0;
+    pick(f.sc, b0.sc, b1.sc, m1);
     asm volatile("s_nop 1");  // the selects feed the first MFMA
   };
   auto store_a = [&](int st, const AStage& r) {
@@ -488,7 +450,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         constexpr int j = decltype(j_)::value;
         constexpr int mt = 2 * gi + j / 4, nt = j % 4;
         constexpr int m = gi * 8 + j;  // MFMA number within the slice
-        mfma_tile<STAGE, mt % 4, nt>(af[cur][j / 4], b, acc[mt][nt], asc[mt / 4]);
+        mfma_tile<mt % 4, nt>(af[cur][j / 4], b, acc[mt][nt], asc[mt / 4]);
         if constexpr (m == 0) {
           // the scalar arithmetic for the addresses of slice ks+2 starts here, behind the first
           // MFMA, instead of ahead of it
@@ -518,7 +480,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     br0.d[j] = 0;
     br1.d[j] = 0;
   });
-  br0.sc[0] = br0.sc[1] = br1.sc[0] = br1.sc[1] = 0;
+  br0.sc = br1.sc = 0;
   as.sc = 0;
   issue_b(0, as, br0, br1, 0);
   issue_b(1, as, br0, br1, 1);
@@ -555,11 +517,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     // [row][q][32 partitions] fp32; then one thread per MX block (8 partitions x 4 q) quantises and
     // writes 32 K-contiguous bytes plus the scale byte.
     float* E = (float*)smem;
-    float bg[2] = {0.f, 0.f}, bu[2] = {0.f, 0.f};
+    // the lane's four partitions within the workgroup's 32: 4*cl + t
+    float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
     if (a.bias) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int64_t p = p0 + 2 * c + t;
+      for (int t = 0; t < 4; ++t) {
+        const int64_t p = p0 + 4 * cl + t;
         const int64_t ig = ((((int64_t)e * a.pI + p) * 2 + 0) * a.nI + tI) * 4 + q;
         const int64_t iu = ((((int64_t)e * a.pI + p) * 2 + 1) * a.nI + tI) * 4 + q;
         if (a.bias_dtype == MOE_DT_BF16) {
@@ -571,7 +534,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         }
       }
     }
-    const int pl0 = 2 * c;  // first of the lane's two partitions within the workgroup's 32
+    const int pl0 = 4 * cl;
     constexpr int NPS = NMT / 4;
     // Clamps as unconditional min/max against +-inf, and the activation kind as a compile-time
     // constant of the pass: a lane evaluates 128 elements here, and per-element decisions made this
@@ -590,17 +553,31 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         static_for<0, 4>([&](auto m_) {
           constexpr int ml = decltype(m_)::value;
           constexpr int mt = ps * 4 + ml;
+          // Lane c < 8 holds gate, lane c + 8 up, of the same four partitions and the same four rows.
+          // The pair splits the rows: the gate lane finishes rows 0,1 of its four, the up lane rows
+          // 2,3; each hands the other the two values it needs (a rotation by 8 within the 16 lanes).
+          // (the accumulators are taken out of their registers here, tile by tile, not all at once
+          // ahead of the passes)
+          asm volatile("" : "+a"(acc[mt][0]), "+a"(acc[mt][1]), "+a"(acc[mt][2]), "+a"(acc[mt][3]));
+          float y[2][4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float y[2];
+          for (int t = 0; t < 4; ++t) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-              const float gg = fminf(fmaxf(acc[mt][t][r] + bg[t], g_lo), g_hi);
-              const float uu = fminf(fmaxf(acc[mt][2 + t][r] + bu[t], u_lo), u_hi);
-              y[t] = act_apply(gg, ACT) * uu;
+            for (int k = 0; k < 2; ++k) {
+              const float mine = hcol ? acc[mt][t][2 + k] : acc[mt][t][k];
+              const float send = hcol ? acc[mt][t][k] : acc[mt][t][2 + k];
+              const float recv = __builtin_bit_cast(
+                  float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+              const float gv = hcol ? recv : mine, uv = hcol ? mine : recv;
+              const float gg = fminf(fmaxf(gv + bg[t], g_lo), g_hi);
+              const float uu = fminf(fmaxf(uv + bu[t], u_lo), u_hi);
+              y[k][t] = act_apply(gg, ACT) * uu;
             }
-            const int rl = ml * 16 + 4 * g + r;
-            *(float2*)(E + rl * MX_EP + q * 32 + pl0) = make_float2(y[0], y[1]);
+          }
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            const int rl = ml * 16 + 4 * g + 2 * hcol + k;
+            *(float4*)(E + rl * MX_EP + q * 32 + pl0) = make_float4(y[k][0], y[k][1], y[k][2], y[k][3]);
           }
         });
         __syncthreads();
