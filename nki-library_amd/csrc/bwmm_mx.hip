@@ -50,7 +50,7 @@ constexpr int MXM = CHUNK_ROWS;                // 256 rows per workgroup
 constexpr int MXROW = 128;                     // LDS pitch of one staged row; 16-byte chunk ch of row r sits in
                                                // slot ch ^ (r & 7), which makes the fragment reads (16 rows x 4
                                                // chunks per instruction) and the staging writes conflict free
-constexpr int MX_NST = 3;                      // depth of the activation ring
+constexpr int MX_NST = 4;                      // depth of the activation ring
 constexpr int MX_SA = MXM * MXROW;             // one A buffer (32 KB)
 constexpr int MX_SS = 4 * 16 * 16;             // one A-scale buffer, [g][c][mt] bytes
 constexpr int MX_EP = 128 + 8;                 // epilogue exchange: floats per row ([q][32 partitions] + pad)
@@ -81,17 +81,39 @@ __device__ __forceinline__ v8i frag_from_lds(const uint8_t* plo, const uint8_t* 
   return r;
 }
 
+// The accumulators live in fixed accumulation registers that only the statements below name: tile
+// (mt, nt) of a wave's 16 x 4 tiles is a[16 mt + 4 nt .. + 3].  They are not C++ values, so the
+// compiler never moves, copies or spills them (it would do so without the wait that a read of an
+// MFMA result needs: it does not know these statements as MFMAs).  Every accumulation register is
+// declared clobbered at both ends of each K slice, so the compiler keeps nothing of its own there.
+#define MX_A10(p) "a" #p "0", "a" #p "1", "a" #p "2", "a" #p "3", "a" #p "4", "a" #p "5", "a" #p "6", "a" #p "7", "a" #p "8", "a" #p "9"
+#define MX_ALL_ACC                                                                                               \
+  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", MX_A10(1), MX_A10(2), MX_A10(3), MX_A10(4),        \
+      MX_A10(5), MX_A10(6), MX_A10(7), MX_A10(8), MX_A10(9), MX_A10(10), MX_A10(11), MX_A10(12), MX_A10(13),     \
+      MX_A10(14), MX_A10(15), MX_A10(16), MX_A10(17), MX_A10(18), MX_A10(19), MX_A10(20), MX_A10(21), MX_A10(22), \
+      MX_A10(23), MX_A10(24), "a250", "a251", "a252", "a253", "a254", "a255"
+__device__ __forceinline__ void acc_fence() { asm volatile("" ::: MX_ALL_ACC); }
+template <int I>
+__device__ __forceinline__ void acc_zero() {
+  asm volatile("v_accvgpr_write_b32 a[%0], 0" : : "n"(I));
+}
+template <int I>
+__device__ __forceinline__ float acc_get() {
+  float x;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(I));
+  return x;
+}
 // One MFMA of row-tile fragment `af` (scale byte OA of `sa`) with column tile NT of `b`, written as
 // an instruction: statements of this kind keep their order, so what the source puts between two
 // MFMAs (a load, an LDS read) is issued between them and runs in the shadow of the first -- with one
 // wave per SIMD nothing else hides it.  op_sel / op_sel_hi carry bit 0 / bit 1 of the two scale
 // byte selectors.
-#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)                                                              \
-  if constexpr (OA == OA_ && OB == OB_)                                                                   \
-    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:" SEL_ " op_sel_hi:" SELHI_ \
-                 : "+a"(c) : "v"(af), "v"(bf), "v"(sa), "v"(sb))
-template <int OA, int OB>
-__device__ __forceinline__ void mfma_asm(v4f& c, const v8i& af, const v8i& bf, int sa, int sb) {
+#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)                                                                  \
+  if constexpr (OA == OA_ && OB == OB_)                                                                       \
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%1], %2, %3, a[%0:%1], %4, %5 op_sel:" SEL_ " op_sel_hi:" SELHI_ \
+                 : : "n"(ACC), "n"(ACC + 3), "v"(af), "v"(bf), "v"(sa), "v"(sb))
+template <int ACC, int OA, int OB>
+__device__ __forceinline__ void mfma_asm(const v8i& af, const v8i& bf, int sa, int sb) {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
   MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
@@ -110,10 +132,6 @@ __device__ __forceinline__ void mfma_asm(v4f& c, const v8i& af, const v8i& bf, i
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
 }
 #undef MX_MFMA_CASE
-template <int OA, int NT>
-__device__ __forceinline__ void mfma_tile(const v8i& af, const BFrag& b, v4f& c, int sa) {
-  mfma_asm<OA, NT>(c, af, b.f[NT], sa, b.sc);
-}
 
 // Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
 // wave-uniform 32-bit byte offset (SGPR), which is exactly the shape of every address in this
@@ -140,21 +158,6 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // in/out operand so that the load updates the variable's register in place.
 __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-}
-// One load into d1 if sel != 0, else into d0.  The choice is made inside the statement, so the
-// compiler sees straight-line code that updates both variables in place (a branch of its own would
-// end in copies of registers whose loads are still in flight).
-__device__ __forceinline__ void ld2_b128(v4i& d0, v4i& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile(
-      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dwordx4 %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
-      ".Lmx%=_1:\n\tbuffer_load_dwordx4 %1, %2, %3, %4 offen\n.Lmx%=_2:"
-      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
-}
-__device__ __forceinline__ void ld2_b32(int& d0, int& d1, int sel, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile(
-      "s_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 .Lmx%=_1\n\tbuffer_load_dword %0, %2, %3, %4 offen\n\ts_branch .Lmx%=_2\n"
-      ".Lmx%=_1:\n\tbuffer_load_dword %1, %2, %3, %4 offen\n.Lmx%=_2:"
-      : "+v"(d0), "+v"(d1) : "v"(voff), "s"(rsrc), "s"(soff), "s"(sel) : "memory", "scc");
 }
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
@@ -289,19 +292,17 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     s_voff = (uint32_t)(g * w_pstride + 4 * c);
   }
 
-  // A K slice's loads, numbered so that they can be issued a few at a time:
-  //   0 .. NAJ-1            activation rows (16 bytes per lane each)
-  //   NAJ                   activation scales
-  //   NAJ+1 .. NAJ+NBL      weights
-  //   NAJ+NBL+1 ..          weight scales
+  // A K slice's loads, numbered in issue order:
+  //   0 .. NAJ-1            activation rows (16 bytes per lane each, straight into the LDS ring)
+  //   NAJ                   activation scales (4 bytes per lane, into a register)
+  //   NAJ+1 .. NAJ+NBL      weights (16 bytes per lane each, into a raw register set)
+  //   NAJ+NBL+1             weight scales
   constexpr int NBL = 8;
-  constexpr int NBS = 1;
-  constexpr int NLOADS = NAJ + 1 + NBL + NBS;
+  constexpr int NLA = NAJ + 1;       // activation loads of a slice
+  constexpr int NLB = NBL + 1;       // weight loads of a slice
+  constexpr int NLOADS = NLA + NLB;
   struct BRaw {
     v4i d[NBL];
-    int sc;
-  };
-  struct AStage {
     int sc;
   };
   const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, 0xffffffffu);
@@ -309,14 +310,13 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // load and kept in scalar registers) + (offset of the slice, computed once per slice): one scalar
   // add per load.  Address arithmetic done per load costs more issue cycles than the MFMAs between
   // two loads take.
-  int w_soff[NBL], s_soff[NBS];
+  int w_soff[NBL];
 #pragma unroll
   for (int i = 0; i < NBL; ++i) {
     const int pr = (i < 4) ? i : (16 + i - 4);
     w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * 4);
   }
-#pragma unroll
-  for (int i = 0; i < NBS; ++i) s_soff[i] = uni(colu);
+  const int s_soff = uni(colu);
   // Everything a slice's loads share: descriptors (of zero records past the end: such a load is out
   // of range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads)
   // and the slice's scalar offsets.
@@ -346,79 +346,60 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
-  auto issue_load = [&](auto idx_, const SliceAddr& sa, AStage& as, BRaw& b, BRaw& b1, int sel) {
+  auto issue_load = [&](auto idx_, const SliceAddr& sa, BRaw& b, int& asc_raw) {
     constexpr int idx = decltype(idx_)::value;
     if constexpr (idx < NAJ) {
       // the wave's 64 lanes fill 8 rows x 128 bytes = 1 KB of the ring stage, in lane order
       ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[idx], sa.ra, sa.a_off);
     } else if constexpr (idx == NAJ) {
-      ld_b32(as.sc, as_voff, sa.ras, sa.as_off);
-    } else if constexpr (idx < NAJ + 1 + NBL) {
-      constexpr int i = idx - NAJ - 1;
-      ld2_b128(b.d[i], b1.d[i], sel, w_voff, sa.rw, w_soff[i] + sa.w_off);
+      // the four scale bytes (K blocks) of row tid
+      ld_b32(asc_raw, as_voff, sa.ras, sa.as_off);
+    } else if constexpr (idx < NLA + NBL) {
+      constexpr int i = idx - NLA;
+      ld_b128(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
     } else {
-      ld2_b32(b.sc, b1.sc, sel, s_voff, sa.rs, s_soff[0] + sa.s_off);
+      ld_b32(b.sc, s_voff, sa.rs, s_soff + sa.s_off);
     }
   };
-  constexpr int NLA = NAJ + 1;        // activation loads come first in the numbering and in issue order
-  constexpr int NLB = NLOADS - NLA;   // weight loads of a slice
-  auto issue_a = [&](int ks, int st, AStage& as, BRaw& b0, BRaw& b1) {
-    const SliceAddr sa = slice_addr(ks, st);
-    static_for<0, NLA>([&](auto i_) { issue_load(i_, sa, as, b0, b1, 0); });
-  };
-  auto issue_b = [&](int ks, AStage& as, BRaw& b0, BRaw& b1, int sel) {
-    const SliceAddr sa = slice_addr(ks, 0);
-    static_for<NLA, NLOADS>([&](auto i_) { issue_load(i_, sa, as, b0, b1, sel); });
-  };
-  // Waits until at most N of this wave's loads are outstanding (they complete in issue order), and
-  // ties the registers that the oldest of them fill to that point.
-  // (The wait itself names no register: an in/out operand may be copied into place before the
-  // statement, i.e. read while its load is still in flight.)
-  auto wait_a = [&](auto n_, AStage& as) {
-    constexpr int N = decltype(n_)::value;
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : N) : "memory");
-    asm volatile("" : "+v"(as.sc));
-  };
-  // `m1` (all ones or zero, uniform) picks set b1 or b0: one select per register does the choice
-  // and the transposition together, with no branch (a branch ends in a block of copies per path).
-  auto pick = [&](int& d, int x0, int x1, uint64_t m1) {
-    asm volatile("v_cndmask_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x0), "v"(x1), "s"(m1));
-  };
-  auto unpack_b = [&](const BRaw& b0, const BRaw& b1, uint64_t m1, BFrag& f) {
-    int t[4][8];
-#pragma unroll
-    for (int i = 0; i < NBL; ++i)
-#pragma unroll
-      for (int x = 0; x < 4; ++x) pick(t[x][i], b0.d[i][x], b1.d[i][x], m1);
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int r = 0; r < 8; ++r) f.f[nt][r] = t[nt][r];
-    pick(f.sc, b0.sc, b1.sc, m1);
-    asm volatile("s_nop 1");  // the selects feed the first MFMA
-  };
-  auto store_a = [&](int st, const AStage& r) {
-    const uint32_t asreg = (uint32_t)r.sc;
-    // scales transposed: row = mt*16 + cc -> [gg][cc][mt]
+  // The MFMA wants a lane's scale byte to be that of row 16*mt + c and K block g, one byte per row
+  // tile: [g][c][mt], so that one 16-byte read gives a lane the scales of all 16 row tiles.  A
+  // thread loads the four scale bytes of row tid and puts them in place.
+  auto scales_to_operand_order = [&](int st, uint32_t raw) {
     uint8_t* sd = sS + st * MX_SS;
     const int mt = tid >> 4, cc = tid & 15;
 #pragma unroll
-    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 16 + mt] = (uint8_t)((asreg >> (8 * gg)) & 0xffu);
+    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 16 + mt] = (uint8_t)((raw >> (8 * gg)) & 0xffu);
   };
 
-  v4f acc[NMT][4];
-  static_for<0, NMT>([&](auto mt) {
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = (v4f){0.f, 0.f, 0.f, 0.f};
-  });
+  acc_fence();
+  static_for<0, NMT * 16>([&](auto i_) { acc_zero<decltype(i_)::value>(); });
 
-  // One K slice: row tiles are multiplied in groups of two; the fragments of the next group are
-  // read from LDS while the current group's eight MFMAs run.  The groups of the first half are each
-  // followed by a share of the loads of slice ks+2.
+  // ---- K loop ---------------------------------------------------------------------------------------
+  // Loads run three slices ahead of the MFMAs (what the memory system delivers is the amount in
+  // flight divided by its latency, and one wave per SIMD has nobody to take over while it waits):
+  // during slice ks the loads of slice ks+3 are issued, one after every second or third MFMA, the
+  // activations into ring stage (ks+3) % 4 (last read in slice ks-1, which every wave left before
+  // the barrier that ended it), the weights into raw register set ks % 3, which was transposed into
+  // MFMA operand order at the top of this slice.  A wave's loads complete in issue order, so a wait
+  // names how many of the most recent ones may still be out.  At the top of slice ks the weights of
+  // slice ks must be in (issued since: all of slices ks+1, ks+2) and, next in line, the activations
+  // of slice ks+1, whose scales are re-ordered during this slice; the barrier at the end of the slice
+  // publishes them to the other waves.  The loop body is written out three times so that the raw
+  // set of a slice is a compile-time choice.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
-  constexpr int NB_AFTER_A = NLB;  // weight loads issued after the last activation load of a slice
-  auto compute = [&](int st, BFrag& b, int ks, int ph, AStage& as, BRaw& b0, BRaw& b1) {
+  BRaw br[3];
+  int asr[3] = {0, 0, 0};  // activation scales as loaded, slice ks in asr[ks % 3]
+  static_for<0, 3>([&](auto u_) {
+    constexpr int u = decltype(u_)::value;
+#pragma unroll
+    for (int j = 0; j < NBL; ++j) br[u].d[j] = 0;
+    br[u].sc = 0;
+  });
+  auto slice = [&](auto u_, int ks, int st) {
+    constexpr int U = decltype(u_)::value;
+    BRaw& braw = br[U];
+    acc_fence();
     const uint8_t* plo = sA + st * MX_SA + rd_lo;
     const uint8_t* phi = sA + st * MX_SA + rd_hi;
     const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
@@ -427,8 +408,28 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
     asm volatile("" ::: "memory");
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLOADS) : "memory");
-    unpack_b(b0, b1, ph ? ~0ull : 0ull, b);
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : 2 * NLOADS - NLA) : "memory");
+    const int st1 = (st + 1) & 3;
+    int& sc_next = asr[(U + 1) % 3];  // activation scales of slice ks+1
+    asm volatile("" : "+v"(sc_next));
+    // (the wait names no register: an in/out operand may be copied into place ahead of its
+    // statement, i.e. read while its load is still in flight; the registers are tied to this point
+    // by statements of their own)
+#pragma unroll
+    for (int j = 0; j < NBL; ++j) asm volatile("" : "+v"(braw.d[j]));
+    asm volatile("" : "+v"(braw.sc));
+    // one 16-byte load gives a lane the same K row of 4 column tiles; an MFMA wants the 8 K rows of
+    // one tile in consecutive registers
+    BFrag b;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      b.f[0][r] = braw.d[r][0];
+      b.f[1][r] = braw.d[r][1];
+      b.f[2][r] = braw.d[r][2];
+      b.f[3][r] = braw.d[r][3];
+    }
+    b.sc = braw.sc;
+    asm volatile("s_nop 1" : "+v"(b.f[0]), "+v"(b.f[1]), "+v"(b.f[2]), "+v"(b.f[3]), "+v"(b.sc));
     SliceAddr sad;
     static_for<0, NG>([&](auto gi_) {
       constexpr int gi = decltype(gi_)::value;
@@ -442,74 +443,60 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       // fragments it returns), so the two fragment sets stay live together and the LDS latency of
       // the next group is covered by this group's eight MFMAs.
       asm volatile("" : "+v"(af[cur][0]), "+v"(af[cur][1]) : : "memory");
-      // Eight MFMAs; after each one, its share of the loads of slice ks+2 (activations first: they
-      // must have arrived by the end of this slice; the weights have until the top of slice ks+2 and
-      // go to the raw set that was transposed at the top of this slice).  One or two loads fit in
-      // the 32 cycles an MFMA occupies the matrix pipe; a burst of them does not.
       static_for<0, 8>([&](auto j_) {
         constexpr int j = decltype(j_)::value;
         constexpr int mt = 2 * gi + j / 4, nt = j % 4;
         constexpr int m = gi * 8 + j;  // MFMA number within the slice
-        mfma_tile<mt % 4, nt>(af[cur][j / 4], b, acc[mt][nt], asc[mt / 4]);
+        mfma_asm<16 * mt + 4 * nt, mt % 4, nt>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
         if constexpr (m == 0) {
-          // the scalar arithmetic for the addresses of slice ks+2 starts here, behind the first
+          // the scalar arithmetic for the addresses of slice ks+3 starts here, behind the first
           // MFMA, instead of ahead of it
-          int ks2 = ks + 2;
-          asm volatile("" : "+s"(ks2));
-          sad = slice_addr(ks2, (st == 0) ? 2 : st - 1);
+          int ks3 = ks + 3;
+          asm volatile("" : "+s"(ks3));
+          sad = slice_addr(ks3, (st + 3) & 3);
         }
-        static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>(
-            [&](auto i_) { issue_load(i_, sad, as, b0, b1, ph); });
+        if constexpr (m == 3) scales_to_operand_order(st1, (uint32_t)sc_next);
+        static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>([&](auto i_) { issue_load(i_, sad, braw, asr[U]); });
       });
     });
+    acc_fence();
+    __syncthreads();
   };
 
-  // ---- main loop ------------------------------------------------------------------------------------
-  // Slice ks multiplies out of ring stage ks % 3 with the weights in `bc`, transposed at its top
-  // from raw set ks % 2.  During its first half the loads of slice ks+2 are issued: the weights
-  // refill that raw set, the activations fill the staging registers, which go to ring stage
-  // (ks+2) % 3 at the end of the slice (that stage was last read in slice ks-1, which every wave
-  // left before the barrier that ended it).  One barrier per slice publishes the stores.  The MFMA
-  // code exists once; only the few instructions that touch a raw set are selected by the parity of
-  // ks (two copies of the MFMA sequence do not survive register allocation).
-  BRaw br0, br1;
-  AStage as;
-  BFrag bc;
-  static_for<0, NBL>([&](auto j_) {
-    constexpr int j = decltype(j_)::value;
-    br0.d[j] = 0;
-    br1.d[j] = 0;
+  // prologue: the first three slices are requested at once; slice 0 needs its activations
+  static_for<0, 3>([&](auto u_) {
+    constexpr int u = decltype(u_)::value;
+    const SliceAddr sa = slice_addr(u, u);
+    static_for<0, NLOADS>([&](auto i_) { issue_load(i_, sa, br[u], asr[u]); });
   });
-  br0.sc = br1.sc = 0;
-  as.sc = 0;
-  issue_b(0, as, br0, br1, 0);
-  issue_b(1, as, br0, br1, 1);
-  // both leading slices in one round trip
-  AStage as1;
-  as1.sc = 0;
-  issue_a(0, 0, as, br0, br1);
-  issue_a(1, 1, as1, br0, br1);
-  wait_a(std::integral_constant<int, 0>{}, as);
-  wait_a(std::integral_constant<int, 0>{}, as1);
-  store_a(0, as);
-  store_a(1, as1);
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + 2 * NLOADS) : "memory");
+  asm volatile("" : "+v"(asr[0]));
+  scales_to_operand_order(0, (uint32_t)asr[0]);
   __syncthreads();
   int st = 0;
+  int ks = 0;
 #pragma clang loop unroll(disable)
-  for (int ks = 0; ks < nks; ++ks) {
-    const int ph = ks & 1;
-    // weights of this slice: requested two slices ago; everything issued since is one slice's loads
-    compute(st, bc, ks, ph, as, br0, br1);
-    const int st2 = (st == 0) ? 2 : st - 1;  // (st + 2) % 3
-    // activations of slice ks+2: requested in this slice, NB_AFTER_A weight loads ago
-    wait_a(std::integral_constant<int, NB_AFTER_A>{}, as);
-    store_a(st2, as);  // past the end: zeros into a stage that nobody reads any more
-    __syncthreads();
-    st = (st == 2) ? 0 : st + 1;
+  for (; ks + 3 <= nks; ks += 3) {
+    slice(std::integral_constant<int, 0>{}, ks, st);
+    slice(std::integral_constant<int, 1>{}, ks + 1, (st + 1) & 3);
+    slice(std::integral_constant<int, 2>{}, ks + 2, (st + 2) & 3);
+    st = (st + 3) & 3;
   }
-  // the last MFMAs are still in the pipe: as instructions of unknown kind to the compiler, it adds
-  // no wait between them and the first read of an accumulator
+  if (ks < nks) {
+    slice(std::integral_constant<int, 0>{}, ks, st);
+    if (ks + 1 < nks) slice(std::integral_constant<int, 1>{}, ks + 1, (st + 1) & 3);
+  }
+  // the last MFMAs are still in the pipe, and nothing but the distance in instructions separates
+  // them from the first read of an accumulator
   asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // The loads of the slices past the end are never used, but they do arrive (as zeros): the registers
+  // they were aimed at stay reserved until the wait above has passed.
+#pragma unroll
+  for (int u = 0; u < 3; ++u) {
+#pragma unroll
+    for (int j = 0; j < NBL; ++j) asm volatile("" : : "v"(br[u].d[j]));
+    asm volatile("" : : "v"(br[u].sc), "v"(asr[u]));
+  }
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
@@ -556,16 +543,19 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           // Lane c < 8 holds gate, lane c + 8 up, of the same four partitions and the same four rows.
           // The pair splits the rows: the gate lane finishes rows 0,1 of its four, the up lane rows
           // 2,3; each hands the other the two values it needs (a rotation by 8 within the 16 lanes).
-          // (the accumulators are taken out of their registers here, tile by tile, not all at once
-          // ahead of the passes)
-          asm volatile("" : "+a"(acc[mt][0]), "+a"(acc[mt][1]), "+a"(acc[mt][2]), "+a"(acc[mt][3]));
+          float av[4][4];  // [column tile][row]
+          static_for<0, 16>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            av[i / 4][i % 4] = acc_get<16 * mt + i>();
+          });
           float y[2][4];
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
-              const float mine = hcol ? acc[mt][t][2 + k] : acc[mt][t][k];
-              const float send = hcol ? acc[mt][t][k] : acc[mt][t][2 + k];
+              const float lo = av[t][k], hi = av[t][2 + k];
+              const float mine = hcol ? hi : lo;
+              const float send = hcol ? lo : hi;
               const float recv = __builtin_bit_cast(
                   float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
               const float gv = hcol ? recv : mine, uv = hcol ? mine : recv;
@@ -639,6 +629,11 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     typedef float v2f __attribute__((ext_vector_type(2)));
     static_for<0, NMT>([&](auto mt_) {
       constexpr int mt = decltype(mt_)::value;
+      float av[4][4];  // [column tile][row]
+      static_for<0, 16>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        av[i / 4][i % 4] = acc_get<16 * mt + i>();
+      });
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = mt * 16 + 4 * g + r;
@@ -646,7 +641,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         v2i o;
 #pragma unroll
         for (int t = 0; t < 4; t += 2) {
-          const v2f d = {(acc[mt][t][r] + bd[t]) * af, (acc[mt][t + 1][r] + bd[t + 1]) * af};
+          const v2f d = {(av[t][r] + bd[t]) * af, (av[t + 1][r] + bd[t + 1]) * af};
           o[t >> 1] = __builtin_bit_cast(int, __builtin_convertvector(d, v2bf));
         }
         st_b64(o, d_voff, rd, (mt * 16 + r) * rowb);
