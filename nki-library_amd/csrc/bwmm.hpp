@@ -43,6 +43,7 @@ struct MxArgs {
   int64_t a_stride;
   const uint8_t* A_scale;  // E8M0 [rows, a_scale_stride]
   int64_t a_scale_stride;
+  int64_t a_rows;          // rows of A and A_scale
   const uint32_t* W;       // x4 weights in the reference layout
   const uint8_t* W_scale;
   const void* bias;

@@ -156,8 +156,13 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // for the set that was only just requested.  Loads the compiler cannot see get no waits from it;
 // the waits are placed by hand where the data is first used (vm_wait).  The destination is an
 // in/out operand so that the load updates the variable's register in place.
+// NT: non-temporal, for data that nobody will ask the L2 for again.
+template <bool NT>
 __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  if constexpr (NT)
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  else
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
@@ -167,13 +172,20 @@ __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
+typedef int v3i __attribute__((ext_vector_type(3)));
+__device__ __forceinline__ void ld_b96(v3i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_load_dwordx3 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
 __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 // NMT = number of 16-row tiles this instantiation multiplies (the chunk has at most NMT*16 rows).
 // Keeping it a compile-time constant keeps the K loop free of branches around the MFMAs.
-template <int STAGE, int NMT>
+// LASTUSE: this chunk is the last one of its expert, so its weights are streamed past the L2 (which
+// then keeps the activation tiles that the sibling workgroups share); an earlier chunk loads them
+// normally, for the chunk after it to find.
+template <int STAGE, int NMT, bool LASTUSE>
 __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
                                              int64_t slot0, int xt) {
   uint8_t* sA = smem;
@@ -294,7 +306,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 
   // A K slice's loads, numbered in issue order:
   //   0 .. NAJ-1            activation rows (16 bytes per lane each, straight into the LDS ring)
-  //   NAJ                   activation scales (4 bytes per lane, into a register)
+  //   NAJ                   activation scales of three slices (12 bytes per lane, into registers), only in
+  //                         the first slice of every three
   //   NAJ+1 .. NAJ+NBL      weights (16 bytes per lane each, into a raw register set)
   //   NAJ+NBL+1             weight scales
   constexpr int NBL = 8;
@@ -305,7 +318,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     v4i d[NBL];
     int sc;
   };
-  const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, 0xffffffffu);
+  const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_rows * a.a_scale_stride));
   // Scalar byte offset of a weight load = (offset of its row and column within the slice, fixed per
   // load and kept in scalar registers) + (offset of the slice, computed once per slice): one scalar
   // add per load.  Address arithmetic done per load costs more issue cycles than the MFMAs between
@@ -346,24 +359,26 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
-  auto issue_load = [&](auto idx_, const SliceAddr& sa, BRaw& b, int& asc_raw) {
+  auto issue_load = [&](auto idx_, const SliceAddr& sa, BRaw& b, v3i& asc_raw, auto with_scales_) {
     constexpr int idx = decltype(idx_)::value;
     if constexpr (idx < NAJ) {
       // the wave's 64 lanes fill 8 rows x 128 bytes = 1 KB of the ring stage, in lane order
       ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[idx], sa.ra, sa.a_off);
     } else if constexpr (idx == NAJ) {
-      // the four scale bytes (K blocks) of row tid
-      ld_b32(asc_raw, as_voff, sa.ras, sa.as_off);
+      // the four scale bytes (K blocks) of row tid, for this slice and the two after it: a lane's
+      // dwords sit in different cache lines, so this load costs the memory pipeline as many
+      // requests as all the activation rows of a slice together -- hence one in three slices
+      if constexpr (decltype(with_scales_)::value) ld_b96(asc_raw, as_voff, sa.ras, sa.as_off);
     } else if constexpr (idx < NLA + NBL) {
       constexpr int i = idx - NLA;
-      ld_b128(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
+      ld_b128<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
     } else {
       ld_b32(b.sc, s_voff, sa.rs, s_soff + sa.s_off);
     }
   };
   // The MFMA wants a lane's scale byte to be that of row 16*mt + c and K block g, one byte per row
   // tile: [g][c][mt], so that one 16-byte read gives a lane the scales of all 16 row tiles.  A
-  // thread loads the four scale bytes of row tid and puts them in place.
+  // thread loads the scale bytes of row tid and puts them in place.
   auto scales_to_operand_order = [&](int st, uint32_t raw) {
     uint8_t* sd = sS + st * MX_SS;
     const int mt = tid >> 4, cc = tid & 15;
@@ -389,7 +404,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
   BRaw br[3];
-  int asr[3] = {0, 0, 0};  // activation scales as loaded, slice ks in asr[ks % 3]
+  v3i asr3 = {0, 0, 0};  // activation scales as loaded, of the three slices of a turn of the loop
   static_for<0, 3>([&](auto u_) {
     constexpr int u = decltype(u_)::value;
 #pragma unroll
@@ -408,10 +423,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
     asm volatile("" ::: "memory");
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : 2 * NLOADS - NLA) : "memory");
-    const int st1 = (st + 1) & 3;
-    int& sc_next = asr[(U + 1) % 3];  // activation scales of slice ks+1
-    asm volatile("" : "+v"(sc_next));
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + NLOADS - 1) : "memory");
+    if constexpr (U == 2) asm volatile("" : "+v"(asr3));  // activation scales of slices ks+1 .. ks+3
     // (the wait names no register: an in/out operand may be copied into place ahead of its
     // statement, i.e. read while its load is still in flight; the registers are tied to this point
     // by statements of their own)
@@ -455,8 +468,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           asm volatile("" : "+s"(ks3));
           sad = slice_addr(ks3, (st + 3) & 3);
         }
-        if constexpr (m == 3) scales_to_operand_order(st1, (uint32_t)sc_next);
-        static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>([&](auto i_) { issue_load(i_, sad, braw, asr[U]); });
+        if constexpr (U == 2 && m >= 3 && m <= 5) scales_to_operand_order((st + m - 2) & 3, (uint32_t)asr3[m - 3]);
+        static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>([&](auto i_) { issue_load(i_, sad, braw, asr3, std::integral_constant<bool, U == 0>{}); });
       });
     });
     acc_fence();
@@ -467,11 +480,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   static_for<0, 3>([&](auto u_) {
     constexpr int u = decltype(u_)::value;
     const SliceAddr sa = slice_addr(u, u);
-    static_for<0, NLOADS>([&](auto i_) { issue_load(i_, sa, br[u], asr[u]); });
+    static_for<0, NLOADS>([&](auto i_) { issue_load(i_, sa, br[u], asr3, std::integral_constant<bool, u == 0>{}); });
   });
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + 2 * NLOADS) : "memory");
-  asm volatile("" : "+v"(asr[0]));
-  scales_to_operand_order(0, (uint32_t)asr[0]);
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + 2 * (NLOADS - 1)) : "memory");
+  asm volatile("" : "+v"(asr3));
+#pragma unroll
+  for (int j = 0; j < 3; ++j) scales_to_operand_order(j, (uint32_t)asr3[j]);
   __syncthreads();
   int st = 0;
   int ks = 0;
@@ -495,8 +509,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   for (int u = 0; u < 3; ++u) {
 #pragma unroll
     for (int j = 0; j < NBL; ++j) asm volatile("" : : "v"(br[u].d[j]));
-    asm volatile("" : : "v"(br[u].sc), "v"(asr[u]));
+    asm volatile("" : : "v"(br[u].sc));
   }
+  asm volatile("" : : "v"(asr3));
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
@@ -671,9 +686,16 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int nrows = __builtin_amdgcn_readfirstlane(a.chunk_rows[chunk]);
   const int e = __builtin_amdgcn_readfirstlane(a.chunk_expert[chunk]);
   const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
-  if (nrows <= 64) mx_gemm_body<STAGE, 4>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  else if (nrows <= 128) mx_gemm_body<STAGE, 8>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  else mx_gemm_body<STAGE, 16>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  const bool last = (chunk + 1 >= n_chunks) || (__builtin_amdgcn_readfirstlane(a.chunk_expert[chunk + 1]) != e);
+  if (last) {
+    if (nrows <= 64) mx_gemm_body<STAGE, 4, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 128) mx_gemm_body<STAGE, 8, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else mx_gemm_body<STAGE, 16, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  } else {
+    if (nrows <= 64) mx_gemm_body<STAGE, 4, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 128) mx_gemm_body<STAGE, 8, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else mx_gemm_body<STAGE, 16, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  }
 }
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {

@@ -234,6 +234,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     if (mx_fast) {
       MxArgs m1 = m;
       m1.A = g1.A; m1.a_stride = g1.a_stride; m1.A_scale = g1.A_scale; m1.a_scale_stride = g1.a_scale_stride;
+      m1.a_rows = n_real;
       m1.W = (const uint32_t*)a->gate_up_proj_weight; m1.W_scale = (const uint8_t*)a->gate_up_proj_scale;
       m1.bias = a->gate_and_up_proj_bias;
       rc = launch_mx_gemm(1, m1, (unsigned)(p.nI * 4), gyc, s);
@@ -250,6 +251,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     if (mx_fast) {
       MxArgs m2 = m;
       m2.A = ws + p.yq; m2.a_stride = p.Iw; m2.A_scale = ws + p.ys; m2.a_scale_stride = p.Iw / 32;
+      m2.a_rows = a->N * a->B;
       m2.W = (const uint32_t*)a->down_proj_weight; m2.W_scale = (const uint8_t*)a->down_proj_scale;
       m2.bias = a->down_proj_bias;
       rc = launch_mx_gemm(2, m2, (unsigned)(a->H / 256), gyc, s);
