@@ -46,18 +46,29 @@
 namespace moe {
 
 constexpr int MXT = 256;                       // threads
-constexpr int MXM = CHUNK_ROWS;                // 256 rows per workgroup
+constexpr int MX_ROWS_MAX = CHUNK_ROWS_MAX;    // rows of the largest chunk (320)
 constexpr int MXROW = 128;                     // LDS pitch of one staged row; 16-byte chunk ch of row r sits in
                                                // slot ch ^ (r & 7), which makes the fragment reads (16 rows x 4
                                                // chunks per instruction) and the staging writes conflict free
-constexpr int MX_NST = 4;                      // depth of the activation ring
-constexpr int MX_SA = MXM * MXROW;             // one A buffer (32 KB)
-constexpr int MX_SS = 4 * 16 * 16;             // one A-scale buffer, [g][c][mt] bytes
 constexpr int MX_EP = 128 + 8;                 // epilogue exchange: floats per row ([q][32 partitions] + pad)
-constexpr int MX_LDS_LOOP = MX_NST * (MX_SA + MX_SS);
+// Per variant (NMT row tiles): how many slices the loads run ahead, the ring of activation stages, and
+// the bytes of one stage.  Chunks of up to 256 rows: 3 slices ahead, 4 stages of 256 rows.  Chunks of
+// 257..320 rows (an expert's usual load plus a small excess, which would otherwise cost a second pass
+// over the expert's weights): 2 slices ahead, 3 stages of 320 rows -- the 64 extra accumulators
+// live in ordinary registers, which leaves room for two raw weight sets, not three.
+template <int NMT>
+struct MxCfg {
+  static constexpr int D = NMT > 16 ? 2 : 3;          // slices between a load and its use
+  static constexpr int RING = D + 1;                  // activation stages
+  static constexpr int ROWS = NMT > 16 ? 320 : 256;   // rows of a stage
+  static constexpr int SA = ROWS * MXROW;             // bytes of a stage's rows
+  static constexpr int SSP = NMT > 16 ? 32 : 16;      // scale bytes per (K block, row within tile): one per row tile
+  static constexpr int SS = 64 * SSP;                 // bytes of a stage's scales, [g][c][mt]
+  static constexpr int LDS = RING * (SA + SS);
+};
+constexpr int MX_LDS_LOOP = MxCfg<16>::LDS > MxCfg<20>::LDS ? MxCfg<16>::LDS : MxCfg<20>::LDS;
 constexpr int MX_LDS_EPI = 64 * MX_EP * 4;
 constexpr int MX_LDS = MX_LDS_EPI > MX_LDS_LOOP ? MX_LDS_EPI : MX_LDS_LOOP;
-static_assert(MXM == 256, "the kernel is written for 256-row chunks");
 
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -132,6 +143,31 @@ __device__ __forceinline__ void mfma_asm(const v8i& af, const v8i& bf, int sa, i
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
 }
 #undef MX_MFMA_CASE
+// The same with the accumulator tile in ordinary registers (row tiles 16..19 of a 320-row chunk).
+#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)                                                                  \
+  if constexpr (OA == OA_ && OB == OB_)                                                                       \
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:" SEL_ " op_sel_hi:" SELHI_ \
+                 : "+v"(c) : "v"(af), "v"(bf), "v"(sa), "v"(sb))
+template <int OA, int OB>
+__device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const v8i& bf, int sa, int sb) {
+  MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
+  MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
+  MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
+  MX_MFMA_CASE(3, 0, "[1,0,0]", "[1,0,0]");
+  MX_MFMA_CASE(0, 1, "[0,1,0]", "[0,0,0]");
+  MX_MFMA_CASE(1, 1, "[1,1,0]", "[0,0,0]");
+  MX_MFMA_CASE(2, 1, "[0,1,0]", "[1,0,0]");
+  MX_MFMA_CASE(3, 1, "[1,1,0]", "[1,0,0]");
+  MX_MFMA_CASE(0, 2, "[0,0,0]", "[0,1,0]");
+  MX_MFMA_CASE(1, 2, "[1,0,0]", "[0,1,0]");
+  MX_MFMA_CASE(2, 2, "[0,0,0]", "[1,1,0]");
+  MX_MFMA_CASE(3, 2, "[1,0,0]", "[1,1,0]");
+  MX_MFMA_CASE(0, 3, "[0,1,0]", "[0,1,0]");
+  MX_MFMA_CASE(1, 3, "[1,1,0]", "[0,1,0]");
+  MX_MFMA_CASE(2, 3, "[0,1,0]", "[1,1,0]");
+  MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
+}
+#undef MX_MFMA_CASE
 
 // Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
 // wave-uniform 32-bit byte offset (SGPR), which is exactly the shape of every address in this
@@ -173,8 +209,11 @@ __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v
                : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
 typedef int v3i __attribute__((ext_vector_type(3)));
-__device__ __forceinline__ void ld_b96(v3i& d, uint32_t voff, const v4i& rsrc, int soff) {
+__device__ __forceinline__ void ld_dwords(v3i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dwordx3 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+__device__ __forceinline__ void ld_dwords(v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
@@ -188,8 +227,13 @@ __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, i
 template <int STAGE, int NMT, bool LASTUSE>
 __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
                                              int64_t slot0, int xt) {
+  using Cfg = MxCfg<NMT>;
+  constexpr int D = Cfg::D, RING = Cfg::RING, SA = Cfg::SA, SS = Cfg::SS, SSP = Cfg::SSP;
+  constexpr bool BIG = NMT > 16;  // row tiles 16.. accumulate in ordinary registers
   uint8_t* sA = smem;
-  uint8_t* sS = smem + MX_NST * MX_SA;
+  uint8_t* sS = smem + RING * SA;
+  // ring arithmetic: x in [0, 2 RING)
+  auto wrapst = [](int x) { return (RING == 4) ? (x & 3) : ((x >= RING) ? x - RING : x); };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -212,19 +256,19 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   const int q = w;
 
   // ---- rows: token ids, affinities ---------------------------------------------------------------
-  {
+  for (int r = tid; r < NMT * 16; r += MXT) {
     int id = -1;
-    if (tid < nrows) {
-      id = a.tp2id[slot0 + tid];
+    if (r < nrows) {
+      id = a.tp2id[slot0 + r];
       if (id < 0 || id >= a.n_real) id = -1;
     }
-    s_tok[tid] = id;
+    s_tok[r] = id;
     if (STAGE == 2) {
       float af = 0.f;
       if (id >= 0 && a.aff)
         af = (a.aff_dtype == MOE_DT_BF16) ? bf16_bits_to_f32(((const uint16_t*)a.aff)[(int64_t)id * a.E + e])
                                           : ((const float*)a.aff)[(int64_t)id * a.E + e];
-      s_aff[tid] = af;
+      s_aff[r] = af;
     }
   }
   __syncthreads();
@@ -251,14 +295,20 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     }
     a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)((ach ^ (arow0 & 7)) * 16);
   }
-  // A scales: thread covers row tid
-  uint32_t as_voff;
-  if (STAGE == 1) {
-    const int tok = s_tok[tid];
-    as_voff = ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
-  } else {
-    as_voff = (uint32_t)(slot0 + ((tid < nrows) ? tid : (nrows - 1))) * (uint32_t)a.a_scale_stride;
-  }
+  // A scales: thread covers row tid (and, in a chunk of more than 256 rows, row 256 + tid % 64: every
+  // wave issues that load so that all waves count the same loads, the first wave's is used)
+  auto scale_row_off = [&](int row) {
+    if (STAGE == 1) {
+      const int tok = s_tok[row];
+      return ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
+    }
+    return (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1))) * (uint32_t)a.a_scale_stride;
+  };
+  const uint32_t as_voff = scale_row_off(tid);
+  const uint32_t as_voff2 = BIG ? scale_row_off(256 + (tid & 63)) : 0u;
+  // where the scales of row 256 + tid go: the other waves' copies land in a row tile that does not
+  // exist (no branch inside the K loop: values that cross one stop being known as uniform)
+  const int row_hi = (tid < 64) ? 256 + tid : 31 * 16 + (tid & 15);
 
   // ---- K schedule -----------------------------------------------------------------------------------
   // stage 1: ks -> (H tile ks>>2, partition group ks&3), all slices full.
@@ -306,14 +356,16 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 
   // A K slice's loads, numbered in issue order:
   //   0 .. NAJ-1            activation rows (16 bytes per lane each, straight into the LDS ring)
-  //   NAJ                   activation scales of three slices (12 bytes per lane, into registers), only in
-  //                         the first slice of every three
-  //   NAJ+1 .. NAJ+NBL      weights (16 bytes per lane each, into a raw register set)
-  //   NAJ+NBL+1             weight scales
+  //   NAJ .. NAJ+NSC-1      activation scales of D slices (4 D bytes per lane, into registers), only in the
+  //                         first slice of every D
+  //   then NBL              weights (16 bytes per lane each, into a raw register set)
+  //   then 1                weight scales
   constexpr int NBL = 8;
-  constexpr int NLA = NAJ + 1;       // activation loads of a slice
-  constexpr int NLB = NBL + 1;       // weight loads of a slice
-  constexpr int NLOADS = NLA + NLB;
+  constexpr int NSC = BIG ? 2 : 1;
+  constexpr int NLB = NBL + 1;              // weight loads of a slice
+  constexpr int N1 = NAJ + NLB;             // loads of a slice that carries no activation scales
+  constexpr int N0 = N1 + NSC;              // loads of one that does
+  typedef typename std::conditional<D == 3, v3i, v2i>::type ScaleRegs;
   struct BRaw {
     v4i d[NBL];
     int sc;
@@ -341,7 +393,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   const uint32_t lds_ring = (uint32_t)(uintptr_t)sA;
   auto slice_addr = [&](int ks, int st) {
     SliceAddr r;
-    r.lds_a = uni((int)(lds_ring + (uint32_t)st * MX_SA));
+    r.lds_a = uni((int)(lds_ring + (uint32_t)st * SA));
     const int live = (ks < nks) ? -1 : 0;
     auto sel = [&](const v4i& d) {
       v4i x;
@@ -359,18 +411,21 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
-  auto issue_load = [&](auto idx_, const SliceAddr& sa, BRaw& b, v3i& asc_raw, auto with_scales_) {
+  auto issue_load = [&](auto idx_, const SliceAddr& sa, BRaw& b, ScaleRegs& sc0, ScaleRegs& sc1, auto with_scales_) {
     constexpr int idx = decltype(idx_)::value;
     if constexpr (idx < NAJ) {
       // the wave's 64 lanes fill 8 rows x 128 bytes = 1 KB of the ring stage, in lane order
       ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[idx], sa.ra, sa.a_off);
-    } else if constexpr (idx == NAJ) {
-      // the four scale bytes (K blocks) of row tid, for this slice and the two after it: a lane's
+    } else if constexpr (idx < NAJ + NSC) {
+      // the four scale bytes (K blocks) of a row, for this slice and the D-1 after it: a lane's
       // dwords sit in different cache lines, so this load costs the memory pipeline as many
-      // requests as all the activation rows of a slice together -- hence one in three slices
-      if constexpr (decltype(with_scales_)::value) ld_b96(asc_raw, as_voff, sa.ras, sa.as_off);
-    } else if constexpr (idx < NLA + NBL) {
-      constexpr int i = idx - NLA;
+      // requests as all the activation rows of a slice together -- hence one in D slices
+      if constexpr (decltype(with_scales_)::value) {
+        if constexpr (idx == NAJ) ld_dwords(sc0, as_voff, sa.ras, sa.as_off);
+        else ld_dwords(sc1, as_voff2, sa.ras, sa.as_off);
+      }
+    } else if constexpr (idx < NAJ + NSC + NBL) {
+      constexpr int i = idx - NAJ - NSC;
       ld_b128<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
     } else {
       ld_b32(b.sc, s_voff, sa.rs, s_soff + sa.s_off);
@@ -379,33 +434,39 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // The MFMA wants a lane's scale byte to be that of row 16*mt + c and K block g, one byte per row
   // tile: [g][c][mt], so that one 16-byte read gives a lane the scales of all 16 row tiles.  A
   // thread loads the scale bytes of row tid and puts them in place.
-  auto scales_to_operand_order = [&](int st, uint32_t raw) {
-    uint8_t* sd = sS + st * MX_SS;
-    const int mt = tid >> 4, cc = tid & 15;
+  auto scales_to_operand_order = [&](int st, uint32_t raw, int row) {
+    uint8_t* sd = sS + st * SS;
+    const int mt = row >> 4, cc = row & 15;
 #pragma unroll
-    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * 16 + mt] = (uint8_t)((raw >> (8 * gg)) & 0xffu);
+    for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * SSP + mt] = (uint8_t)((raw >> (8 * gg)) & 0xffu);
   };
 
   acc_fence();
-  static_for<0, NMT * 16>([&](auto i_) { acc_zero<decltype(i_)::value>(); });
+  static_for<0, (BIG ? 16 : NMT) * 16>([&](auto i_) { acc_zero<decltype(i_)::value>(); });
+  v4f accv[4][4];  // row tiles 16..19
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) accv[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   // ---- K loop ---------------------------------------------------------------------------------------
-  // Loads run three slices ahead of the MFMAs (what the memory system delivers is the amount in
-  // flight divided by its latency, and one wave per SIMD has nobody to take over while it waits):
-  // during slice ks the loads of slice ks+3 are issued, one after every second or third MFMA, the
-  // activations into ring stage (ks+3) % 4 (last read in slice ks-1, which every wave left before
-  // the barrier that ended it), the weights into raw register set ks % 3, which was transposed into
+  // Loads run D slices ahead of the MFMAs (what the memory system delivers is the amount in flight
+  // divided by its latency, and one wave per SIMD has nobody to take over while it waits): during
+  // slice ks the loads of slice ks+D are issued, one after every second or third MFMA, the
+  // activations into ring stage (ks+D) % RING (last read in slice ks-1, which every wave left before
+  // the barrier that ended it), the weights into raw register set ks % D, which was transposed into
   // MFMA operand order at the top of this slice.  A wave's loads complete in issue order, so a wait
   // names how many of the most recent ones may still be out.  At the top of slice ks the weights of
-  // slice ks must be in (issued since: all of slices ks+1, ks+2) and, next in line, the activations
-  // of slice ks+1, whose scales are re-ordered during this slice; the barrier at the end of the slice
-  // publishes them to the other waves.  The loop body is written out three times so that the raw
-  // set of a slice is a compile-time choice.
+  // slice ks must be in and, next in line, the activations of slice ks+1 (issued since: the weights
+  // of slice ks+1 and all of the slices after it); the barrier at the end of the slice publishes
+  // them to the other waves.  The activation scales of D slices arrive together in the first slice
+  // of every D and are re-ordered into the stages of the next D slices during the last.  The loop
+  // body is written out D times so that the raw set of a slice is a compile-time choice.
   const int rd_lo = c * MXROW + ((g ^ (c & 7)) * 16), rd_hi = c * MXROW + (((g + 4) ^ (c & 7)) * 16);
   constexpr int NG = NMT / 2;
-  BRaw br[3];
-  v3i asr3 = {0, 0, 0};  // activation scales as loaded, of the three slices of a turn of the loop
-  static_for<0, 3>([&](auto u_) {
+  BRaw br[D];
+  ScaleRegs asr = 0, asr2 = 0;  // activation scales as loaded: row tid, row 256 + tid % 64
+  static_for<0, D>([&](auto u_) {
     constexpr int u = decltype(u_)::value;
 #pragma unroll
     for (int j = 0; j < NBL; ++j) br[u].d[j] = 0;
@@ -415,16 +476,21 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     constexpr int U = decltype(u_)::value;
     BRaw& braw = br[U];
     acc_fence();
-    const uint8_t* plo = sA + st * MX_SA + rd_lo;
-    const uint8_t* phi = sA + st * MX_SA + rd_hi;
-    const v4i asc = *(const v4i*)(sS + st * MX_SS + (g * 16 + c) * 16);
+    const uint8_t* plo = sA + st * SA + rd_lo;
+    const uint8_t* phi = sA + st * SA + rd_hi;
+    const v4i asc = *(const v4i*)(sS + st * SS + (g * 16 + c) * SSP);
+    int asc_hi = 0;
+    if constexpr (BIG) asc_hi = *(const int*)(sS + st * SS + (g * 16 + c) * SSP + 16);
     // first fragments of this slice: in flight while the weights are transposed
     v8i af[2][2];
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
     asm volatile("" ::: "memory");
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + NLOADS - 1) : "memory");
-    if constexpr (U == 2) asm volatile("" : "+v"(asr3));  // activation scales of slices ks+1 .. ks+3
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + (D - 2) * N1) : "memory");
+    if constexpr (U == D - 1) {  // activation scales of slices ks+1 .. ks+D
+      asm volatile("" : "+v"(asr));
+      if constexpr (BIG) asm volatile("" : "+v"(asr2));
+    }
     // (the wait names no register: an in/out operand may be copied into place ahead of its
     // statement, i.e. read while its load is still in flight; the registers are tied to this point
     // by statements of their own)
@@ -460,58 +526,69 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         constexpr int j = decltype(j_)::value;
         constexpr int mt = 2 * gi + j / 4, nt = j % 4;
         constexpr int m = gi * 8 + j;  // MFMA number within the slice
-        mfma_asm<16 * mt + 4 * nt, mt % 4, nt>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
+        if constexpr (mt < 16)
+          mfma_asm<16 * mt + 4 * nt, mt % 4, nt>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
+        else
+          mfma_asm_v<mt % 4, nt>(accv[mt - 16][nt], af[cur][j / 4], b.f[nt], asc_hi, b.sc);
         if constexpr (m == 0) {
-          // the scalar arithmetic for the addresses of slice ks+3 starts here, behind the first
+          // the scalar arithmetic for the addresses of slice ks+D starts here, behind the first
           // MFMA, instead of ahead of it
-          int ks3 = ks + 3;
-          asm volatile("" : "+s"(ks3));
-          sad = slice_addr(ks3, (st + 3) & 3);
+          int ksd = ks + D;
+          asm volatile("" : "+s"(ksd));
+          sad = slice_addr(ksd, wrapst(st + D));
         }
-        if constexpr (U == 2 && m >= 3 && m <= 5) scales_to_operand_order((st + m - 2) & 3, (uint32_t)asr3[m - 3]);
-        static_for<m * NLOADS / (8 * NG), (m + 1) * NLOADS / (8 * NG)>([&](auto i_) { issue_load(i_, sad, braw, asr3, std::integral_constant<bool, U == 0>{}); });
+        if constexpr (U == D - 1 && m >= 3 && m < 3 + D) {
+          scales_to_operand_order(wrapst(st + m - 2), (uint32_t)asr[m - 3], tid);
+          if constexpr (BIG) scales_to_operand_order(wrapst(st + m - 2), (uint32_t)asr2[m - 3], row_hi);
+        }
+        static_for<m * N0 / (8 * NG), (m + 1) * N0 / (8 * NG)>(
+            [&](auto i_) { issue_load(i_, sad, braw, asr, asr2, std::integral_constant<bool, U == 0>{}); });
       });
     });
+    // (accumulators in ordinary registers are C++ values: should the compiler copy one where paths
+    // join, the MFMA that wrote it has left the pipe)
+    if constexpr (BIG) asm volatile("s_nop 15");
     acc_fence();
     __syncthreads();
   };
 
-  // prologue: the first three slices are requested at once; slice 0 needs its activations
-  static_for<0, 3>([&](auto u_) {
+  // prologue: the first D slices are requested at once; slice 0 needs its activations
+  static_for<0, D>([&](auto u_) {
     constexpr int u = decltype(u_)::value;
     const SliceAddr sa = slice_addr(u, u);
-    static_for<0, NLOADS>([&](auto i_) { issue_load(i_, sa, br[u], asr3, std::integral_constant<bool, u == 0>{}); });
+    static_for<0, N0>([&](auto i_) { issue_load(i_, sa, br[u], asr, asr2, std::integral_constant<bool, u == 0>{}); });
   });
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + 2 * (NLOADS - 1)) : "memory");
-  asm volatile("" : "+v"(asr3));
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + (D - 1) * N1) : "memory");
+  asm volatile("" : "+v"(asr));
+  if constexpr (BIG) asm volatile("" : "+v"(asr2));
 #pragma unroll
-  for (int j = 0; j < 3; ++j) scales_to_operand_order(j, (uint32_t)asr3[j]);
+  for (int j = 0; j < D; ++j) {
+    scales_to_operand_order(j, (uint32_t)asr[j], tid);
+    if constexpr (BIG) scales_to_operand_order(j, (uint32_t)asr2[j], row_hi);
+  }
   __syncthreads();
   int st = 0;
   int ks = 0;
 #pragma clang loop unroll(disable)
-  for (; ks + 3 <= nks; ks += 3) {
-    slice(std::integral_constant<int, 0>{}, ks, st);
-    slice(std::integral_constant<int, 1>{}, ks + 1, (st + 1) & 3);
-    slice(std::integral_constant<int, 2>{}, ks + 2, (st + 2) & 3);
-    st = (st + 3) & 3;
+  for (; ks + D <= nks; ks += D) {
+    static_for<0, D>([&](auto u_) { slice(u_, ks + decltype(u_)::value, wrapst(st + decltype(u_)::value)); });
+    st = wrapst(st + D);
   }
-  if (ks < nks) {
-    slice(std::integral_constant<int, 0>{}, ks, st);
-    if (ks + 1 < nks) slice(std::integral_constant<int, 1>{}, ks + 1, (st + 1) & 3);
-  }
+  static_for<0, D - 1>([&](auto u_) {
+    if (ks + decltype(u_)::value < nks) slice(u_, ks + decltype(u_)::value, wrapst(st + decltype(u_)::value));
+  });
   // the last MFMAs are still in the pipe, and nothing but the distance in instructions separates
   // them from the first read of an accumulator
   asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   // The loads of the slices past the end are never used, but they do arrive (as zeros): the registers
   // they were aimed at stay reserved until the wait above has passed.
 #pragma unroll
-  for (int u = 0; u < 3; ++u) {
+  for (int u = 0; u < D; ++u) {
 #pragma unroll
     for (int j = 0; j < NBL; ++j) asm volatile("" : : "v"(br[u].d[j]));
     asm volatile("" : : "v"(br[u].sc));
   }
-  asm volatile("" : : "v"(asr3));
+  asm volatile("" : : "v"(asr), "v"(asr2));
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
   if (STAGE == 1) {
@@ -561,7 +638,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           float av[4][4];  // [column tile][row]
           static_for<0, 16>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
-            av[i / 4][i % 4] = acc_get<16 * mt + i>();
+            if constexpr (mt < 16) av[i / 4][i % 4] = acc_get<16 * mt + i>();
+            else av[i / 4][i % 4] = accv[mt - 16][i / 4][i % 4];
           });
           float y[2][4];
 #pragma unroll
@@ -647,7 +725,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       float av[4][4];  // [column tile][row]
       static_for<0, 16>([&](auto i_) {
         constexpr int i = decltype(i_)::value;
-        av[i / 4][i % 4] = acc_get<16 * mt + i>();
+        if constexpr (mt < 16) av[i / 4][i % 4] = acc_get<16 * mt + i>();
+        else av[i / 4][i % 4] = accv[mt - 16][i / 4][i % 4];
       });
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -668,8 +747,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 template <int STAGE>
 __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ int s_tok[MXM];
-  __shared__ float s_aff[MXM];
+  __shared__ int s_tok[MX_ROWS_MAX];
+  __shared__ float s_aff[MX_ROWS_MAX];
   // Workgroups are handed to the 8 XCDs round-robin by linear index, and each XCD has its own L2.
   // XCD x therefore takes the x-th contiguous eighth of the chunk list (chunks are ordered by
   // expert), and walks it chunk by chunk with the column tiles innermost: the workgroups that share
@@ -690,11 +769,13 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   if (last) {
     if (nrows <= 64) mx_gemm_body<STAGE, 4, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
     else if (nrows <= 128) mx_gemm_body<STAGE, 8, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else mx_gemm_body<STAGE, 16, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 256) mx_gemm_body<STAGE, 16, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else mx_gemm_body<STAGE, 20, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
   } else {
     if (nrows <= 64) mx_gemm_body<STAGE, 4, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
     else if (nrows <= 128) mx_gemm_body<STAGE, 8, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else mx_gemm_body<STAGE, 16, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 256) mx_gemm_body<STAGE, 16, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else mx_gemm_body<STAGE, 20, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
   }
 }
 

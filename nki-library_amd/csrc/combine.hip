@@ -77,7 +77,10 @@ __global__ __launch_bounds__(1024) void build_chunks_kernel(const int32_t* __res
       if (start && e >= 0 && e < E) {
         for (int64_t j = b; j < na && b2e[j] == e; ++j)
           if (valid_rows[j] > 0) last_end = j * B + valid_rows[j];
-        if (last_end > b * B) nch = (int)((last_end - b * B + CHUNK_ROWS - 1) / CHUNK_ROWS);
+        // chunks of CHUNK_ROWS rows; the last one absorbs a remainder of up to CHUNK_ROWS_MAX - CHUNK_ROWS
+        // rows, which saves the pass over the expert's weights that a small chunk of its own would cost
+        const int64_t len = last_end - b * B;
+        if (len > 0) nch = (len <= CHUNK_ROWS_MAX) ? 1 : (int)((len - CHUNK_ROWS_MAX + CHUNK_ROWS - 1) / CHUNK_ROWS) + 1;
       }
     }
     s_scan[threadIdx.x] = nch;
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(1024) void build_chunks_kernel(const int32_t* __res
       const int64_t s0 = b * B + (int64_t)k * CHUNK_ROWS;
       if (base + k < max_chunks) {
         chunk_slot[base + k] = (int32_t)s0;
-        chunk_rows[base + k] = (int32_t)((last_end - s0 < CHUNK_ROWS) ? (last_end - s0) : CHUNK_ROWS);
+        chunk_rows[base + k] = (int32_t)((k + 1 < nch) ? CHUNK_ROWS : (last_end - s0));
         chunk_expert[base + k] = e;
       }
     }

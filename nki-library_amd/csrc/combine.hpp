@@ -14,8 +14,8 @@ struct Bookkeeping {
   int32_t* cursor;      // [T1]
   int32_t* off;         // [T1+1] exclusive scan of cnt
   int32_t* list;        // [N*B] slot indices grouped by token
-  // Expert chunks: maximal runs of consecutive active blocks of one expert, cut into pieces of at
-  // most CHUNK_ROWS slots.  chunk c covers slots [chunk_slot[c], chunk_slot[c] + chunk_rows[c]).
+  // Expert chunks: maximal runs of consecutive active blocks of one expert, cut into pieces of
+  // CHUNK_ROWS slots (the last piece: up to CHUNK_ROWS_MAX).  chunk c covers slots [chunk_slot[c], chunk_slot[c] + chunk_rows[c]).
   int32_t* n_chunks;      // [1]
   int32_t* chunk_slot;    // [max_chunks]
   int32_t* chunk_rows;    // [max_chunks]
@@ -23,7 +23,8 @@ struct Bookkeeping {
   int64_t max_chunks;
 };
 
-constexpr int CHUNK_ROWS = 256;
+constexpr int CHUNK_ROWS = 256;      // rows of every chunk of a run but the last
+constexpr int CHUNK_ROWS_MAX = 320;  // the last chunk of a run takes up to this many
 inline int64_t max_chunks_for(int64_t N, int64_t B) { return N * ((B + CHUNK_ROWS - 1) / CHUNK_ROWS); }
 
 size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B);

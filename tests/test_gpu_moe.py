@@ -205,6 +205,8 @@ def _golden_mx(c, act=0):
         (512, 2048, 768, 16, 8, 128, False, False, True, 0.3, True),    # Qwen3-MoE-like tail tile (I=768), skewed, dynamic
         (200, 512, 256, 4, 2, 128, False, True, False, None, False),   # I < 512, skip_token
         (256, 512, 96, 4, 2, 256, True, False, False, None, True),     # tiny I, B=256
+        (300, 512, 256, 2, 2, 128, True, False, False, None, False),   # 300 rows per expert: one 320-row chunk each
+        (330, 1024, 384, 2, 2, 128, False, False, False, None, False), # 330 rows per expert: chunks of 256 + 74
     ],
 )
 def test_mx_variants(T, H, I, E, k, B, bias, skip, dynamic, alpha, prequant):
