@@ -190,13 +190,23 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
       float acc[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) acc[k] = 0.f;
-      for (int j = 0; j < cnt; ++j) {
-        const uint4 d = *(const uint4*)(D + (int64_t)s_sorted[j] * H + c);
-        const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+      // the additions form one dependent chain (bf16 rounding after each, in slot order), so the loads
+      // are what can overlap: up to eight rows are requested before the first is added
+      for (int j0 = 0; j0 < cnt; j0 += 8) {
+        uint4 d[8];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          acc[2 * k] = round_to_bf16(acc[2 * k] + bf16_bits_to_f32((uint16_t)(w[k] & 0xffff)));
-          acc[2 * k + 1] = round_to_bf16(acc[2 * k + 1] + bf16_bits_to_f32((uint16_t)(w[k] >> 16)));
+        for (int j = 0; j < 8; ++j)
+          if (j0 + j < cnt) d[j] = *(const uint4*)(D + (int64_t)s_sorted[j0 + j] * H + c);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (j0 + j < cnt) {
+            const uint32_t w[4] = {d[j].x, d[j].y, d[j].z, d[j].w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              acc[2 * k] = round_to_bf16(acc[2 * k] + bf16_bits_to_f32((uint16_t)(w[k] & 0xffff)));
+              acc[2 * k + 1] = round_to_bf16(acc[2 * k + 1] + bf16_bits_to_f32((uint16_t)(w[k] >> 16)));
+            }
+          }
         }
       }
       uint32_t o[4];
