@@ -43,6 +43,7 @@ int moe_check_device(void);
 #define MOE_DT_FP16 1
 #define MOE_DT_FP32 2
 #define MOE_DT_FP8_E4M3 3 /* OCP e4m3fn bit patterns; Neuron float8_e4m3 is the |v|<=240 subset */
+#define MOE_DT_FP8_E5M2 4 /* OCP e5m2 bit patterns (MXFP8 weights only)                              */
 
 /* ---- RMSNorm + quantise front end -------------------------------------------------- */
 
@@ -179,7 +180,9 @@ typedef struct moe_bwmm_args {
   int32_t scale_experts;  /* leading dim of the fp32 scales: E or 1 (BF16 / FP8_ROW)              */
   /* -- options ------------------------------------------------------------------------- */
   int32_t kind;           /* MOE_KIND_*                                                           */
-  int32_t weight_dtype;   /* BF16 kind: MOE_DT_BF16 or MOE_DT_FP8_E4M3                            */
+  int32_t weight_dtype;   /* BF16 kind: MOE_DT_BF16 or MOE_DT_FP8_E4M3; MXFP8 kind: MOE_DT_FP8_E4M3 (also
+                           * taken for MOE_DT_BF16, the zero value) or MOE_DT_FP8_E5M2 (large-tile shapes
+                           * only: H % 512 == 0 and I % 128 == 0), nl.float8_e5m2_x4 in the reference       */
   int32_t affinity_dtype; /* MOE_DT_BF16 or MOE_DT_FP32                                           */
   int32_t bias_dtype;     /* MOE_DT_BF16 or MOE_DT_FP32                                           */
   int32_t act_fn;         /* MOE_ACT_*                                                            */

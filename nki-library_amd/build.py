@@ -2,43 +2,69 @@
 
 Usage: ``python nki-library_amd/build.py``.  The library is written in-tree to
 ``nki-library_amd/nkilib/_lib/libmoe_gfx950.so`` where ``nkilib._native`` loads it.
-hipcc cross-compiles, so no GPU is needed to build.
+hipcc cross-compiles, so no GPU is needed to build.  Translation units are compiled in
+parallel into ``nki-library_amd/build/`` and linked; the MXFP8 large-tile GEMM
+(``csrc/bwmm_mx.hip``) is compiled once per (stage, weight format) plus once as the dispatcher.
 """
 
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(HERE, "build")
 OUT_DIR = os.path.join(HERE, "nkilib", "_lib")
 OUT = os.path.join(OUT_DIR, "libmoe_gfx950.so")
 SOURCES = ["rmsnorm_quant.hip", "build_blocks.hip", "combine.hip", "bwmm.hip", "bwmm_mx.hip", "router_topk.hip", "capi.hip"]
+# (stage, weight format) instances of the large-tile MX GEMM; formats as MX_WFMT_* in csrc/bwmm.hpp
+MX_INSTANCES = [(1, 0), (2, 0), (1, 1), (2, 1)]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # packed fp32 ALU ops are kept off for every HIP translation unit
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+NOISE = "is not a recognized feature for this target"
 
 
-def build(verbose=True):
-    os.makedirs(OUT_DIR, exist_ok=True)
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = ["hipcc", *FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC, *srcs, "-o", OUT]
-    if verbose:
-        print(" ".join(cmd), flush=True)
+def _run(cmd):
     res = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    err = "\n".join(l for l in res.stderr.splitlines() if NOISE not in l)
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
-    if verbose and err.strip():
-        print(err)
+        raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}\n{err}")
+    return err
+
+
+def build(verbose=True, jobs=None):
+    os.makedirs(OUT_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", CSRC]
+    units = []  # (object path, extra defines, source)
+    for s in SOURCES:
+        units.append((os.path.join(OBJ_DIR, s.replace(".hip", ".o")), [], os.path.join(CSRC, s)))
+    for stage, fmt in MX_INSTANCES:
+        units.append((os.path.join(OBJ_DIR, f"bwmm_mx_s{stage}_f{fmt}.o"),
+                      [f"-DMX_INST_STAGE={stage}", f"-DMX_INST_WFMT={fmt}"], os.path.join(CSRC, "bwmm_mx.hip")))
+    cmds = [["hipcc", *FLAGS, *defs, *inc, "-c", src, "-o", obj] for obj, defs, src in units]
+    if verbose:
+        for c in cmds:
+            print(" ".join(c), flush=True)
+    jobs = jobs or min(len(cmds), os.cpu_count() or 4, 16)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        errs = list(ex.map(_run, cmds))
+    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *[u[0] for u in units], "-o", OUT]
+    if verbose:
+        print(" ".join(link), flush=True)
+    errs.append(_run(link))
+    if verbose:
+        for e in errs:
+            if e.strip():
+                print(e)
     return OUT
 
 

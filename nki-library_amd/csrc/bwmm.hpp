@@ -64,7 +64,10 @@ struct MxArgs {
   int32_t act_fn, scaling_mode, clamp_mask;
   float clamp[4];
   int32_t col_tiles;       // column tiles per chunk (set by the launcher)
+  int32_t wfmt;            // element format of the weights, MX_WFMT_*
 };
+
+constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1;
 
 // True when the large-tile kernels cover the shape: every intermediate tile holds a multiple
 // of 32 partitions (I % 128 == 0); other shapes run the general kernel.

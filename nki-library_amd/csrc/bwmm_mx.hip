@@ -119,11 +119,16 @@ __device__ __forceinline__ float acc_get() {
 // MFMAs (a load, an LDS read) is issued between them and runs in the shadow of the first -- with one
 // wave per SIMD nothing else hides it.  op_sel / op_sel_hi carry bit 0 / bit 1 of the two scale
 // byte selectors.
-#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)                                                                  \
-  if constexpr (OA == OA_ && OB == OB_)                                                                       \
-    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%1], %2, %3, a[%0:%1], %4, %5 op_sel:" SEL_ " op_sel_hi:" SELHI_ \
-                 : : "n"(ACC), "n"(ACC + 3), "v"(af), "v"(bf), "v"(sa), "v"(sb))
-template <int ACC, int OA, int OB>
+// WFMT: element format of the weights (B operand): 0 = e4m3, 1 = e5m2 (blgp:1).
+#define MX_MFMA_ASM(FMT_, SEL_, SELHI_)                                                                          \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%1], %2, %3, a[%0:%1], %4, %5 op_sel:" SEL_ " op_sel_hi:" SELHI_ FMT_ \
+               : : "n"(ACC), "n"(ACC + 3), "v"(af), "v"(bf), "v"(sa), "v"(sb))
+#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)               \
+  if constexpr (OA == OA_ && OB == OB_) {                  \
+    if constexpr (WFMT == 0) MX_MFMA_ASM("", SEL_, SELHI_); \
+    else MX_MFMA_ASM(" blgp:1", SEL_, SELHI_);             \
+  }
+template <int ACC, int OA, int OB, int WFMT>
 __device__ __forceinline__ void mfma_asm(const v8i& af, const v8i& bf, int sa, int sb) {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
@@ -143,12 +148,17 @@ __device__ __forceinline__ void mfma_asm(const v8i& af, const v8i& bf, int sa, i
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
 }
 #undef MX_MFMA_CASE
+#undef MX_MFMA_ASM
 // The same with the accumulator tile in ordinary registers (row tiles 16..19 of a 320-row chunk).
-#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)                                                                  \
-  if constexpr (OA == OA_ && OB == OB_)                                                                       \
-    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:" SEL_ " op_sel_hi:" SELHI_ \
-                 : "+v"(c) : "v"(af), "v"(bf), "v"(sa), "v"(sb))
-template <int OA, int OB>
+#define MX_MFMA_ASM(FMT_, SEL_, SELHI_)                                                                        \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:" SEL_ " op_sel_hi:" SELHI_ FMT_ \
+               : "+v"(c) : "v"(af), "v"(bf), "v"(sa), "v"(sb))
+#define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)               \
+  if constexpr (OA == OA_ && OB == OB_) {                  \
+    if constexpr (WFMT == 0) MX_MFMA_ASM("", SEL_, SELHI_); \
+    else MX_MFMA_ASM(" blgp:1", SEL_, SELHI_);             \
+  }
+template <int OA, int OB, int WFMT>
 __device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const v8i& bf, int sa, int sb) {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
@@ -168,6 +178,7 @@ __device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const v8i& bf,
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
 }
 #undef MX_MFMA_CASE
+#undef MX_MFMA_ASM
 
 // Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
 // wave-uniform 32-bit byte offset (SGPR), which is exactly the shape of every address in this
@@ -224,7 +235,7 @@ __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, i
 // LASTUSE: this chunk is the last one of its expert, so its weights are streamed past the L2 (which
 // then keeps the activation tiles that the sibling workgroups share); an earlier chunk loads them
 // normally, for the chunk after it to find.
-template <int STAGE, int NMT, bool LASTUSE>
+template <int STAGE, int NMT, bool LASTUSE, int WFMT>
 __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
                                              int64_t slot0, int xt) {
   using Cfg = MxCfg<NMT>;
@@ -527,9 +538,9 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
         constexpr int mt = 2 * gi + j / 4, nt = j % 4;
         constexpr int m = gi * 8 + j;  // MFMA number within the slice
         if constexpr (mt < 16)
-          mfma_asm<16 * mt + 4 * nt, mt % 4, nt>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
+          mfma_asm<16 * mt + 4 * nt, mt % 4, nt, WFMT>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
         else
-          mfma_asm_v<mt % 4, nt>(accv[mt - 16][nt], af[cur][j / 4], b.f[nt], asc_hi, b.sc);
+          mfma_asm_v<mt % 4, nt, WFMT>(accv[mt - 16][nt], af[cur][j / 4], b.f[nt], asc_hi, b.sc);
         if constexpr (m == 0) {
           // the scalar arithmetic for the addresses of slice ks+D starts here, behind the first
           // MFMA, instead of ahead of it
@@ -744,7 +755,10 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   }
 }
 
-template <int STAGE>
+// One translation unit per (stage, weight format): the build compiles this file once for each with
+// MX_INST_STAGE / MX_INST_WFMT defined, and once without them for the dispatcher below.
+#if defined(MX_INST_STAGE)
+template <int STAGE, int WFMT>
 __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_tok[MX_ROWS_MAX];
@@ -767,35 +781,48 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
   const bool last = (chunk + 1 >= n_chunks) || (__builtin_amdgcn_readfirstlane(a.chunk_expert[chunk + 1]) != e);
   if (last) {
-    if (nrows <= 64) mx_gemm_body<STAGE, 4, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 128) mx_gemm_body<STAGE, 8, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 256) mx_gemm_body<STAGE, 16, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else mx_gemm_body<STAGE, 20, true>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    if (nrows <= 64) mx_gemm_body<STAGE, 4, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 128) mx_gemm_body<STAGE, 8, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 256) mx_gemm_body<STAGE, 16, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else mx_gemm_body<STAGE, 20, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
   } else {
-    if (nrows <= 64) mx_gemm_body<STAGE, 4, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 128) mx_gemm_body<STAGE, 8, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 256) mx_gemm_body<STAGE, 16, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else mx_gemm_body<STAGE, 20, false>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    if (nrows <= 64) mx_gemm_body<STAGE, 4, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 128) mx_gemm_body<STAGE, 8, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else if (nrows <= 256) mx_gemm_body<STAGE, 16, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+    else mx_gemm_body<STAGE, 20, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
   }
 }
+
+#define MX_CAT_(a, b, c, d) a##b##c##d
+#define MX_CAT(a, b, c, d) MX_CAT_(a, b, c, d)
+int MX_CAT(launch_mx_gemm_s, MX_INST_STAGE, _f, MX_INST_WFMT)(const MxArgs& m, unsigned grid, hipStream_t s) {
+  const hipError_t err = hipFuncSetAttribute((const void*)mx_gemm_kernel<MX_INST_STAGE, MX_INST_WFMT>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
+  if (err != hipSuccess) return MOE_E_LAUNCH;
+  hipLaunchKernelGGL((mx_gemm_kernel<MX_INST_STAGE, MX_INST_WFMT>), dim3(grid), dim3(MXT), MX_LDS, s, m);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+#else  // dispatcher
+
+int launch_mx_gemm_s1_f0(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s2_f0(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s1_f1(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s2_f1(const MxArgs& m, unsigned grid, hipStream_t s);
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {
   if (gx == 0 || gy == 0) return MOE_OK;
   MxArgs m = m0;
   m.col_tiles = (int32_t)gx;
   const unsigned grid = 8u * ((gy + 7u) / 8u) * gx;  // gy = upper bound on the number of chunks
-  hipError_t err;
-  if (stage == 1) {
-    err = hipFuncSetAttribute((const void*)mx_gemm_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
-    if (err != hipSuccess) return MOE_E_LAUNCH;
-    hipLaunchKernelGGL(mx_gemm_kernel<1>, dim3(grid), dim3(MXT), MX_LDS, s, m);
-  } else {
-    err = hipFuncSetAttribute((const void*)mx_gemm_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MX_LDS);
-    if (err != hipSuccess) return MOE_E_LAUNCH;
-    hipLaunchKernelGGL(mx_gemm_kernel<2>, dim3(grid), dim3(MXT), MX_LDS, s, m);
+  switch (m.wfmt) {
+    case MX_WFMT_E4M3: return stage == 1 ? launch_mx_gemm_s1_f0(m, grid, s) : launch_mx_gemm_s2_f0(m, grid, s);
+    case MX_WFMT_E5M2: return stage == 1 ? launch_mx_gemm_s1_f1(m, grid, s) : launch_mx_gemm_s2_f1(m, grid, s);
+    default: return MOE_E_BAD_ARG;
   }
-  MOE_CHECK_LAUNCH();
-  return MOE_OK;
 }
+
+#endif
 
 }  // namespace moe

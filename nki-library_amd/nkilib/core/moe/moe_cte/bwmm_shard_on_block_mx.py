@@ -59,7 +59,7 @@ def _bwmm_shard_on_block_mx(
 ):
     """Returns bf16 ``[2, T+1, H]`` with the result in ``[0]`` (``[1]`` is zero).
 
-    gate_up_proj_weight: MXFP8-e4m3 x4 ``[E, 128, 2, H/512, I]`` (4-byte elements, or uint8 with a
+    gate_up_proj_weight: MXFP8 (e4m3 or e5m2) x4 ``[E, 128, 2, H/512, I]`` (4-byte elements, or uint8 with a
     trailing axis of 4); gate_up_proj_scale uint8 ``[E, 16, 2, H/512, I]``; down_proj_weight x4
     ``[E, p_I, ceil(I/512), H]``; down_proj_scale uint8 ``[E, ceil(p_I/8), ceil(I/512), H]``;
     biases ``[E, p_I, 2, ceil(I/512), 4]`` and ``[E, H]``.  ``n_static_blocks`` /
@@ -71,9 +71,12 @@ def _bwmm_shard_on_block_mx(
     kernel_assert(block_size is not None, "block_size must be given")
     kernel_assert(gate_up_proj_scale is not None and down_proj_scale is not None,
                   "gate_up_proj_scale and down_proj_scale are required for MX weights")
-    wd = str(weight_dtype) if weight_dtype is not None else ""
-    kernel_assert("float4" not in wd and "e5m2" not in wd,
-                  f"only MXFP8 e4m3 weights are supported on gfx950, got weight_dtype={weight_dtype}")
+    # the element format of the x4 weights: the reference reads it off the tensor's nl dtype or takes
+    # it from ``weight_dtype`` for uint containers; here it is ``weight_dtype`` (a name containing
+    # "e5m2", or torch.float8_e5m2), else the weight tensor's torch dtype, else e4m3
+    wd = str(weight_dtype) if weight_dtype is not None else str(getattr(gate_up_proj_weight, "dtype", ""))
+    kernel_assert("float4" not in wd, f"MXFP4 weights are not supported on gfx950 yet, got weight_dtype={weight_dtype}")
+    wdt = nv.DT_FP8_E5M2 if "e5m2" in wd else nv.DT_FP8
     hidden_states = nv.require_device_tensor(hidden_states, "hidden_states")
     kernel_assert(hidden_states.dim() == 2, f"hidden_states must be [T+1, H] but got {tuple(hidden_states.shape)}")
     T1, H = hidden_states.shape
@@ -126,7 +129,7 @@ def _bwmm_shard_on_block_mx(
         activation_function=activation_function, skip_dma=skip_dma,
         expert_affinities_scaling_mode=expert_affinities_scaling_mode,
         gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
-        up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit,
+        up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit, weight_dtype=wdt,
     )
 
 

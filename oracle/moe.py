@@ -219,7 +219,7 @@ def moe_blockwise_fp8_row_ref(
 # ----------------------------------------------------------------------------- MX
 
 
-def gate_up_proj_mx(hidden, weight, weight_scale, bias, H, I, BxS):
+def gate_up_proj_mx(hidden, weight, weight_scale, bias, H, I, BxS, weight_format="e4m3"):
     """One of the two gate/up projections for one block (test_mlp_common.py:550-632).
 
     hidden fp32 [BxS, H]; weight uint8 [128, H/512, I, 4]; weight_scale uint8
@@ -234,7 +234,7 @@ def gate_up_proj_mx(hidden, weight, weight_scale, bias, H, I, BxS):
     ws = weight_scale.transpose(1, 0, 2).reshape(H // 32, I)
     h_mx = h_mx.reshape(PMAX, nH, BxS, Q_WIDTH).transpose(1, 0, 2, 3).reshape(H // Q_WIDTH, BxS * Q_WIDTH)
     h_scale = h_scale.reshape(PMAX // Q_HEIGHT, nH, BxS).transpose(1, 0, 2).reshape(H // 32, BxS)
-    result = mx_matmul(w, h_mx, ws, h_scale)  # [I, BxS]
+    result = mx_matmul(w, h_mx, ws, h_scale, stationary_fmt=weight_format)  # [I, BxS]
     nI = math.ceil(I / 512)
     res = np.zeros((PMAX, nI, BxS, 4), dtype=np.float32)
     for t in range(nI):
@@ -256,7 +256,7 @@ def gate_up_proj_mx(hidden, weight, weight_scale, bias, H, I, BxS):
     return res
 
 
-def down_proj_mx(inter_sb, weight, weight_scale, bias, H, I, BxS):
+def down_proj_mx(inter_sb, weight, weight_scale, bias, H, I, BxS, weight_format="e4m3"):
     """Down projection for one block (test_mlp_common.py:635-682).
 
     inter_sb fp32 [128, ceil(I/512), BxS, 4]; weight uint8 [p_I, ceil(I/512), H, 4];
@@ -277,7 +277,7 @@ def down_proj_mx(inter_sb, weight, weight_scale, bias, H, I, BxS):
     else:
         w = w[:P_aligned]
     x_mx, x_scale = quantize_mx(x)
-    result = mx_matmul(x_mx, w, x_scale, ws)  # [BxS, H]
+    result = mx_matmul(x_mx, w, x_scale, ws, moving_fmt=weight_format)  # [BxS, H]
     if bias is not None:
         result = result + np.asarray(bias, dtype=np.float32).reshape(1, H)
     return result
@@ -304,8 +304,10 @@ def moe_blockwise_mx_ref(
     up_clamp_upper_limit=None,
     up_clamp_lower_limit=None,
     max_blocks=None,
+    weight_format="e4m3",
 ):
-    """MXFP8 blockwise MoE golden (test_utils.py:474-735, MX branch).
+    """MXFP8 blockwise MoE golden (test_utils.py:474-735, MX branch); ``weight_format`` "e4m3" or "e5m2"
+    (activations and the intermediate are always quantised to e4m3, bwmm_shard_on_block_mx.py:304).
 
     hidden_states bf16-valued fp32 [T+1, H], quantised online per block;
     gate_up_proj_weight uint8 [E, 128, 2, H/512, I, 4]; gate_up_proj_scale uint8
@@ -341,13 +343,13 @@ def moe_blockwise_mx_ref(
         if gate_up_proj_bias is not None:
             gb = np.asarray(gate_up_proj_bias, dtype=np.float32)[e][:, 0]
             ub = np.asarray(gate_up_proj_bias, dtype=np.float32)[e][:, 1]
-        g = gate_up_proj_mx(x, gate_up_proj_weight[e][:, 0], gate_up_proj_scale[e][:, 0], gb, H, I, B)
-        u = gate_up_proj_mx(x, gate_up_proj_weight[e][:, 1], gate_up_proj_scale[e][:, 1], ub, H, I, B)
+        g = gate_up_proj_mx(x, gate_up_proj_weight[e][:, 0], gate_up_proj_scale[e][:, 0], gb, H, I, B, weight_format)
+        u = gate_up_proj_mx(x, gate_up_proj_weight[e][:, 1], gate_up_proj_scale[e][:, 1], ub, H, I, B, weight_format)
         _clip(g, gate_clamp_lower_limit, gate_clamp_upper_limit)
         _clip(u, up_clamp_lower_limit, up_clamp_upper_limit)
         y = (act_fn(g, activation_function) * u).astype(np.float32)
         db = None if down_proj_bias is None else np.asarray(down_proj_bias, dtype=np.float32)[e]
-        d = down_proj_mx(y, down_proj_weight[e], down_proj_scale[e], db, H, I, B)
+        d = down_proj_mx(y, down_proj_weight[e], down_proj_scale[e], db, H, I, B, weight_format)
         if expert_affinities_scaling_mode == POST_SCALE:
             d = d * a
         _accumulate(out, ids, d.astype(np.float32))

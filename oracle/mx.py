@@ -25,38 +25,47 @@ both goldens for all-zero blocks' data (zeros).  Parity unpinned for
 
 import numpy as np
 
-from .numerics import E4M3FN_MAX, e4m3fn_decode, e4m3fn_encode, float32_exponent_field
+from .numerics import (E4M3FN_MAX, E5M2_MAX, e4m3fn_decode, e4m3fn_encode, e5m2_decode, e5m2_encode,
+                       float32_exponent_field)
 
 Q_HEIGHT = 8  # partitions per block
 Q_WIDTH = 4  # packed free elements per block
 E4M3_MAX_EXP = 8  # 448 = 1.75 * 2**8
+# element formats of an MXFP8 tensor: (largest exponent, largest value, encode, decode), the table of
+# mx_torch_common.py:190-198
+FORMATS = {
+    "e4m3": (E4M3_MAX_EXP, E4M3FN_MAX, e4m3fn_encode, e4m3fn_decode),
+    "e5m2": (15, E5M2_MAX, e5m2_encode, e5m2_decode),
+}
 
 
-def quantize_mx(x):
-    """[P, F] float -> (uint8 data [P, F], uint8 scale [P/8, F/4]) as MXFP8 e4m3fn."""
+def quantize_mx(x, fmt="e4m3"):
+    """[P, F] float -> (uint8 data [P, F], uint8 scale [P/8, F/4]) as MXFP8 (e4m3fn unless fmt says e5m2)."""
+    max_exp, max_val, encode, _ = FORMATS[fmt]
     x = np.ascontiguousarray(x, dtype=np.float32)
     P, F = x.shape
     assert P % Q_HEIGHT == 0 and F % Q_WIDTH == 0, (P, F)
     SP, SF = P // Q_HEIGHT, F // Q_WIDTH
     exp = float32_exponent_field(x).reshape(SP, Q_HEIGHT, SF, Q_WIDTH)
     emax = exp.max(axis=(1, 3)).astype(np.int32)
-    scale_u8 = np.clip(emax - E4M3_MAX_EXP, 0, 255).astype(np.uint8)
+    scale_u8 = np.clip(emax - max_exp, 0, 255).astype(np.uint8)
     factor = np.power(2.0, scale_u8.astype(np.float64) - 127.0)
     factor = np.repeat(np.repeat(factor, Q_HEIGHT, axis=0), Q_WIDTH, axis=1)
-    v = np.clip(x.astype(np.float64) / factor, -E4M3FN_MAX, E4M3FN_MAX).astype(np.float32)
-    return e4m3fn_encode(v), scale_u8
+    v = np.clip(x.astype(np.float64) / factor, -max_val, max_val).astype(np.float32)
+    return encode(v), scale_u8
 
 
-def dequantize_mx(data_u8, scale_u8):
+def dequantize_mx(data_u8, scale_u8, fmt="e4m3"):
     """Inverse of quantize_mx: uint8 [P, F], uint8 [P/8, F/4] -> float32 [P, F] (exact)."""
+    decode = FORMATS[fmt][3]
     P, F = data_u8.shape
     assert scale_u8.shape == (P // Q_HEIGHT, F // Q_WIDTH), (data_u8.shape, scale_u8.shape)
     factor = np.power(2.0, np.clip(scale_u8.astype(np.int32) - 127, -127, 127).astype(np.float64))
     factor = np.repeat(np.repeat(factor, Q_HEIGHT, axis=0), Q_WIDTH, axis=1)
-    return (e4m3fn_decode(data_u8).astype(np.float64) * factor).astype(np.float32)
+    return (decode(data_u8).astype(np.float64) * factor).astype(np.float32)
 
 
-def mx_matmul(stationary_u8, moving_u8, stationary_scale, moving_scale):
+def mx_matmul(stationary_u8, moving_u8, stationary_scale, moving_scale, stationary_fmt="e4m3", moving_fmt="e4m3"):
     """Block-scaled matmul golden.
 
     stationary [K/4 (P), M*4] bytes + scale [K/32, M]; moving [K/4, N*4] bytes +
@@ -66,8 +75,8 @@ def mx_matmul(stationary_u8, moving_u8, stationary_scale, moving_scale):
     like the golden's float32 einsum (summation order is BLAS's, as unspecified
     there as in numpy's einsum).
     """
-    s = dequantize_mx(stationary_u8, stationary_scale)
-    m = dequantize_mx(moving_u8, moving_scale)
+    s = dequantize_mx(stationary_u8, stationary_scale, stationary_fmt)
+    m = dequantize_mx(moving_u8, moving_scale, moving_fmt)
     KP = s.shape[0]
     s = s.reshape(KP, -1, Q_WIDTH)
     m = m.reshape(KP, -1, Q_WIDTH)

@@ -87,6 +87,47 @@ def e4m3fn_encode(x):
     return (code.astype(np.uint8) | (sign << 7)).reshape(x.shape)
 
 
+def _build_e5m2_table():
+    """All 256 e5m2 bit patterns as the reference decodes them
+    (src/nkilib_src/nkilib/core/utils/mx_torch_common.py:87-111): S(1) E(5) M(2), bias 15; the
+    exponent field 31 is decoded like any other (no inf / NaN), codes the quantiser never emits."""
+    codes = np.arange(256, dtype=np.int64)
+    sign = (codes >> 7) & 1
+    exp = (codes >> 2) & 0x1F
+    man = codes & 0x3
+    sub = (man / 4.0) * 2.0**-14
+    nor = (1.0 + man / 4.0) * np.power(2.0, exp - 15.0)
+    val = np.where(exp == 0, sub, nor)
+    return np.where(sign == 1, -val, val).astype(np.float32)
+
+
+E5M2_TABLE = _build_e5m2_table()
+E5M2_MAX = 57344.0
+
+
+def e5m2_decode(codes):
+    """uint8 bit patterns -> float32 (exact)."""
+    return E5M2_TABLE[np.asarray(codes, dtype=np.uint8)]
+
+
+def e5m2_encode(x):
+    """float32 -> uint8 e5m2 bit patterns, round-to-nearest-even, saturating at +-57344 (the callers
+    clip first, like the goldens: mx_torch_common.py:216-219)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    bits = x.view(np.uint32)
+    sign = ((bits >> 31) & 1).astype(np.uint8)
+    a = np.abs(x)
+    abits = (bits & 0x7FFFFFFF).astype(np.uint64)
+    # normal path: keep 2 mantissa bits, RNE on the 21 dropped bits
+    r = (abits + 0xFFFFF + ((abits >> 21) & 1)) >> 21  # (exp8 << 2) | man2
+    code_n = r.astype(np.int64) - (112 << 2)  # rebias 127 -> 15
+    # subnormal path (|x| < 2**-14): multiples of 2**-16, RNE; 4 == smallest normal
+    code_s = np.rint(a.astype(np.float64) * 65536.0).astype(np.int64)
+    code = np.where(a < 2.0**-14, code_s, code_n)
+    code = np.clip(code, 0, 0x7B)
+    return (code.astype(np.uint8) | (sign << 7)).reshape(x.shape)
+
+
 def e8m0_decode(b):
     """uint8 E8M0 -> float64 power of two, 2**(b-127)."""
     return np.power(2.0, np.asarray(b).astype(np.int32) - 127)

@@ -69,12 +69,12 @@ def dense_case(T, H, I, E, k, B, seed=0, skip_token=False, bias=False, quant=Fal
     return c
 
 
-def mx_weights(rng, E, H, I, std=0.02):
-    """Random MXFP8 expert weights in the reference's x4 layouts (byte axis last)."""
+def mx_weights(rng, E, H, I, std=0.02, fmt="e4m3"):
+    """Random MXFP8 expert weights (element format ``fmt``) in the reference's x4 layouts (byte axis last)."""
     nH, nI = H // 512, math.ceil(I / 512)
     pI = 128 if I > 512 else I // 4
     gu_fp = (rng.standard_normal((E * 128, 2 * nH * I * 4)) * std).astype(np.float32)
-    gu_q, gu_s = omx.quantize_mx(gu_fp)
+    gu_q, gu_s = omx.quantize_mx(gu_fp, fmt)
     gu_q = gu_q.reshape(E, 128, 2, nH, I, 4)
     gu_s = gu_s.reshape(E, 16, 2, nH, I)
     d_fp = (rng.standard_normal((E, pI, nI, H, 4)) * std).astype(np.float32)
@@ -84,14 +84,14 @@ def mx_weights(rng, E, H, I, std=0.02):
     pI8 = math.ceil(pI / 8) * 8
     d2 = np.zeros((E, pI8, nI, H, 4), np.float32)
     d2[:, :pI] = d_fp
-    d_q, d_s = omx.quantize_mx(d2.reshape(E * pI8, nI * H * 4))
+    d_q, d_s = omx.quantize_mx(d2.reshape(E * pI8, nI * H * 4), fmt)
     d_q = d_q.reshape(E, pI8, nI, H, 4)[:, :pI].copy()
     d_s = d_s.reshape(E, pI8 // 8, nI, H)
     return gu_q, gu_s, d_q, d_s
 
 
 def mx_case(T, H, I, E, k, B, seed=0, skip_token=False, bias=False, alpha=None, hidden_std=1.0, weight_std=0.05,
-            dynamic=False):
+            dynamic=False, weight_format="e4m3"):
     rng = np.random.default_rng(seed)
     N, mask, tp2id, b2e, cond = routing(T, k, E, B, skip_token, alpha, n_block_per_iter=2, is_block_parallel=True,
                                         is_mx=True)
@@ -99,10 +99,10 @@ def mx_case(T, H, I, E, k, B, seed=0, skip_token=False, bias=False, alpha=None, 
     hs = to_bf16((rng.standard_normal((T1, H)) * hidden_std).astype(np.float32))
     if not skip_token:
         hs[T] = 0
-    gu_q, gu_s, d_q, d_s = mx_weights(rng, E, H, I, weight_std)
+    gu_q, gu_s, d_q, d_s = mx_weights(rng, E, H, I, weight_std, weight_format)
     c = {"T": T, "T1": T1, "H": H, "I": I, "E": E, "k": k, "B": B, "N": N, "skip_token": skip_token,
          "hidden": hs, "aff": affinities(rng, T, E, mask, skip_token), "tp2id": tp2id, "b2e": b2e,
-         "cond": cond if dynamic else None, "mask": mask,
+         "cond": cond if dynamic else None, "mask": mask, "weight_format": weight_format,
          "gate_up_q": gu_q, "gate_up_s": gu_s, "down_q": d_q, "down_s": d_s}
     if bias:
         nI = math.ceil(I / 512)

@@ -162,7 +162,7 @@ def test_fp8_row_pipeline(T, H, I, E, k, B):
     _check(from_bf16_tensor(out)[:, 0], g, "fp8 row")
 
 
-def _run_mx(c, prequant=False, act=0):
+def _run_mx(c, prequant=False, act=0, weight_dtype=None):
     import torch
     from nkilib.core.moe.moe_cte import QuantizationConfig, SkipMode, moe_cte
     from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize
@@ -190,11 +190,33 @@ def _run_mx(c, prequant=False, act=0):
     return out
 
 
+def _run_mx_direct(c, weight_dtype):
+    """bwmm_shard_on_block_mx with an explicit weight_dtype for uint containers (the reference's use_uint_weights cases)."""
+    import torch
+    from nkilib.core.moe.moe_cte.bwmm_shard_on_block_mx import bwmm_shard_on_block_mx
+    from nkilib.core.moe.moe_cte import SkipMode
+
+    dev = torch.device("cuda:0")
+    kw = {}
+    if "gate_up_bias" in c:
+        kw["gate_and_up_proj_bias"] = bf16_tensor(c["gate_up_bias"], dev)
+        kw["down_proj_bias"] = bf16_tensor(c["down_bias"], dev)
+    gu = torch.from_numpy(c["gate_up_q"].view(np.int32).reshape(c["gate_up_q"].shape[:-1])).to(dev)
+    dw = torch.from_numpy(c["down_q"].view(np.int32).reshape(c["down_q"].shape[:-1])).to(dev)
+    out = bwmm_shard_on_block_mx[2](
+        bf16_tensor(c["hidden"], dev), bf16_tensor(c["aff"].reshape(-1, 1), dev), gu, dw,
+        i32_tensor(c["tp2id"], dev), i32_tensor(c["b2e"], dev), gate_up_proj_scale=u8_tensor(c["gate_up_s"], dev),
+        down_proj_scale=u8_tensor(c["down_s"], dev), block_size=c["B"], skip_dma=SkipMode(c["skip_token"], False),
+        weight_dtype=weight_dtype, **kw)
+    torch.cuda.synchronize()
+    return out
+
+
 def _golden_mx(c, act=0):
     return omoe.moe_blockwise_mx_ref(
         c["hidden"], c["aff"], c["gate_up_q"], c["down_q"], c["gate_up_s"], c["down_s"], c["tp2id"], c["b2e"], c["B"],
         conditions=c["cond"], gate_up_proj_bias=c.get("gate_up_bias"), down_proj_bias=c.get("down_bias"),
-        activation_function=act, skip_token=c["skip_token"])
+        activation_function=act, skip_token=c["skip_token"], weight_format=c.get("weight_format", "e4m3"))
 
 
 @pytest.mark.parametrize(
@@ -220,6 +242,18 @@ def test_mx_variants(T, H, I, E, k, B, bias, skip, dynamic, alpha, prequant):
         _check(o[0, :T], g[:T], f"mx H={H} I={I} E={E}")
     else:
         _check(o[0], g, f"mx H={H} I={I} E={E}")
+
+
+@pytest.mark.parametrize("T,H,I,E,k,B,bias", [(256, 512, 512, 8, 2, 128, False), (300, 1024, 384, 2, 2, 128, True)])
+def test_mx_e5m2_weights(T, H, I, E, k, B, bias):
+    """MXFP8 weights in e5m2 (nl.float8_e5m2_x4; test_moe_bwmm_mx_cte.py:74-76, :80): uint32 containers + weight_dtype."""
+    c = mx_case(T, H, I, E, k, B, seed=11, bias=bias, weight_format="e5m2")
+    o = from_bf16_tensor(_run_mx_direct(c, "float8_e5m2_x4"))
+    g = _golden_mx(c)
+    _check(o[0, :T], g[:T], f"mx e5m2 H={H} I={I} E={E}")
+    # the same bytes read as e4m3 give a different answer: the format switch is what the result depends on
+    o4 = from_bf16_tensor(_run_mx_direct(c, "float8_e4m3fn_x4"))
+    assert max_abs_rel(o4[0, :T], g[:T]) > 0.1
 
 
 def test_mx_prequantised_equals_online():

@@ -109,3 +109,32 @@ def test_dequant_helpers_agree_with_block_form():
     res = omoe.gate_up_proj_mx(x, w[:, 0], s[:, 0], None, H, I, B)  # [128, 1, B, 4]
     got = res[:, 0].transpose(2, 0, 1).reshape(I, B)  # i = q*128 + p
     assert np.allclose(got.T, dense[0][kp], rtol=0, atol=0)
+
+
+def test_e5m2_block_scale_closed_forms_and_round_trip():
+    """e5m2 target (mx_torch_common.py:190-198: largest exponent 15, largest value 57344): an all-ones block gets
+    scale byte 127 - 15 and the code of 2**15; values already on the e5m2 grid of their block survive a round trip."""
+    d, s = mx.quantize_mx(np.ones((8, 4), np.float32), fmt="e5m2")
+    assert s[0, 0] == 112 and (d == 0x78).all()
+    assert np.array_equal(mx.dequantize_mx(d, s, fmt="e5m2"), np.ones((8, 4), np.float32))
+    rng = np.random.default_rng(5)
+    codes = rng.integers(0, 0x7C, size=(64, 32)).astype(np.uint8) | (rng.integers(0, 2, size=(64, 32)).astype(np.uint8) << 7)
+    codes.reshape(8, 8, 8, 4)[:, 0, :, 0] = 0x7B  # every block holds the format maximum: scale == the one given
+    sc = rng.integers(100, 150, size=(8, 8)).astype(np.uint8)
+    x = mx.dequantize_mx(codes, sc, fmt="e5m2")
+    q, s2 = mx.quantize_mx(x, fmt="e5m2")
+    assert np.array_equal(s2, sc) and np.array_equal(mx.dequantize_mx(q, s2, fmt="e5m2"), x)
+
+
+def test_mx_matmul_mixed_formats_is_the_plain_product():
+    """e5m2 stationary x e4m3 moving equals the fp64 product of the dequantised operands."""
+    rng = np.random.default_rng(6)
+    a = (rng.standard_normal((32, 16 * 4)) * 0.1).astype(np.float32)
+    b = rng.standard_normal((32, 8 * 4)).astype(np.float32)
+    aq, asc = mx.quantize_mx(a, fmt="e5m2")
+    bq, bsc = mx.quantize_mx(b)
+    got = mx.mx_matmul(aq, bq, asc, bsc, stationary_fmt="e5m2")
+    ad = mx.dequantize_mx(aq, asc, fmt="e5m2").astype(np.float64).reshape(32, 16, 4)
+    bd = mx.dequantize_mx(bq, bsc).astype(np.float64).reshape(32, 8, 4)
+    want = np.einsum("kiq,kjq->ij", ad, bd)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)

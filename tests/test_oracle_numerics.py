@@ -35,6 +35,30 @@ def test_e4m3fn_roundtrip_every_code():
     assert np.array_equal(nm.e4m3fn_encode(nm.e4m3fn_decode(codes)), codes)
 
 
+def test_e5m2_decode_is_the_closed_form_and_matches_torch():
+    codes = np.arange(256, dtype=np.uint8)
+    v = nm.e5m2_decode(codes)
+    tv = torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+    finite = ((codes >> 2) & 0x1F) != 31  # torch reads exponent field 31 as inf / NaN, the reference as 2**16 * (1 + m/4)
+    assert np.array_equal(v[finite], tv[finite])
+    assert v[0x7B] == 57344.0 and v[0x3C] == 1.0 and v[0x01] == 2.0**-16 and v[0x04] == 2.0**-14 and v[0x7C] == 65536.0
+
+
+def test_e5m2_encode_matches_torch_rne_on_random_and_boundaries():
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal(400000) * rng.choice([1e-6, 1e-4, 1.0, 300.0, 30000.0], 400000)).astype(np.float32)
+    x = np.clip(x, -57344, 57344)
+    v = np.sort(nm.e5m2_decode(np.arange(0, 0x7C, dtype=np.uint8)))
+    mids = ((v[:-1].astype(np.float64) + v[1:]) / 2).astype(np.float32)
+    ties = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)), -mids])
+    x = np.concatenate([x, ties, v, -v])
+    ours = nm.e5m2_encode(x)
+    theirs = torch.from_numpy(x).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    assert np.array_equal(ours, theirs)
+    codes = np.array([c for c in range(256) if ((c >> 2) & 0x1F) != 31], dtype=np.uint8)
+    assert np.array_equal(nm.e5m2_encode(nm.e5m2_decode(codes)), codes)
+
+
 def test_bf16_round_matches_torch():
     rng = np.random.default_rng(1)
     x = (rng.standard_normal(300000) * rng.choice([1e-20, 1e-3, 1.0, 1e4, 1e30], 300000)).astype(np.float32)
