@@ -44,6 +44,7 @@ int moe_check_device(void);
 #define MOE_DT_FP32 2
 #define MOE_DT_FP8_E4M3 3 /* OCP e4m3fn bit patterns; Neuron float8_e4m3 is the |v|<=240 subset */
 #define MOE_DT_FP8_E5M2 4 /* OCP e5m2 bit patterns (MXFP8 weights only)                              */
+#define MOE_DT_FP4_E2M1 5 /* OCP e2m1 (MXFP4 weights only): four 4-bit values per 2-byte x4 element   */
 
 /* ---- RMSNorm + quantise front end -------------------------------------------------- */
 
@@ -181,8 +182,10 @@ typedef struct moe_bwmm_args {
   /* -- options ------------------------------------------------------------------------- */
   int32_t kind;           /* MOE_KIND_*                                                           */
   int32_t weight_dtype;   /* BF16 kind: MOE_DT_BF16 or MOE_DT_FP8_E4M3; MXFP8 kind: MOE_DT_FP8_E4M3 (also
-                           * taken for MOE_DT_BF16, the zero value) or MOE_DT_FP8_E5M2 (large-tile shapes
-                           * only: H % 512 == 0 and I % 128 == 0), nl.float8_e5m2_x4 in the reference       */
+                           * taken for MOE_DT_BF16, the zero value), MOE_DT_FP8_E5M2 or MOE_DT_FP4_E2M1 (the
+                           * last two on large-tile shapes only: H % 512 == 0 and I % 128 == 0):
+                           * nl.float8_e4m3fn_x4 / float8_e5m2_x4 / float4_e2m1fn_x4 in the reference; 4-bit
+                           * weights have the same shapes with 2-byte elements                              */
   int32_t affinity_dtype; /* MOE_DT_BF16 or MOE_DT_FP32                                           */
   int32_t bias_dtype;     /* MOE_DT_BF16 or MOE_DT_FP32                                           */
   int32_t act_fn;         /* MOE_ACT_*                                                            */

@@ -44,7 +44,7 @@ struct MxArgs {
   const uint8_t* A_scale;  // E8M0 [rows, a_scale_stride]
   int64_t a_scale_stride;
   int64_t a_rows;          // rows of A and A_scale
-  const uint32_t* W;       // x4 weights in the reference layout
+  const uint32_t* W;       // x4 weights in the reference layout (4-byte elements; 2-byte ones for 4-bit weights)
   const uint8_t* W_scale;
   const void* bias;
   int32_t bias_dtype;
@@ -67,7 +67,7 @@ struct MxArgs {
   int32_t wfmt;            // element format of the weights, MX_WFMT_*
 };
 
-constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1;
+constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1, MX_WFMT_E2M1 = 2;
 
 // True when the large-tile kernels cover the shape: every intermediate tile holds a multiple
 // of 32 partitions (I % 128 == 0); other shapes run the general kernel.

@@ -78,9 +78,10 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+template <class Operand>
 struct BFrag {
-  v8i f[4];  // four column tiles
-  int sc;    // their E8M0 scale bytes (byte t = tile t)
+  Operand f[4];  // four column tiles (8 registers each for 8-bit weights, 4 for 4-bit ones)
+  int sc;        // their E8M0 scale bytes (byte t = tile t)
 };
 
 __device__ __forceinline__ v8i frag_from_lds(const uint8_t* plo, const uint8_t* phi) {
@@ -119,17 +120,19 @@ __device__ __forceinline__ float acc_get() {
 // MFMAs (a load, an LDS read) is issued between them and runs in the shadow of the first -- with one
 // wave per SIMD nothing else hides it.  op_sel / op_sel_hi carry bit 0 / bit 1 of the two scale
 // byte selectors.
-// WFMT: element format of the weights (B operand): 0 = e4m3, 1 = e5m2 (blgp:1).
+// WFMT: element format of the weights (B operand): 0 = e4m3, 1 = e5m2 (blgp:1), 2 = e2m1 (blgp:4; 4-bit
+// elements: the operand is four registers, lane group g holding K 32g .. 32g+31, eight to a register).
 #define MX_MFMA_ASM(FMT_, SEL_, SELHI_)                                                                          \
   asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%1], %2, %3, a[%0:%1], %4, %5 op_sel:" SEL_ " op_sel_hi:" SELHI_ FMT_ \
                : : "n"(ACC), "n"(ACC + 3), "v"(af), "v"(bf), "v"(sa), "v"(sb))
 #define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)               \
   if constexpr (OA == OA_ && OB == OB_) {                  \
     if constexpr (WFMT == 0) MX_MFMA_ASM("", SEL_, SELHI_); \
-    else MX_MFMA_ASM(" blgp:1", SEL_, SELHI_);             \
+    else if constexpr (WFMT == 1) MX_MFMA_ASM(" blgp:1", SEL_, SELHI_); \
+    else MX_MFMA_ASM(" blgp:4", SEL_, SELHI_);             \
   }
-template <int ACC, int OA, int OB, int WFMT>
-__device__ __forceinline__ void mfma_asm(const v8i& af, const v8i& bf, int sa, int sb) {
+template <int ACC, int OA, int OB, int WFMT, class BOp>
+__device__ __forceinline__ void mfma_asm(const v8i& af, const BOp& bf, int sa, int sb) {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
   MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
@@ -156,10 +159,11 @@ __device__ __forceinline__ void mfma_asm(const v8i& af, const v8i& bf, int sa, i
 #define MX_MFMA_CASE(OA_, OB_, SEL_, SELHI_)               \
   if constexpr (OA == OA_ && OB == OB_) {                  \
     if constexpr (WFMT == 0) MX_MFMA_ASM("", SEL_, SELHI_); \
-    else MX_MFMA_ASM(" blgp:1", SEL_, SELHI_);             \
+    else if constexpr (WFMT == 1) MX_MFMA_ASM(" blgp:1", SEL_, SELHI_); \
+    else MX_MFMA_ASM(" blgp:4", SEL_, SELHI_);             \
   }
-template <int OA, int OB, int WFMT>
-__device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const v8i& bf, int sa, int sb) {
+template <int OA, int OB, int WFMT, class BOp>
+__device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const BOp& bf, int sa, int sb) {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
   MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
@@ -218,6 +222,13 @@ __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& r
 __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+}
+template <bool NT>
+__device__ __forceinline__ void ld_b64(v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  if constexpr (NT)
+    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen nt" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  else
+    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 typedef int v3i __attribute__((ext_vector_type(3)));
 __device__ __forceinline__ void ld_dwords(v3i& d, uint32_t voff, const v4i& rsrc, int soff) {
@@ -346,22 +357,29 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // fetches 128 contiguous bytes of gate and of up for 4 K rows.  (8-byte loads, one tile pair per
   // load, cost the memory pipeline as much per instruction as 16-byte ones.)
   const int hcol = (STAGE == 1) ? (c >> 3) : 0, cl = (STAGE == 1) ? (c & 7) : c;
+  // 4-bit weights (x4: four K values in a 2-byte element): lane group g needs K 32g .. 32g+31 of the
+  // slice = partitions 8g .. 8g+7, one 8-byte load (4 columns) per partition; 8-bit weights (4-byte
+  // elements): partitions 4g .. 4g+3 and 16+4g .. 16+4g+3, one 16-byte load each.
+  constexpr bool FP4 = WFMT == 2;
+  constexpr int ES = FP4 ? 2 : 4;      // bytes of a weight element
+  constexpr int GROWS = FP4 ? 8 : 4;   // partition rows between the lane groups' first rows
+  const uint8_t* Wb = (const uint8_t*)a.W;
   if (STAGE == 1) {
     w_pstride = 2 * nH * a.I;
     w_tstride = a.I;
     colu = (int64_t)tI * 512 + (int64_t)q * Pt + p0;
-    rw_ = make_rsrc(a.W + (int64_t)e * 128 * w_pstride, (uint32_t)(128 * w_pstride * 4));
+    rw_ = make_rsrc(Wb + (int64_t)e * 128 * w_pstride * ES, (uint32_t)(128 * w_pstride * ES));
     rs_ = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
-    w_voff = (uint32_t)((4 * g * w_pstride + hcol * nH * a.I + 4 * cl) * 4);
+    w_voff = (uint32_t)((GROWS * g * w_pstride + hcol * nH * a.I + 4 * cl) * ES);
     s_voff = (uint32_t)(g * w_pstride + hcol * nH * a.I + 4 * cl);
   } else {
     w_pstride = (int64_t)a.nI * a.H;
     w_tstride = a.H;
     colu = h0 + 64 * q;
     const int64_t sp = (a.pI + 7) / 8;
-    rw_ = make_rsrc(a.W + (int64_t)e * a.pI * w_pstride, (uint32_t)(a.pI * w_pstride * 4));
+    rw_ = make_rsrc(Wb + (int64_t)e * a.pI * w_pstride * ES, (uint32_t)(a.pI * w_pstride * ES));
     rs_ = make_rsrc(a.W_scale + (int64_t)e * sp * w_pstride, (uint32_t)(sp * w_pstride));
-    w_voff = (uint32_t)((4 * g * w_pstride + 4 * c) * 4);
+    w_voff = (uint32_t)((GROWS * g * w_pstride + 4 * c) * ES);
     s_voff = (uint32_t)(g * w_pstride + 4 * c);
   }
 
@@ -377,8 +395,10 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   constexpr int N1 = NAJ + NLB;             // loads of a slice that carries no activation scales
   constexpr int N0 = N1 + NSC;              // loads of one that does
   typedef typename std::conditional<D == 3, v3i, v2i>::type ScaleRegs;
+  typedef typename std::conditional<FP4, v2i, v4i>::type RawLoad;
+  typedef typename std::conditional<FP4, v4i, v8i>::type BOperand;
   struct BRaw {
-    v4i d[NBL];
+    RawLoad d[NBL];
     int sc;
   };
   const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_rows * a.a_scale_stride));
@@ -389,8 +409,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   int w_soff[NBL];
 #pragma unroll
   for (int i = 0; i < NBL; ++i) {
-    const int pr = (i < 4) ? i : (16 + i - 4);
-    w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * 4);
+    const int pr = FP4 ? i : ((i < 4) ? i : (16 + i - 4));
+    w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * ES);
   }
   const int s_soff = uni(colu);
   // Everything a slice's loads share: descriptors (of zero records past the end: such a load is out
@@ -418,7 +438,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     const int kt = ks >> 2, pb = ks & 3;
     r.a_off = ks * 128;
     r.as_off = ks * 4;
-    r.w_off = uni(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * 4);
+    r.w_off = uni(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * ES);
     r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
@@ -437,7 +457,8 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       }
     } else if constexpr (idx < NAJ + NSC + NBL) {
       constexpr int i = idx - NAJ - NSC;
-      ld_b128<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
+      if constexpr (FP4) ld_b64<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
+      else ld_b128<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
     } else {
       ld_b32(b.sc, s_voff, sa.rs, s_soff + sa.s_off);
     }
@@ -508,15 +529,28 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
     for (int j = 0; j < NBL; ++j) asm volatile("" : "+v"(braw.d[j]));
     asm volatile("" : "+v"(braw.sc));
-    // one 16-byte load gives a lane the same K row of 4 column tiles; an MFMA wants the 8 K rows of
-    // one tile in consecutive registers
-    BFrag b;
+    // one load gives a lane the same K row (partition) of 4 column tiles; an MFMA wants the K rows of
+    // one tile in consecutive registers (8-bit: one register per partition; 4-bit: two partitions,
+    // 16 bits each, per register)
+    BFrag<BOperand> b;
+    if constexpr (FP4) {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      b.f[0][r] = braw.d[r][0];
-      b.f[1][r] = braw.d[r][1];
-      b.f[2][r] = braw.d[r][2];
-      b.f[3][r] = braw.d[r][3];
+      for (int r = 0; r < 4; ++r) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t lo = (uint32_t)braw.d[2 * r][t >> 1], hi = (uint32_t)braw.d[2 * r + 1][t >> 1];
+          // low halves (even tile) or high halves (odd tile) of the two partitions' dwords
+          b.f[t][r] = (int)__builtin_amdgcn_perm(hi, lo, (t & 1) ? 0x07060302u : 0x05040100u);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        b.f[0][r] = braw.d[r][0];
+        b.f[1][r] = braw.d[r][1];
+        b.f[2][r] = braw.d[r][2];
+        b.f[3][r] = braw.d[r][3];
+      }
     }
     b.sc = braw.sc;
     asm volatile("s_nop 1" : "+v"(b.f[0]), "+v"(b.f[1]), "+v"(b.f[2]), "+v"(b.f[3]), "+v"(b.sc));
@@ -810,6 +844,8 @@ int launch_mx_gemm_s1_f0(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f0(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s1_f1(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f1(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s1_f2(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s2_f2(const MxArgs& m, unsigned grid, hipStream_t s);
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {
   if (gx == 0 || gy == 0) return MOE_OK;
@@ -819,6 +855,7 @@ int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStr
   switch (m.wfmt) {
     case MX_WFMT_E4M3: return stage == 1 ? launch_mx_gemm_s1_f0(m, grid, s) : launch_mx_gemm_s2_f0(m, grid, s);
     case MX_WFMT_E5M2: return stage == 1 ? launch_mx_gemm_s1_f1(m, grid, s) : launch_mx_gemm_s2_f1(m, grid, s);
+    case MX_WFMT_E2M1: return stage == 1 ? launch_mx_gemm_s1_f2(m, grid, s) : launch_mx_gemm_s2_f2(m, grid, s);
     default: return MOE_E_BAD_ARG;
   }
 }

@@ -84,7 +84,7 @@ int validate(const moe_bwmm_args* a) {
       // POST_SCALE only (test_moe_bwmm_mx_cte.py:163-167)
       if (a->scaling_mode == MOE_SCALE_PRE || a->scaling_mode == MOE_SCALE_PRE_DELAYED) return MOE_E_UNSUPPORTED;
       // weight element formats: e4m3 everywhere, e5m2 on the large-tile path
-      if (a->weight_dtype == MOE_DT_FP8_E5M2) {
+      if (a->weight_dtype == MOE_DT_FP8_E5M2 || a->weight_dtype == MOE_DT_FP4_E2M1) {
         if (!mx_fast_path_ok(a->H, a->I)) return MOE_E_UNSUPPORTED;
       } else if (a->weight_dtype != MOE_DT_FP8_E4M3 && a->weight_dtype != MOE_DT_BF16) {
         return MOE_E_BAD_ARG;
@@ -233,7 +233,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     m.H = a->H; m.I = a->I; m.E = a->E; m.n_real = n_real;
     m.pI = (int32_t)p.pI; m.nI = (int32_t)p.nI;
     m.act_fn = a->act_fn; m.scaling_mode = a->scaling_mode; m.clamp_mask = a->clamp_mask;
-    m.wfmt = (a->weight_dtype == MOE_DT_FP8_E5M2) ? MX_WFMT_E5M2 : MX_WFMT_E4M3;
+    m.wfmt = (a->weight_dtype == MOE_DT_FP8_E5M2) ? MX_WFMT_E5M2 : (a->weight_dtype == MOE_DT_FP4_E2M1) ? MX_WFMT_E2M1 : MX_WFMT_E4M3;
     for (int i = 0; i < 4; ++i) m.clamp[i] = g.clamp[i];
   }
   const unsigned gyc = (unsigned)bk.max_chunks;

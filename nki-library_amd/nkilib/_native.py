@@ -16,7 +16,7 @@ from .core.utils.kernel_assert import kernel_assert
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libmoe_gfx950.so")
 
 # element types (MOE_DT_*)
-DT_BF16, DT_FP16, DT_FP32, DT_FP8, DT_FP8_E5M2 = 0, 1, 2, 3, 4
+DT_BF16, DT_FP16, DT_FP32, DT_FP8, DT_FP8_E5M2, DT_FP4_E2M1 = 0, 1, 2, 3, 4, 5
 # MOE_KIND_*
 KIND_BF16, KIND_FP8_ROW, KIND_MXFP8 = 0, 1, 2
 # MOE_MX_LAYOUT_*

@@ -60,7 +60,7 @@ def _bwmm_shard_on_block_mx(
     """Returns bf16 ``[2, T+1, H]`` with the result in ``[0]`` (``[1]`` is zero).
 
     gate_up_proj_weight: MXFP8 (e4m3 or e5m2) x4 ``[E, 128, 2, H/512, I]`` (4-byte elements, or uint8 with a
-    trailing axis of 4); gate_up_proj_scale uint8 ``[E, 16, 2, H/512, I]``; down_proj_weight x4
+    trailing axis of 4) or MXFP4 x4 (2-byte elements: four 4-bit values each); gate_up_proj_scale uint8 ``[E, 16, 2, H/512, I]``; down_proj_weight x4
     ``[E, p_I, ceil(I/512), H]``; down_proj_scale uint8 ``[E, ceil(p_I/8), ceil(I/512), H]``;
     biases ``[E, p_I, 2, ceil(I/512), 4]`` and ``[E, H]``.  ``n_static_blocks`` /
     ``n_dynamic_blocks`` tune the reference's loop structure and are ignored; ``conditions``
@@ -73,10 +73,16 @@ def _bwmm_shard_on_block_mx(
                   "gate_up_proj_scale and down_proj_scale are required for MX weights")
     # the element format of the x4 weights: the reference reads it off the tensor's nl dtype or takes
     # it from ``weight_dtype`` for uint containers; here it is ``weight_dtype`` (a name containing
-    # "e5m2", or torch.float8_e5m2), else the weight tensor's torch dtype, else e4m3
-    wd = str(weight_dtype) if weight_dtype is not None else str(getattr(gate_up_proj_weight, "dtype", ""))
-    kernel_assert("float4" not in wd, f"MXFP4 weights are not supported on gfx950 yet, got weight_dtype={weight_dtype}")
-    wdt = nv.DT_FP8_E5M2 if "e5m2" in wd else nv.DT_FP8
+    # "float4" or "e5m2", or a torch float8 dtype), else the weight tensor's own dtype (2-byte elements
+    # are MXFP4, torch.float8_e5m2 is e5m2), else e4m3
+    if weight_dtype is not None:
+        wd = str(weight_dtype)
+    else:
+        wd = str(getattr(gate_up_proj_weight, "dtype", ""))
+        if getattr(gate_up_proj_weight, "element_size", lambda: 0)() == 2:
+            wd = "float4_e2m1fn_x4"
+    wdt = nv.DT_FP4_E2M1 if "float4" in wd else (nv.DT_FP8_E5M2 if "e5m2" in wd else nv.DT_FP8)
+    wbytes = 2 if wdt == nv.DT_FP4_E2M1 else 4  # bytes of an x4 element
     hidden_states = nv.require_device_tensor(hidden_states, "hidden_states")
     kernel_assert(hidden_states.dim() == 2, f"hidden_states must be [T+1, H] but got {tuple(hidden_states.shape)}")
     T1, H = hidden_states.shape
@@ -95,10 +101,13 @@ def _bwmm_shard_on_block_mx(
     pI = 128 if I > 512 else I // 4
     kernel_assert(I % 16 == 0, f"down_proj_weight I must be divisible by 16, found {I} . Please pad it")
     kernel_assert(I % 512 == 0 or (I % 512) % 32 == 0, f"I tail must be a multiple of 32, found {I}")
-    kernel_assert(guw.numel() == E * 128 * 2 * (H // 512) * I * 4,
-                  f"gate_up_proj_weight must be x4 [E={E}, 128, 2, {H // 512}, {I}] but holds {guw.numel()} bytes")
-    kernel_assert(dw.numel() == E * pI * nI * H * 4,
-                  f"down_proj_weight must be x4 [E={E}, {pI}, {nI}, {H}] but holds {dw.numel()} bytes")
+    kernel_assert(guw.numel() == E * 128 * 2 * (H // 512) * I * wbytes,
+                  f"gate_up_proj_weight must be x4 [E={E}, 128, 2, {H // 512}, {I}] of {wbytes}-byte elements "
+                  f"but holds {guw.numel()} bytes")
+    kernel_assert(dw.numel() == E * pI * nI * H * wbytes,
+                  f"down_proj_weight must be x4 [E={E}, {pI}, {nI}, {H}] of {wbytes}-byte elements but holds {dw.numel()} bytes")
+    kernel_assert(wdt == nv.DT_FP8 or (H % 512 == 0 and I % 128 == 0),
+                  f"e5m2 / MXFP4 weights need I % 128 == 0 on gfx950, found I={I}")
     kernel_assert(tuple(ds.shape) == (E, (pI + 7) // 8, nI, H),
                   f"down_proj_scale must be [{E}, {(pI + 7) // 8}, {nI}, {H}] but got {tuple(ds.shape)}")
     if gate_and_up_proj_bias is not None:

@@ -25,8 +25,8 @@ both goldens for all-zero blocks' data (zeros).  Parity unpinned for
 
 import numpy as np
 
-from .numerics import (E4M3FN_MAX, E5M2_MAX, e4m3fn_decode, e4m3fn_encode, e5m2_decode, e5m2_encode,
-                       float32_exponent_field)
+from .numerics import (E2M1_MAX, E4M3FN_MAX, E5M2_MAX, e2m1_decode, e2m1_encode, e4m3fn_decode, e4m3fn_encode,
+                       e5m2_decode, e5m2_encode, float32_exponent_field)
 
 Q_HEIGHT = 8  # partitions per block
 Q_WIDTH = 4  # packed free elements per block
@@ -36,6 +36,7 @@ E4M3_MAX_EXP = 8  # 448 = 1.75 * 2**8
 FORMATS = {
     "e4m3": (E4M3_MAX_EXP, E4M3FN_MAX, e4m3fn_encode, e4m3fn_decode),
     "e5m2": (15, E5M2_MAX, e5m2_encode, e5m2_decode),
+    "e2m1": (2, E2M1_MAX, e2m1_encode, e2m1_decode),  # MXFP4: one 4-bit pattern per uint8 here
 }
 
 

@@ -128,6 +128,42 @@ def e5m2_encode(x):
     return (code.astype(np.uint8) | (sign << 7)).reshape(x.shape)
 
 
+# float4_e2m1fn: S(1) E(2) M(1), bias 1, no inf / NaN; index = 4-bit pattern
+# (src/nkilib_src/nkilib/core/utils/mx_torch_common.py:32-66)
+E2M1_TABLE = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0],
+                      dtype=np.float32)
+E2M1_MAX = 6.0
+
+
+def e2m1_decode(codes):
+    """4-bit patterns (one per uint8, values 0..15) -> float32 (exact)."""
+    return E2M1_TABLE[np.asarray(codes, dtype=np.uint8) & 0xF]
+
+
+def e2m1_encode(x):
+    """float32 -> 4-bit patterns (one per uint8), nearest value, ties to the even mantissa, saturating at
+    +-6.  Only used to make test weights: the reference packs with the absent ``neuron_dtypes.static_cast``,
+    whose tie rule is unknown; what both sides of a parity test consume are the codes."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    a = np.minimum(np.abs(x).astype(np.float64), 6.0)
+    mag = E2M1_TABLE[:8].astype(np.float64)
+    # midpoints between neighbours; a tie goes to the neighbour with even code (mantissa bit 0)
+    mids = (mag[:-1] + mag[1:]) / 2
+    idx = np.searchsorted(mids, a, side="left")  # a == mid -> lower neighbour
+    tie = np.isin(a, mids)
+    lower_even = (idx % 2) == 0
+    idx = np.where(tie & ~lower_even, idx + 1, idx)
+    sign = (np.signbit(x)).astype(np.uint8)
+    return (idx.astype(np.uint8) | (sign << 3)).reshape(x.shape)
+
+
+def pack_e2m1_x4(codes):
+    """[..., 4] 4-bit patterns -> uint16 x4 elements, value q in bits 4q..4q+3 (mx_torch_common.py:69-81)."""
+    c = np.asarray(codes, dtype=np.uint16)
+    assert c.shape[-1] == 4
+    return (c[..., 0] | (c[..., 1] << 4) | (c[..., 2] << 8) | (c[..., 3] << 12)).astype(np.uint16)
+
+
 def e8m0_decode(b):
     """uint8 E8M0 -> float64 power of two, 2**(b-127)."""
     return np.power(2.0, np.asarray(b).astype(np.int32) - 127)

@@ -201,8 +201,13 @@ def _run_mx_direct(c, weight_dtype):
     if "gate_up_bias" in c:
         kw["gate_and_up_proj_bias"] = bf16_tensor(c["gate_up_bias"], dev)
         kw["down_proj_bias"] = bf16_tensor(c["down_bias"], dev)
-    gu = torch.from_numpy(c["gate_up_q"].view(np.int32).reshape(c["gate_up_q"].shape[:-1])).to(dev)
-    dw = torch.from_numpy(c["down_q"].view(np.int32).reshape(c["down_q"].shape[:-1])).to(dev)
+    if c.get("weight_format") == "e2m1":  # one 4-bit pattern per byte in the case; 2-byte x4 elements on the device
+        from oracle.numerics import pack_e2m1_x4
+        gu = torch.from_numpy(pack_e2m1_x4(c["gate_up_q"]).view(np.int16)).to(dev)
+        dw = torch.from_numpy(pack_e2m1_x4(c["down_q"]).view(np.int16)).to(dev)
+    else:
+        gu = torch.from_numpy(c["gate_up_q"].view(np.int32).reshape(c["gate_up_q"].shape[:-1])).to(dev)
+        dw = torch.from_numpy(c["down_q"].view(np.int32).reshape(c["down_q"].shape[:-1])).to(dev)
     out = bwmm_shard_on_block_mx[2](
         bf16_tensor(c["hidden"], dev), bf16_tensor(c["aff"].reshape(-1, 1), dev), gu, dw,
         i32_tensor(c["tp2id"], dev), i32_tensor(c["b2e"], dev), gate_up_proj_scale=u8_tensor(c["gate_up_s"], dev),
@@ -254,6 +259,20 @@ def test_mx_e5m2_weights(T, H, I, E, k, B, bias):
     # the same bytes read as e4m3 give a different answer: the format switch is what the result depends on
     o4 = from_bf16_tensor(_run_mx_direct(c, "float8_e4m3fn_x4"))
     assert max_abs_rel(o4[0, :T], g[:T]) > 0.1
+
+
+@pytest.mark.parametrize("T,H,I,E,k,B,bias,wd", [
+    (256, 512, 512, 8, 2, 128, False, "float4_e2m1fn_x4"),
+    (300, 1024, 384, 2, 2, 128, True, None),           # 300-row chunks; format inferred from the 2-byte elements
+    (512, 2048, 768, 16, 4, 256, True, "float4_e2m1fn_x4"),
+])
+def test_mx_fp4_weights(T, H, I, E, k, B, bias, wd):
+    """MXFP4 weights (nl.float4_e2m1fn_x4, the first ten cases of test_moe_bwmm_mx_cte.py:60-70): 2-byte x4 elements,
+    E8M0 scales as for MXFP8, activations and intermediate in MXFP8 e4m3."""
+    c = mx_case(T, H, I, E, k, B, seed=12, bias=bias, weight_format="e2m1", weight_std=0.5)
+    o = from_bf16_tensor(_run_mx_direct(c, wd))
+    g = _golden_mx(c)
+    _check(o[0, :T], g[:T], f"mx fp4 H={H} I={I} E={E}")
 
 
 def test_mx_prequantised_equals_online():

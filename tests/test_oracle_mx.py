@@ -138,3 +138,16 @@ def test_mx_matmul_mixed_formats_is_the_plain_product():
     bd = mx.dequantize_mx(bq, bsc).astype(np.float64).reshape(32, 8, 4)
     want = np.einsum("kiq,kjq->ij", ad, bd)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_e2m1_block_scale_closed_forms():
+    """MXFP4 target (largest exponent 2, largest value 6): ones -> scale byte 127 - 2, code of 4.0; the format maximum
+    times 2**n survives a round trip with scale 127 - 2 + n."""
+    d, s = mx.quantize_mx(np.ones((8, 4), np.float32), fmt="e2m1")
+    assert s[0, 0] == 125 and (d == 0x6).all()
+    assert np.array_equal(mx.dequantize_mx(d, s, fmt="e2m1"), np.ones((8, 4), np.float32))
+    x = np.zeros((8, 4), np.float32)
+    x[0, 0], x[1, 1], x[2, 2] = 6 * 2.0**-3, -1.5 * 2.0**-3, 0.5 * 2.0**-3
+    d, s = mx.quantize_mx(x, fmt="e2m1")
+    assert s[0, 0] == 127 - 3 and d[0, 0] == 0x7 and d[1, 1] == 0xB and d[2, 2] == 0x1
+    assert np.array_equal(mx.dequantize_mx(d, s, fmt="e2m1"), x)

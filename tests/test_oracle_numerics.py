@@ -59,6 +59,25 @@ def test_e5m2_encode_matches_torch_rne_on_random_and_boundaries():
     assert np.array_equal(nm.e5m2_encode(nm.e5m2_decode(codes)), codes)
 
 
+def test_e2m1_table_is_the_closed_form_and_encode_is_nearest():
+    codes = np.arange(16, dtype=np.uint8)
+    s_, e_, m_ = (codes >> 3) & 1, (codes >> 1) & 3, codes & 1
+    closed = np.where(e_ == 0, m_ * 0.5, (1 + m_ / 2) * 2.0 ** (e_.astype(np.float64) - 1)) * np.where(s_ == 1, -1.0, 1.0)
+    assert np.array_equal(nm.e2m1_decode(codes), closed.astype(np.float32))
+    assert np.array_equal(nm.e2m1_encode(nm.e2m1_decode(codes)) & 7, codes & 7)
+    rng = np.random.default_rng(4)
+    x = np.concatenate([rng.uniform(-7, 7, 20000), [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -2.5]]).astype(np.float32)
+    got = nm.e2m1_decode(nm.e2m1_encode(x)).astype(np.float64)
+    best = np.abs(nm.E2M1_TABLE[None, :8].astype(np.float64) - np.minimum(np.abs(x), 6.0)[:, None].astype(np.float64)).min(axis=1)
+    assert np.allclose(np.abs(np.abs(got) - np.minimum(np.abs(x), 6.0)), best) and np.array_equal(np.signbit(got), np.signbit(x))
+    # ties go to the even mantissa: 0.25 -> 0, 0.75 -> 1, 1.25 -> 1, 1.75 -> 2, 2.5 -> 2, 3.5 -> 4, 5 -> 4
+    assert list(nm.e2m1_decode(nm.e2m1_encode(np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], np.float32)))) == [0, 1, 1, 2, 2, 4, 4]
+    # packing: value q in bits 4q..4q+3, the inverse of the reference's unpack
+    p = nm.pack_e2m1_x4(np.array([[1, 2, 3, 15]], np.uint8))
+    assert p[0] == (1 | 2 << 4 | 3 << 8 | 15 << 12)
+    assert [(int(p[0]) >> (4 * q)) & 0xF for q in range(4)] == [1, 2, 3, 15]
+
+
 def test_bf16_round_matches_torch():
     rng = np.random.default_rng(1)
     x = (rng.standard_normal(300000) * rng.choice([1e-20, 1e-3, 1.0, 1e4, 1e30], 300000)).astype(np.float32)
