@@ -43,13 +43,16 @@ def parse_args():
     ap.add_argument("--with-router", action="store_true",
                     help="start from hidden states: time the router top-k front end (synthetic router weights) as a "
                          "stage of its own and route with its output; the headline metric stays the MoE layer")
+    ap.add_argument("--weights", default="mxfp8", choices=["mxfp8", "mxfp4"],
+                    help="mxfp8: e4m3 expert weights (the reported workload); mxfp4: float4_e2m1fn_x4 weights, same "
+                         "layer (diagnostic: half the weight bytes; no CPU baseline)")
     ap.add_argument("--routing", default="router", choices=["router", "balanced"],
                     help="router: top-k of synthetic scores (the reported workload); balanced: every expert gets "
                          "exactly T*k/E rows (diagnostic, shows the cost of ragged expert loads)")
     return ap.parse_args()
 
 
-def build_workload(name, dev, routing="router"):
+def build_workload(name, dev, routing="router", weights="mxfp8"):
     import torch
     from nkilib import synthetic as syn
 
@@ -63,7 +66,10 @@ def build_workload(name, dev, routing="router"):
     assert cfg["kind"] == "mxfp8", "bench.py times the MXFP8 layer (configs c3, c4, c5-<T>)"
     T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
     t0 = time.time()
-    gu_q, gu_s, d_q, d_s = syn.mx_expert_weights(E, H, I, 0.02, dev, seed=0)
+    if weights == "mxfp4":
+        gu_q, gu_s, d_q, d_s = syn.mx4_expert_weights(E, H, I, dev, seed=0)
+    else:
+        gu_q, gu_s, d_q, d_s = syn.mx_expert_weights(E, H, I, 0.02, dev, seed=0)
     ids, aff = syn.route(T, E, k, dev, seed=0, **router_kw)
     if routing == "balanced":
         tt = torch.arange(T, device=dev).reshape(T, 1)
@@ -141,12 +147,14 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     dev = torch.device("cuda:0")
     nv.check(nv.lib().moe_check_device(), "device check")
-    cfg, t = build_workload(args.workload, dev, args.routing)
+    cfg, t = build_workload(args.workload, dev, args.routing, args.weights)
+    fp4 = args.weights == "mxfp4"
+    wb = 0.5 if fp4 else 1.0  # bytes per weight value
     T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
     N = get_n_blocks(T, k, E, B, n_block_per_iter=2)
     spec = MoECTESpec(implementation=MoECTEImplementation.shard_on_block_mx)
     qcfg = QuantizationConfig(t["gu_s"], t["d_s"])
-    gu_x4 = t["gu_q"].view(torch.int32).reshape(t["gu_q"].shape[:-1])
+    gu_x4 = t["gu_q"] if fp4 else t["gu_q"].view(torch.int32).reshape(t["gu_q"].shape[:-1])
 
     names = ["norm_quant", "build_blocks", "prep", "gate_up", "down", "combine"]
     if args.with_router:
@@ -207,7 +215,7 @@ def main():
     tflops = flops_layer / (ms_per_step * 1e-3) / 1e12
     gate_up_tflops = flops_gate_up / (stage_ms["gate_up"] * 1e-3) / 1e12
     e_hit = int(torch.unique(t["ids"]).numel())
-    weight_bytes = e_hit * 3 * H * I * (1 + 1 / 32)
+    weight_bytes = e_hit * 3 * H * I * (wb + 1 / 32)
     # HBM-bound front end: bytes = rows*H*(2 in + 1 out) + scales
     nq_gbs = (T + 1) * H * (3 + 1 / 32) / (stage_ms["norm_quant"] * 1e-3) / 1e9
     comb_gbs = (routed * H * 2 + (T + 1) * H * 2) / (stage_ms["combine"] * 1e-3) / 1e9
@@ -217,11 +225,11 @@ def main():
     #   bytes = expert weights hit (2*H*I fp8 + E8M0 scales) + routed activation rows (H fp8 + scales)
     #           + re-quantised intermediate rows written (I fp8 + scales)
     # The roof that binds is the one with the larger time floor at MI355X's published peaks.
-    gu_bytes = e_hit * 2 * H * I * (1 + 1 / 32) + routed * H * (1 + 1 / 32) + routed * I * (1 + 1 / 32)
+    gu_bytes = e_hit * 2 * H * I * (wb + 1 / 32) + routed * H * (1 + 1 / 32) + routed * I * (1 + 1 / 32)
     gu_s = stage_ms["gate_up"] * 1e-3
     floor_mfma = flops_gate_up / (PEAK_FP8_TFLOPS * 1e12)
     floor_hbm = gu_bytes / (PEAK_HBM_GBS * 1e9)
-    measured = MEASURED_TRAFFIC.get((args.workload, args.routing))
+    measured = None if fp4 else MEASURED_TRAFFIC.get((args.workload, args.routing))
     if floor_hbm >= floor_mfma:
         roofline = {"bound": "hbm", "achieved": round(gu_bytes / gu_s / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(gu_bytes / gu_s / 1e9 / PEAK_HBM_GBS, 4)}
@@ -249,9 +257,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "mxfp8_e4m3 (E8M0 block scales, fp32 accumulate)",
+        "dtype": ("mxfp8_e4m3 activations x mxfp4_e2m1 weights" if fp4 else "mxfp8_e4m3") + " (E8M0 block scales, fp32 accumulate)",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: MXFP8 blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} "
+        "config": {"workload": f"{args.workload}: {'MXFP4-weight' if fp4 else 'MXFP8'} blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} "
                                f"(N={N} blocks, {routed} routed rows), RMSNorm->MXFP8 front end + block build + "
                                f"gate/up + down + combine",
                    "T": T, "H": H, "I": I, "E": E, "top_k": k, "block_size": B},
@@ -268,7 +276,7 @@ def main():
         },
         "roofline": roofline,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not fp4:
         res["cpu_baseline"] = cpu_baseline(cfg, t, tp2id, b2e, args.cpu_blocks)
     print(json.dumps(res), flush=True)
 

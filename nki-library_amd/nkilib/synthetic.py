@@ -66,6 +66,22 @@ def mx_expert_weights(E, H, I, std, device, seed=0):
     return gu_q, gu_s, d_q, d_s
 
 
+def mx4_expert_weights(E, H, I, device, seed=0):
+    """Random MXFP4 expert weights for timing runs: uniformly random 4-bit patterns in the reference's x4 layouts with
+    2-byte elements (gate_up int16 [E,128,2,H/512,I], down int16 [E,p_I,ceil(I/512),H]) and one E8M0 scale
+    (2**-8: values up to 6/256) everywhere."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    nH, nI = H // 512, math.ceil(I / 512)
+    pI = 128 if I > 512 else I // 4
+    pI8 = math.ceil(pI / 8) * 8
+    gu_q = torch.randint(-32768, 32768, (E, 128, 2, nH, I), generator=g, device=device, dtype=torch.int16)
+    d_q = torch.randint(-32768, 32768, (E, pI, nI, H), generator=g, device=device, dtype=torch.int16)
+    gu_s = torch.full((E, 16, 2, nH, I), 119, dtype=torch.uint8, device=device)
+    d_s = torch.full((E, pI8 // 8, nI, H), 119, dtype=torch.uint8, device=device)
+    return gu_q, gu_s, d_q, d_s
+
+
 def fp8_channel_weights(E, H, I, std, device, seed=0):
     """~N(0, std) weights quantised to e4m3 (range 240) with per-output-channel fp32 scales (BASELINE config 2)."""
     g = torch.Generator(device=device)
