@@ -216,7 +216,7 @@ __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, 
     asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen nt" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 // 16 bytes per lane straight into LDS at lds + 16 * lane (no destination registers).
 __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v4i& rsrc, int soff) {
