@@ -765,6 +765,14 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     const int rowb = uni(a.H * 2);
     typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
     typedef float v2f __attribute__((ext_vector_type(2)));
+    // the affinities of the lane's rows (4 consecutive rows per row tile), all requested before the
+    // first is used: a read per store, waited for on the spot, made the LDS latency the epilogue's pace
+    v4f aff4[NMT];
+#pragma unroll
+    for (int mt = 0; mt < NMT; ++mt) {
+      aff4[mt] = *(const v4f*)(s_aff + mt * 16 + 4 * g);
+      if (!post) aff4[mt] = (v4f){1.f, 1.f, 1.f, 1.f};
+    }
     static_for<0, NMT>([&](auto mt_) {
       constexpr int mt = decltype(mt_)::value;
       float av[4][4];  // [column tile][row]
@@ -775,8 +783,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       });
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int row = mt * 16 + 4 * g + r;
-        const float af = post ? s_aff[row] : 1.f;
+        const float af = aff4[mt][r];
         v2i o;
 #pragma unroll
         for (int t = 0; t < 4; t += 2) {
@@ -796,7 +803,7 @@ template <int STAGE, int WFMT>
 __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   __shared__ int s_tok[MX_ROWS_MAX];
-  __shared__ float s_aff[MX_ROWS_MAX];
+  __shared__ __attribute__((aligned(16))) float s_aff[MX_ROWS_MAX];
   // Workgroups are handed to the 8 XCDs round-robin by linear index, and each XCD has its own L2.
   // XCD x therefore takes the x-th contiguous eighth of the chunk list (chunks are ordered by
   // expert), and walks it chunk by chunk with the column tiles innermost: the workgroups that share
