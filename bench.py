@@ -29,7 +29,7 @@ PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the gate/up kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by
 # the copy-kernel calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); see profiles/ for the runs they come from.
-MEASURED_TRAFFIC = {("c4", "router"): 8520000000}
+MEASURED_TRAFFIC = {("c4", "router"): 8530000000}
 
 
 def parse_args():
