@@ -1,38 +1,40 @@
-// MXFP8 blockwise expert GEMMs for gfx950, large-tile version.
+// MX (MXFP8 / MXFP4 weights, MXFP8 activations) blockwise expert GEMMs for gfx950, large-tile version.
 //
-// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 256 consecutive
-// slots of one expert (two 128-token blocks) and 256 output columns:
+// A 256-thread workgroup (4 waves, one per SIMD) owns an "expert chunk" of up to 320 consecutive
+// slots of one expert and 256 output columns:
 //   gate/up: 32 intermediate partitions p x 4 q, for gate and for up; wave w owns q = w
 //   down:    256 hidden columns; wave w owns 64 of them
-// so every weight byte that enters the CU is used by 256 rows, and both operands enter the CU
-// exactly once per workgroup: the bytes a CU pulls through its L1 per flop are what bounds this
-// kernel (smaller or split tiles were measured: 128-row workgroups double the traffic into the
-// CU and, because sibling workgroups drift apart by more K slices than the L2 holds, the traffic
-// over the fabric as well).  Each wave keeps a 256 x 64 accumulator tile (16 x 4 MFMA 16x16
-// tiles, 256 accumulator registers).
+// so every weight byte that enters the CU is used by all rows of the chunk, and both operands enter
+// the CU exactly once per workgroup (smaller or split tiles were measured: 128-row workgroups double
+// the traffic into the CU and, because sibling workgroups drift apart by more K slices than the L2
+// holds, the traffic over the fabric as well).  A wave accumulates rows x 64 columns: 16 x 4 MFMA
+// tiles in the 256 accumulation registers, plus 4 x 4 tiles in ordinary registers for chunks of
+// 257..320 rows.
 //
-// With one wave per SIMD nothing overlaps unless the instruction stream says so:
-//   * the loads of the coming K slices are issued a few at a time between the MFMA groups of slice ks
-//     (a burst of loads blocks the wave at the issue stage for thousands of cycles while the
-//     matrix pipe drains);
+// With one wave per SIMD nothing overlaps unless the instruction stream says so, so the K loop is
+// written as a fixed sequence of instructions (MFMAs, loads, waits) around which the compiler only
+// allocates registers:
+//   * the loads of slice ks+D (D = 3, or 2 for 320-row chunks) are issued one by one between the
+//     MFMAs of slice ks (a burst of loads blocks the wave at the issue stage while the matrix pipe
+//     drains);
 //   * expert weights (B operand) go global -> registers, never through LDS.  In the reference
-//     layout a weight column's K runs over partitions p (4 K-bytes per 4-byte element), and lane
+//     layout a weight column's K runs over partitions p (4 K values per x4 element), and lane
 //     group g of v_mfma_scale_f32_16x16x128_f8f6f4 needs K bytes [16g,16g+16) and [64+16g,
 //     64+16g+16) of the 128-byte K slice, i.e. partitions 4g..4g+3 and 16+4g..16+4g+3 of the 32
-//     partitions of the slice: eight loads per lane, each fetching 2 (gate/up) or 4 (down)
-//     adjacent columns = 2 or 4 MFMA column tiles at once.  One load instruction reads four
-//     full 128/256-byte row segments.  The loads land in one of two "raw" register sets, two
-//     slices ahead; a set is transposed into MFMA operand order at the top of the slice that uses
-//     it;
-//   * activations (A operand, rows gathered through token_position_to_id) are staged through a
-//     three-deep LDS ring of 256 rows x 128 K-bytes, read by all four waves; the fragments of the
-//     next two row tiles are read while the current two multiply;
-//   * E8M0 scales ride along: A scales sit in LDS transposed to [g][row%16][row/16] so that one
-//     16-byte read gives a lane the scales of all 16 row tiles (selected with op_sel); B scales
-//     are 2-4 bytes per lane per K slice straight from global.
-// The gate/up epilogue computes act(gate)*up in registers (a lane holds gate and up of the same
-// element) and exchanges the products through LDS so that the MX re-quantisation sees the
-// reference's blocks (8 partitions x 4 q) and writes K-contiguous rows for the down GEMM.
+//     partitions of the slice (4-bit weights: K 32g..32g+31 = partitions 8g..8g+7): eight loads
+//     per lane, each fetching 4 adjacent columns = 4 MFMA column tiles at once.  The loads land in
+//     one of D "raw" register sets; a set is transposed into MFMA operand order at the top of the
+//     slice that uses it;
+//   * activations (A operand, rows gathered through token_position_to_id) go global -> LDS
+//     directly into a ring of D+1 stages of 256 (320) rows x 128 K-bytes, read by all four waves;
+//     the fragments of the next two row tiles are read while the current two multiply;
+//   * E8M0 scales ride along: A scales sit in LDS as [g][row%16][row/16] so that one 16-byte read
+//     gives a lane the scales of 16 row tiles (selected with op_sel); B scales are 4 bytes per lane
+//     per K slice straight from global.
+// The gate/up epilogue computes act(gate)*up in registers (a pair of lanes holds gate and up of the
+// same elements and exchanges them) and passes the products through LDS so that the MX
+// re-quantisation sees the reference's blocks (8 partitions x 4 q) and writes K-contiguous rows for
+// the down GEMM.
 //
 // Reference semantics: test/integration/nkilib/core/mlp/test_mlp_common.py:550-682 (layouts,
 // re-quantisation), test/integration/nkilib/core/moe/moe_cte/test_utils.py:474-735 (block loop).
