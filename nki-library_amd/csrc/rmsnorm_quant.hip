@@ -160,7 +160,10 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
 // contiguous elements at h = q*(H/4) + tile*128 + p8*8 + r.
 constexpr int MXQ_MAX_BLK = RQ_MAX_H / 32 / RQ_THREADS;  // 2
 
-__global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
+// MAXB = MX blocks per thread (1 for H <= 32 * RQ_THREADS: half the registers, twice the rows in flight per CU:
+// a row is one load round trip, one reduction and one store, so rows in flight are what fills the memory pipeline).
+template <int MAXB>
+__global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? 5 : 3, 8))) void rmsnorm_quant_mx_kernel(
     const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
     uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, uint16_t* __restrict__ out_norm, int64_t rows,
     int64_t H, float eps, float hidden_actual, int do_norm, int layout) {
@@ -172,10 +175,10 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
   const int nT = (int)(H / 512);
   const int64_t Hq = H / 4;
 
-  float v[MXQ_MAX_BLK][4][8];
+  float v[MAXB][4][8];
   double ss = 0.0;
 #pragma unroll
-  for (int j = 0; j < MXQ_MAX_BLK; ++j) {
+  for (int j = 0; j < MAXB; ++j) {
     const int blk = j * RQ_THREADS + threadIdx.x;
     if (blk < nblk) {
       const int tile = blk >> 4, p8 = blk & 15;
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_mx_kernel(
     inv = 1.0f / rms;
   }
 #pragma unroll
-  for (int j = 0; j < MXQ_MAX_BLK; ++j) {
+  for (int j = 0; j < MAXB; ++j) {
     const int blk = j * RQ_THREADS + threadIdx.x;
     if (blk < nblk) {
       const int tile = blk >> 4, p8 = blk & 15;
@@ -292,9 +295,14 @@ extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* g
     return MOE_E_BAD_ARG;
   if (rows == 0) return MOE_OK;
   const float ha = (float)(hidden_actual > 0 ? hidden_actual : H);
-  hipLaunchKernelGGL(rmsnorm_quant_mx_kernel, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
-                     x_dtype, gamma, gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H,
-                     eps, ha, do_norm, layout);
+  if (H <= 32 * RQ_THREADS)
+    hipLaunchKernelGGL(rmsnorm_quant_mx_kernel<1>, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
+                       x_dtype, gamma, gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H,
+                       eps, ha, do_norm, layout);
+  else
+    hipLaunchKernelGGL(rmsnorm_quant_mx_kernel<MXQ_MAX_BLK>, dim3((unsigned)rows), dim3(RQ_THREADS), 0,
+                       (hipStream_t)stream, x, x_dtype, gamma, gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale,
+                       (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
 }
