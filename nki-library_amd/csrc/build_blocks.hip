@@ -55,8 +55,8 @@ __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __r
 
 // ws layout: counts[E] | first_slot[E] | n_padding[1]
 // One workgroup: blocks per expert (padding blocks to the last expert, or split), exclusive scan ->
-// first slot of every expert, block_to_expert, conditions.  The scan over experts is serial (E is a
-// few hundred) but runs out of LDS; everything else is spread over the threads.
+// first slot of every expert, block_to_expert, conditions; sums and scans over the experts are
+// workgroup-wide (shuffles + one exchange), a tile of BB_THREADS experts at a time.
 __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ counts,
                                                               int32_t* __restrict__ first_slot,
                                                               int32_t* __restrict__ block_to_expert,
@@ -66,11 +66,17 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __
   extern __shared__ int s_nb[];  // [E] blocks per expert, then [E] first block of every expert
   int* s_first = s_nb + E;
   __shared__ int s_npad;
-  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) s_nb[e] = (int)((counts[e] + B - 1) / B);
-  __syncthreads();
+  __shared__ int s_ws[16];
+  // blocks per expert and their sum
+  int mine = 0;
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
+    const int nb = (int)((counts[e] + B - 1) / B);
+    s_nb[e] = nb;
+    mine += nb;
+  }
+  int used;
+  (void)block_excl_scan(mine, s_ws, &used);
   if (threadIdx.x == 0) {
-    int64_t used = 0;
-    for (int64_t e = 0; e < E; ++e) used += s_nb[e];
     int64_t npad = N - used;
     if (status) *status = npad < 0;
     if (npad < 0) npad = 0;
@@ -81,11 +87,17 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __
     } else {
       s_nb[E - 1] += (int)npad;
     }
-    int64_t blk = 0;
-    for (int64_t e = 0; e < E; ++e) {
-      s_first[e] = (int)blk;
-      blk += s_nb[e];
-    }
+  }
+  __syncthreads();
+  // first block of every expert: exclusive scan over the experts, a tile of BB_THREADS at a time
+  int carry = 0;
+  for (int64_t base = 0; base < E; base += BB_THREADS) {
+    const int64_t e = base + threadIdx.x;
+    const int v = (e < E) ? s_nb[e] : 0;
+    int total;
+    const int ex = block_excl_scan(v, s_ws, &total);
+    if (e < E) s_first[e] = carry + ex;
+    carry += total;
   }
   __syncthreads();
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {

@@ -126,26 +126,18 @@ __global__ __launch_bounds__(256) void inv_count_kernel(const int32_t* __restric
 // Exclusive scan of cnt[0..n) into off[0..n], single workgroup of 1024 threads.
 __global__ __launch_bounds__(1024) void inv_scan_kernel(const int32_t* __restrict__ cnt, int32_t* __restrict__ off,
                                                         int64_t n) {
-  __shared__ int s_part[1024];
-  const int64_t per = (n + 1023) / 1024;
-  const int64_t lo = threadIdx.x * per, hi = (lo + per < n) ? lo + per : n;
-  int sum = 0;
-  for (int64_t i = lo; i < hi; ++i) sum += cnt[i];
-  s_part[threadIdx.x] = sum;
-  __syncthreads();
-  // Hillis-Steele inclusive scan over the 1024 partials
-  for (int o = 1; o < 1024; o <<= 1) {
-    int v = (threadIdx.x >= (unsigned)o) ? s_part[threadIdx.x - o] : 0;
-    __syncthreads();
-    s_part[threadIdx.x] += v;
-    __syncthreads();
+  __shared__ int s_ws[16];
+  // thread t owns elements t, t + 1024, ... of each 1024-element tile: coalesced, one scan per tile
+  int carry = 0;
+  for (int64_t base = 0; base < n; base += 1024) {
+    const int64_t i = base + threadIdx.x;
+    const int v = (i < n) ? cnt[i] : 0;
+    int total;
+    const int ex = block_excl_scan(v, s_ws, &total);
+    if (i < n) off[i] = carry + ex;
+    carry += total;
   }
-  int run = s_part[threadIdx.x] - sum;
-  for (int64_t i = lo; i < hi; ++i) {
-    off[i] = run;
-    run += cnt[i];
-  }
-  if (threadIdx.x == 1023) off[n] = s_part[1023];
+  if (threadIdx.x == 0) off[n] = carry;
 }
 
 __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict__ tp2id,

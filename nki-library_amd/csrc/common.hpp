@@ -114,6 +114,29 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return t;
 }
 
+// Exclusive prefix sum of v over the workgroup (blockDim.x a multiple of 64, at most 1024): shuffles
+// inside a wave, one exchange of the wave totals through `ws` (16 ints).  *total = sum over the workgroup.
+__device__ __forceinline__ int block_excl_scan(int v, int* ws, int* total) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += t;
+  }
+  __syncthreads();  // `ws` may still be read from a previous call
+  if (lane == 63) ws[w] = inc;
+  __syncthreads();
+  int base = 0, tot = 0;
+  for (int i = 0; i < nw; ++i) {
+    const int t = ws[i];
+    base += (i < w) ? t : 0;
+    tot += t;
+  }
+  *total = tot;
+  return base + inc - v;
+}
+
 // ---- activation functions (ActFnType, common_types.py:32-36) ---------------------------
 // x * sigmoid(k x) with the hardware exp2 and reciprocal (about 1 ulp each): the library expf and
 // the IEEE division cost ~100 instructions per element, which made the gate/up epilogue as long
