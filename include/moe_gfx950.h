@@ -45,6 +45,7 @@ int moe_check_device(void);
 #define MOE_DT_FP8_E4M3 3 /* OCP e4m3fn bit patterns; Neuron float8_e4m3 is the |v|<=240 subset */
 #define MOE_DT_FP8_E5M2 4 /* OCP e5m2 bit patterns (MXFP8 weights only)                              */
 #define MOE_DT_FP4_E2M1 5 /* OCP e2m1 (MXFP4 weights only): four 4-bit values per 2-byte x4 element   */
+#define MOE_DT_INT32 6    /* the index operators only                                                */
 
 /* ---- RMSNorm + quantise front end -------------------------------------------------- */
 
@@ -121,6 +122,36 @@ int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, i
                      int skip_token, int use_split_padding, int32_t* token_position_to_id,
                      int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
                      void* workspace, size_t workspace_bytes, int32_t* status_out, void* stream);
+
+/* The reference's device-side pieces of the same construction, as separate operators
+ * (mask [T, E] -> per-expert token lists -> block offsets -> flat token_position_to_id).
+ *
+ * moe_find_nonzero_indices replaces find_nonzero_indices
+ * (src/nkilib_src/nkilib/core/subkernels/find_nonzero_indices.py:34-110; semantics
+ * find_nonzero_indices_torch_ref, find_nonzero_indices_torch.py:20-63), bit exact.  input [T, C_full]
+ * (MOE_DT_INT32 / FP32 / BF16 / FP16); columns col_start_id[0] .. + n_cols (col_start_id: device
+ * int32[1], NULL = column 0; columns outside the input count as all zero).  indices int32
+ * [n_cols, T]: per column the ascending row numbers of its nonzero elements, then -1;
+ * nonzero_counts int32 [n_cols].
+ *
+ * moe_indexed_flatten replaces indexed_flatten (src/nkilib_src/nkilib/core/subkernels/
+ * indexed_flatten.py:28-86; semantics indexed_flatten_torch_ref, indexed_flatten_torch.py:18-66).
+ * input int32 [E, T] seen as [E, T / f_len, f_len]; block p of row e goes to output block
+ * row_offsets[start + e] + p when that lies in [0, output_len / f_len) (start =
+ * row_offsets_start[0], device int32[1], NULL = 0); where rows overlap the later row wins (the
+ * reference's loop order); everything else is padding_val.  output int32 [output_len].
+ *
+ * moe_cumsum replaces cumsum (src/nkilib_src/nkilib/core/cumsum/cumsum.py:30-75; cumsum_torch.py:20-32):
+ * inclusive prefix sum along the last axis of [rows, H]; fp32 accumulation for BF16 / FP16 / FP32
+ * (result rounded to the element type), exact for MOE_DT_INT32. */
+size_t moe_find_nonzero_indices_workspace_bytes(int64_t T, int64_t n_cols);
+int moe_find_nonzero_indices(const void* input, int dtype, int64_t T, int64_t C_full, const int32_t* col_start_id,
+                             int64_t n_cols, int32_t* indices, int32_t* nonzero_counts, void* workspace,
+                             size_t workspace_bytes, void* stream);
+int moe_indexed_flatten(const int32_t* input, int64_t E, int64_t T, int64_t f_len, int64_t output_len,
+                        const int32_t* row_offsets, int64_t n_offsets, const int32_t* row_offsets_start,
+                        int32_t padding_val, int32_t* output, void* stream);
+int moe_cumsum(const void* x, void* y, int dtype, int64_t rows, int64_t H, void* stream);
 
 /* ---- blockwise MoE ------------------------------------------------------------------- */
 

@@ -16,7 +16,7 @@ from .core.utils.kernel_assert import kernel_assert
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libmoe_gfx950.so")
 
 # element types (MOE_DT_*)
-DT_BF16, DT_FP16, DT_FP32, DT_FP8, DT_FP8_E5M2, DT_FP4_E2M1 = 0, 1, 2, 3, 4, 5
+DT_BF16, DT_FP16, DT_FP32, DT_FP8, DT_FP8_E5M2, DT_FP4_E2M1, DT_INT32 = 0, 1, 2, 3, 4, 5, 6
 # MOE_KIND_*
 KIND_BF16, KIND_FP8_ROW, KIND_MXFP8 = 0, 1, 2
 # MOE_MX_LAYOUT_*
@@ -34,6 +34,10 @@ EXPORTED_SYMBOLS = (
     "moe_rmsnorm_quant_mxfp8",
     "moe_build_blocks_workspace_bytes",
     "moe_build_blocks",
+    "moe_find_nonzero_indices_workspace_bytes",
+    "moe_find_nonzero_indices",
+    "moe_indexed_flatten",
+    "moe_cumsum",
     "moe_router_topk_workspace_bytes",
     "moe_router_topk",
     "moe_blockwise_workspace_bytes",
@@ -125,6 +129,16 @@ def lib():
     L.moe_build_blocks.restype = c_int
     L.moe_build_blocks.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p,
                                    c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]
+    L.moe_find_nonzero_indices_workspace_bytes.restype = c_size_t
+    L.moe_find_nonzero_indices_workspace_bytes.argtypes = [c_int64, c_int64]
+    L.moe_find_nonzero_indices.restype = c_int
+    L.moe_find_nonzero_indices.argtypes = [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p,
+                                           c_void_p, c_size_t, c_void_p]
+    L.moe_indexed_flatten.restype = c_int
+    L.moe_indexed_flatten.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
+                                      c_int32, c_void_p, c_void_p]
+    L.moe_cumsum.restype = c_int
+    L.moe_cumsum.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p]
     L.moe_router_topk_workspace_bytes.restype = c_size_t
     L.moe_router_topk_workspace_bytes.argtypes = [c_int64, c_int64]
     L.moe_router_topk.restype = c_int
@@ -161,6 +175,14 @@ _DT = {torch.bfloat16: DT_BF16, torch.float16: DT_FP16, torch.float32: DT_FP32}
 
 def dtype_code(t, what):
     kernel_assert(t.dtype in _DT, f"{what} must be bfloat16, float16 or float32 but got {t.dtype}")
+    return _DT[t.dtype]
+
+
+def index_dtype_code(t, what):
+    """Element type code for the index operators, which also take int32."""
+    if t.dtype == torch.int32:
+        return DT_INT32
+    kernel_assert(t.dtype in _DT, f"{what} must be int32, bfloat16, float16 or float32 but got {t.dtype}")
     return _DT[t.dtype]
 
 

@@ -28,6 +28,7 @@ Modules
   numerics   bf16 / fp8-e4m3fn / E8M0 encode + decode
   mx         OCP-MX (8x4 block) quantise / dequantise / matmul goldens
   blocks     token -> block index construction (bit exact, integer)
+  index_ops  find_nonzero_indices / indexed_flatten / cumsum (bit exact, integer)
   rmsnorm    RMSNorm + fp8 ROW / STATIC quantise, RMSNorm -> MXFP8
   moe        blockwise MoE goldens (bf16, fp8-weight, fp8-row, MXFP8)
   router     router top-k (logits, top-k selection, affinities)
