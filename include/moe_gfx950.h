@@ -224,6 +224,14 @@ typedef struct moe_bwmm_args {
   int32_t skip_token;     /* 1: padding id is -1 and tables have T rows                           */
   int32_t clamp_mask;     /* MOE_CLAMP_* bits                                                     */
   float gate_clamp_upper, gate_clamp_lower, up_clamp_upper, up_clamp_lower;
+  /* Activation checkpoints of the bf16 kind (checkpoint_activation, bwmm_shard_on_I.py:160-176;
+   * golden test_moe_cte_common.py:312-314,404-405,420-421), both bf16 and nullable:
+   * gate_up_activations_T [N, 2, I, B] = gate / up projections after scale, bias and clamp, before the
+   * activation; down_activations [N, B, H] = down projection after scale and bias, before the affinity.
+   * All B rows of every executed block are written (padding rows hold what a zero input row gives),
+   * blocks that conditions stops are zero. */
+  void* gate_up_activations_T;
+  void* down_activations;
 } moe_bwmm_args;
 
 /* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /

@@ -61,7 +61,8 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
   const int b = rt / a.tiles_per_block;
   const int r0 = (rt % a.tiles_per_block) * TM;
   if (b >= *a.n_active) return;
-  const int vr = a.valid_rows[b];
+  // with checkpoint outputs every row of an executed block is computed: padding rows are zero inputs
+  const int vr = a.ckpt ? (int)a.B : a.valid_rows[b];
   if (r0 >= vr) return;
   const int e = a.b2e[b];
   const int64_t slot0 = (int64_t)b * a.B + r0;
@@ -390,6 +391,11 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
             if (a.clamp_mask & MOE_CLAMP_GATE_HI) gv = fminf(gv, a.clamp[0]);
             if (a.clamp_mask & MOE_CLAMP_UP_LO) uv = fmaxf(uv, a.clamp[3]);
             if (a.clamp_mask & MOE_CLAMP_UP_HI) uv = fminf(uv, a.clamp[2]);
+            if (KIND == MOE_KIND_BF16 && a.ckpt && iv && r0 + row < a.B) {
+              uint16_t* ck = a.ckpt + (((int64_t)b * 2) * a.I + i) * a.B + r0 + row;
+              ck[0] = f32_to_bf16_bits(gv);
+              ck[a.I * a.B] = f32_to_bf16_bits(uv);
+            }
             const float y = iv ? act_apply(gv, a.act_fn) * uv : 0.f;
             if (r0 + row < vr) {
               const int64_t slot = slot0 + row;
@@ -419,11 +425,15 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int row = m0 + 16 * mt + 4 * g + r;
-          if (s_tok[row] < 0) continue;
+          if (s_tok[row] < 0 && !(KIND == MOE_KIND_BF16 && a.ckpt)) continue;
           float d = acc[nt][mt][r];
           if (KIND == MOE_KIND_BF16) d *= sd;
           if (KIND == MOE_KIND_FP8_ROW) d = (d * sd) * __uint_as_float(sAs[row]);
           d += bd;
+          if (KIND == MOE_KIND_BF16 && a.ckpt) {
+            if (r0 + row < a.B) a.ckpt[(slot0 + row) * a.H + h] = f32_to_bf16_bits(d);
+            if (s_tok[row] < 0) continue;
+          }
           if (post) d *= s_aff[row];
           D[(slot0 + row) * a.H + h] = f32_to_bf16_bits(d);
         }

@@ -35,6 +35,7 @@ struct GemmArgs {
   int32_t act_fn, scaling_mode, clamp_mask;
   float clamp[4];          // gate hi, gate lo, up hi, up lo
   int32_t pI, nI;          // MXFP8: partitions per intermediate tile in the down weight, number of tiles
+  uint16_t* ckpt;          // BF16 kind, nullable: stage 1 gate/up checkpoint [N, 2, I, B], stage 2 down checkpoint [N, B, H]
 };
 
 // Arguments of the large-tile MXFP8 kernels (bwmm_mx.hip).

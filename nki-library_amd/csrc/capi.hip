@@ -22,7 +22,7 @@ extern "C" const char* moe_error_string(int code) {
   }
 }
 
-extern "C" int moe_abi_version(void) { return 1; }
+extern "C" int moe_abi_version(void) { return 2; }
 
 extern "C" int moe_check_device(void) {
   int dev = 0;
@@ -60,6 +60,8 @@ int validate(const moe_bwmm_args* a) {
   if (a->N * a->B >= ((int64_t)1 << 31) || a->T1 * a->E >= ((int64_t)1 << 31)) return MOE_E_BAD_SHAPE;
   const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
   if (Ipad < a->I) return MOE_E_BAD_SHAPE;
+  if ((a->gate_up_activations_T || a->down_activations) && (a->kind != MOE_KIND_BF16 || a->weight_dtype != MOE_DT_BF16))
+    return MOE_E_UNSUPPORTED;
   switch (a->kind) {
     case MOE_KIND_BF16:
       if (a->H % 8 != 0) return MOE_E_BAD_SHAPE;  // 16-byte row slices of bf16 hidden states
@@ -182,6 +184,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
   g2.W_scale = (const uint8_t*)a->down_proj_scale;
   g2.bias = a->down_proj_bias;
   g2.out = ws + p.d;
+  g1.ckpt = (uint16_t*)a->gate_up_activations_T;
+  g2.ckpt = (uint16_t*)a->down_activations;
   unsigned gx1, gx2 = (unsigned)((a->H + 127) / 128);
 
   if (a->kind == MOE_KIND_MXFP8) {
@@ -237,6 +241,15 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     for (int i = 0; i < 4; ++i) m.clamp[i] = g.clamp[i];
   }
   const unsigned gyc = (unsigned)bk.max_chunks;
+  // checkpoints of blocks that never run stay zero
+  if (a->gate_up_activations_T && (stages & MOE_STAGE_GATE_UP)) {
+    rc = launch_fill_zero_bytes(a->gate_up_activations_T, (size_t)a->N * 2 * a->I * a->B * 2, s);
+    if (rc != MOE_OK) return rc;
+  }
+  if (a->down_activations && (stages & MOE_STAGE_DOWN)) {
+    rc = launch_fill_zero_bytes(a->down_activations, (size_t)a->N * a->B * a->H * 2, s);
+    if (rc != MOE_OK) return rc;
+  }
   if (stages & MOE_STAGE_GATE_UP) {
     if (mx_fast) {
       MxArgs m1 = m;

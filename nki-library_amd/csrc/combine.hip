@@ -278,4 +278,15 @@ int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, 
   return MOE_OK;
 }
 
+int launch_fill_zero_bytes(void* p, size_t bytes, hipStream_t s) {
+  if (bytes == 0) return MOE_OK;
+  if ((bytes & 3) != 0 || ((uintptr_t)p & 3) != 0) return MOE_E_BAD_ARG;
+  const int64_t words = (int64_t)(bytes / 4);
+  const int64_t grid = (words + 255) / 256;
+  if (grid >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)grid), dim3(256), 0, s, (int32_t*)p, words);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
 }  // namespace moe

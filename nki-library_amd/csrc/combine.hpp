@@ -32,5 +32,7 @@ Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B);
 // n_real: number of real token rows (ids in [0, n_real) are tokens, everything else is padding).
 int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hipStream_t s);
 int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, int64_t n_real, hipStream_t s);
+// Zero `bytes` bytes at p (a multiple of 4, p 4-byte aligned) with a kernel, so that callers may capture it in a graph.
+int launch_fill_zero_bytes(void* p, size_t bytes, hipStream_t s);
 
 }  // namespace moe

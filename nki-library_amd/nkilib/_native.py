@@ -91,6 +91,8 @@ class BwmmArgs(ctypes.Structure):
         ("gate_clamp_lower", c_float),
         ("up_clamp_upper", c_float),
         ("up_clamp_lower", c_float),
+        ("gate_up_activations_T", c_void_p),
+        ("down_activations", c_void_p),
     ]
 
 

@@ -54,8 +54,12 @@ def run_blockwise(
     up_clamp_lower_limit: Optional[float] = None,
     weight_dtype: int = nv.DT_BF16,
     scale_experts: int = 0,
+    checkpoint_gate_up: bool = False,
+    checkpoint_down: bool = False,
 ):
-    """dims: T1, H, I, E, I_pad.  out_shape_kind: "T2H" ([T1,2,H], slot 0), "2TH" ([2,T1,H], slot 0) or "TH"."""
+    """dims: T1, H, I, E, I_pad.  out_shape_kind: "T2H" ([T1,2,H], slot 0), "2TH" ([2,T1,H], slot 0) or "TH".
+    With ``checkpoint_gate_up`` / ``checkpoint_down`` (bf16 weights only) the result is a tuple: the output, then
+    ``gate_up_activations_T`` ``[N, 2, I, B]`` and / or ``down_activations`` ``[N, B, H]`` (bfloat16)."""
     L = nv.lib()
     skip_dma = skip_dma or SkipMode(False, False)
     T1, H, I, E = dims["T1"], dims["H"], dims["I"], dims["E"]
@@ -140,6 +144,16 @@ def run_blockwise(
             mask |= bit
             setattr(a, name, float(v))
     a.clamp_mask = mask
+    ck_gu = ck_down = None
+    if checkpoint_gate_up or checkpoint_down:
+        kernel_assert(kind == nv.KIND_BF16 and weight_dtype == nv.DT_BF16,
+                      "activation checkpoints need bfloat16 hidden states and weights")
+    if checkpoint_gate_up:
+        ck_gu = torch.empty((N, 2, I, B), dtype=torch.bfloat16, device=dev)
+        a.gate_up_activations_T = nv.ptr(ck_gu)
+    if checkpoint_down:
+        ck_down = torch.empty((N, B, H), dtype=torch.bfloat16, device=dev)
+        a.down_activations = nv.ptr(ck_down)
 
     need = L.moe_blockwise_workspace_bytes(ctypes.byref(a))
     if need == 0:
@@ -165,4 +179,6 @@ def run_blockwise(
                     break
                 stage_callback(name)
     nv.check(rc, "moe_cte")
-    return out
+    if ck_gu is None and ck_down is None:
+        return out
+    return tuple(t for t in (out, ck_gu, ck_down) if t is not None)

@@ -24,8 +24,12 @@ def _blockwise_mm_baseline_shard_intermediate(
     up_clamp_lower_limit: Optional[float] = None, up_clamp_upper_limit: Optional[float] = None,
     checkpoint_activation=False, expert_affinity_multiply_on_I=False,
 ):
-    kernel_assert(not checkpoint_activation, "checkpoint_activation is not supported on gfx950")
-    kernel_assert(not expert_affinity_multiply_on_I, "expert_affinity_multiply_on_I is not supported on gfx950")
+    """``checkpoint_activation``: also returns ``gate_up_activations_T`` ``[N, 2, I, B]`` (gate / up projections
+    after scale, bias and clamp, before the activation: the golden's in-place views,
+    test_moe_cte_common.py:383-405) and, unless ``expert_affinity_multiply_on_I``, ``down_activations``
+    ``[N, B, H]`` (before the affinity, :410-421), as bwmm_shard_on_I.py:314-323 does.
+    ``expert_affinity_multiply_on_I`` itself only moves a multiplication inside the reference kernel; the one
+    golden serves both settings and so does this kernel."""
     return run_dense_variant(
         hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size,
         token_position_to_id, block_to_expert, "TH", gate_and_up_proj_bias=gate_and_up_proj_bias,
@@ -34,6 +38,8 @@ def _blockwise_mm_baseline_shard_intermediate(
         expert_affinities_scaling_mode=expert_affinities_scaling_mode,
         gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
         up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit,
+        checkpoint_gate_up=bool(checkpoint_activation),
+        checkpoint_down=bool(checkpoint_activation) and not expert_affinity_multiply_on_I,
     )
 
 
@@ -72,9 +78,26 @@ def _blockwise_mm_shard_intermediate_dropping(
     gate_clamp_lower_limit: Optional[float] = None, up_clamp_lower_limit: Optional[float] = None,
     up_clamp_upper_limit: Optional[float] = None,
 ):
-    """Token-dropping layer: N == E blocks, one per expert; the block math is unchanged.
-    The reference variant also returns checkpoint activations, which are not built."""
-    kernel_assert(False, "shard_on_i_dropping returns activation checkpoints, which are not supported on gfx950")
+    """Token-dropping layer (bwmm_shard_on_I.py:2014-2159): N == E blocks, block b belongs to expert b
+    (``block_to_expert`` is not read), tokens beyond an expert's block were dropped by the caller.  Always returns
+    the checkpoints: ``(output, gate_up_activations_T)`` with ``expert_affinity_multiply_on_I``, else
+    ``(output, gate_up_activations_T, down_activations)``."""
+    if expert_affinities_scaling_mode == ExpertAffinityScaleMode.PRE_SCALE_DELAYED:
+        expert_affinities_scaling_mode = ExpertAffinityScaleMode.PRE_SCALE  # bwmm_shard_on_I.py:2084-2085
+    E = gate_up_proj_weight.shape[0]
+    N = token_position_to_id.numel() // int(block_size)
+    kernel_assert(N == E, f"the dropping layer has one block per expert: N ({N}) must equal E ({E})")
+    own_expert = torch.arange(N, dtype=torch.int32, device=hidden_states.device)
+    return run_dense_variant(
+        hidden_states, expert_affinities_masked, gate_up_proj_weight, down_proj_weight, block_size,
+        token_position_to_id, own_expert, "TH", gate_and_up_proj_bias=gate_and_up_proj_bias,
+        down_proj_bias=down_proj_bias, gate_up_proj_scale=gate_up_proj_scale, down_proj_scale=down_proj_scale,
+        activation_function=activation_function, skip_dma=skip_dma,
+        expert_affinities_scaling_mode=expert_affinities_scaling_mode,
+        gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
+        up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit,
+        checkpoint_gate_up=True, checkpoint_down=not expert_affinity_multiply_on_I,
+    )
 
 
 blockwise_mm_baseline_shard_intermediate = KernelEntry(_blockwise_mm_baseline_shard_intermediate)

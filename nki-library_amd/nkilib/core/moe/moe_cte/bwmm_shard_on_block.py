@@ -41,7 +41,8 @@ def run_dense_variant(
     block_to_expert, out_shape_kind, conditions=None, gate_and_up_proj_bias=None, down_proj_bias=None,
     gate_up_proj_scale=None, down_proj_scale=None, activation_function=ActFnType.SiLU, skip_dma=None,
     expert_affinities_scaling_mode=ExpertAffinityScaleMode.POST_SCALE, gate_clamp_upper_limit=None,
-    gate_clamp_lower_limit=None, up_clamp_upper_limit=None, up_clamp_lower_limit=None,
+    gate_clamp_lower_limit=None, up_clamp_upper_limit=None, up_clamp_lower_limit=None, checkpoint_gate_up=False,
+    checkpoint_down=False,
 ):
     """Common body of the non-MX variants (they share one golden, test_moe_cte_common.py:267-447)."""
     hidden_states = nv.require_device_tensor(hidden_states, "hidden_states")
@@ -100,7 +101,7 @@ def run_dense_variant(
         expert_affinities_scaling_mode=expert_affinities_scaling_mode,
         gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
         up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit, weight_dtype=wdt,
-        scale_experts=scale_experts,
+        scale_experts=scale_experts, checkpoint_gate_up=checkpoint_gate_up, checkpoint_down=checkpoint_down,
     )
 
 

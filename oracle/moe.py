@@ -88,12 +88,19 @@ def moe_blockwise_ref(
     gate_clamp_lower_limit=None,
     up_clamp_upper_limit=None,
     up_clamp_lower_limit=None,
+    checkpoint_activation=False,
 ):
     """bf16 (and weight-only fp8 with per-channel scales) blockwise MoE.
 
     hidden_states [T+1, H] (or [T, H] with skip_token); weights already as float32
     values ([E, H, 2, I], [E, I_pad, H]); scales [E or 1, 1, 2I], [E or 1, 1, H].
     Returns float32 (bf16-valued) [T+1, H] (or [T, H] with skip_token).
+
+    checkpoint_activation: returns (out, gate_up_activations_T [N, 2, I, B], down_activations [N, B, H]),
+    bf16-valued float32 (test_moe_cte_common.py:312-314,404-405,420-421).  In the golden the gate and up
+    projections are views of one array that scale, bias and clip modify in place (:383-402), so the checkpoint
+    holds the values after them (moe_cte_torch.py:163-165 clones instead and keeps the bare matmul; the two agree
+    when there is no scale, bias or clamp).
     """
     E, H = gate_up_proj_weight.shape[0], gate_up_proj_weight.shape[1]
     I = gate_up_proj_weight.shape[-1]
@@ -107,6 +114,8 @@ def moe_blockwise_ref(
     w_gu = np.asarray(gate_up_proj_weight, dtype=np.float32).reshape(E, H, 2 * I)
     w_d = np.asarray(down_proj_weight, dtype=np.float32)
     quant = gate_up_proj_scale is not None
+    ck_gu = np.zeros((N, 2, I, B), dtype=np.float32)
+    ck_d = np.zeros((N, B, H), dtype=np.float32)
     for b in range(N):
         if conditions is not None and conditions[b] == 0:
             break
@@ -131,6 +140,8 @@ def moe_blockwise_ref(
             u += np.asarray(gate_up_proj_bias, dtype=np.float32)[e, 1, :]
         _clip(g, gate_clamp_lower_limit, gate_clamp_upper_limit)
         _clip(u, up_clamp_lower_limit, up_clamp_upper_limit)
+        ck_gu[b, 0] = to_bf16(g).T
+        ck_gu[b, 1] = to_bf16(u).T
         y = act_fn(g, activation_function) * u
         # down weight may be padded on I (test_moe_cte_common.py:645,663)
         d = np.matmul(y, w_d[e, :I, :]) if w_d.shape[1] != I else np.matmul(y, w_d[e])
@@ -140,10 +151,14 @@ def moe_blockwise_ref(
             d = d * s.reshape(-1)
         if down_proj_bias is not None:
             d = d + np.asarray(down_proj_bias, dtype=np.float32)[e]
+        ck_d[b] = to_bf16(d)
         if expert_affinities_scaling_mode == POST_SCALE:
             d = d * a
         _accumulate(out, ids, d.astype(np.float32))
-    return out[:T1] if skip_token else out
+    out = out[:T1] if skip_token else out
+    if checkpoint_activation:
+        return out, ck_gu, ck_d
+    return out
 
 
 def moe_blockwise_fp8_row_ref(

@@ -114,6 +114,87 @@ def test_dense_variants(T, H, I, E, k, B, impl, act, mode, bias, skip, clamp):
     _check(o, g, f"dense {impl} act={act} mode={mode}")
 
 
+def _run_checkpointed(c, impl, act=0, mode=1, clamps=None, on_I=False, tp2id=None, b2e=None):
+    import torch
+    from nkilib.core.moe.moe_cte import MoECTEImplementation, MoECTESpec, ShardOnIConfig, SkipMode, moe_cte
+    from nkilib.core.utils.common_types import ActFnType, ExpertAffinityScaleMode
+
+    dev = torch.device("cuda:0")
+    kw = dict(clamps or {})
+    if "gate_up_bias" in c:
+        kw["gate_and_up_proj_bias"] = bf16_tensor(c["gate_up_bias"], dev)
+        kw["down_proj_bias"] = bf16_tensor(c["down_bias"], dev)
+    spec = MoECTESpec(implementation=getattr(MoECTEImplementation, impl),
+                      shard_on_I=ShardOnIConfig(checkpoint_activation=True, expert_affinity_multiply_on_I=on_I))
+    outs = moe_cte[2](
+        bf16_tensor(c["hidden"], dev), bf16_tensor(c["aff"].reshape(-1, 1), dev), bf16_tensor(c["gate_up_w"], dev),
+        bf16_tensor(c["down_w"], dev), i32_tensor(c["tp2id"] if tp2id is None else tp2id, dev),
+        i32_tensor((c["b2e"] if b2e is None else b2e).reshape(-1, 1), dev), c["B"], spec,
+        activation_function=ActFnType(act), skip_dma=SkipMode(c["skip_token"], False),
+        expert_affinities_scaling_mode=ExpertAffinityScaleMode(mode), **kw)
+    torch.cuda.synchronize()
+    return outs
+
+
+@pytest.mark.parametrize(
+    "T,H,I,E,k,B,act,mode,bias,skip,clamp,on_I",
+    [
+        (300, 512, 384, 4, 2, 128, 0, 1, False, False, False, False),  # ragged last blocks: padding rows are checkpointed too
+        (300, 512, 256, 4, 2, 256, 3, 2, True, False, True, False),    # B = 2 tiles, PRE_SCALE, bias and clamps in the checkpoint
+        (256, 256, 136, 8, 2, 64, 0, 1, True, True, False, True),      # skip_token, I % 64 != 0, affinity on I: no down checkpoint
+    ],
+)
+def test_dense_checkpoint_activation(T, H, I, E, k, B, act, mode, bias, skip, clamp, on_I):
+    """checkpoint_activation (bwmm_shard_on_I.py:160-176): gate_up_activations_T [N, 2, I, B] and down_activations
+    [N, B, H] against the golden's (test_moe_cte_common.py:404-405,420-421), every row of every block."""
+    c = dense_case(T, H, I, E, k, B, seed=7, skip_token=skip, bias=bias, hidden_std=1.0)
+    clamps = dict(gate_clamp_upper_limit=0.8, gate_clamp_lower_limit=-0.7, up_clamp_upper_limit=0.9,
+                  up_clamp_lower_limit=-0.5) if clamp else None
+    outs = _run_checkpointed(c, "shard_on_i", act, mode, clamps, on_I)
+    assert len(outs) == (2 if on_I else 3)
+    cl = clamps or {}
+    g_out, g_gu, g_d = omoe.moe_blockwise_ref(
+        c["hidden"], c["aff"], c["gate_up_w"], c["down_w"], c["tp2id"], c["b2e"], B,
+        gate_up_proj_bias=c.get("gate_up_bias"), down_proj_bias=c.get("down_bias"), activation_function=act,
+        skip_token=skip, expert_affinities_scaling_mode=mode, checkpoint_activation=True,
+        gate_clamp_upper_limit=cl.get("gate_clamp_upper_limit"), gate_clamp_lower_limit=cl.get("gate_clamp_lower_limit"),
+        up_clamp_upper_limit=cl.get("up_clamp_upper_limit"), up_clamp_lower_limit=cl.get("up_clamp_lower_limit"))
+    o = from_bf16_tensor(outs[0])
+    rows = T
+    _check(o[:rows], g_out[:rows], "checkpointed output")
+    gu = from_bf16_tensor(outs[1])
+    assert gu.shape == (c["N"], 2, I, B)
+    _check(gu, g_gu, "gate_up_activations_T")
+    if not on_I:
+        d = from_bf16_tensor(outs[2])
+        assert d.shape == (c["N"], B, H)
+        _check(d, g_d, "down_activations")
+
+
+@pytest.mark.parametrize("mode,on_I", [(2, False), (1, True)])
+def test_dropping_variant(mode, on_I):
+    """shard_on_i_dropping (bwmm_shard_on_I.py:2014-2159): one block per expert (block b = expert b, block_to_expert
+    not read), tokens past an expert's capacity dropped by the caller; always returns the checkpoints."""
+    T, H, I, E, k, B = 384, 512, 256, 8, 2, 64
+    c = dense_case(T, H, I, E, k, B, seed=9, hidden_std=1.0)
+    tp = np.full((E, B), T, dtype=np.int32)
+    for e in range(E):
+        ids = np.flatnonzero(c["mask"][:, e])[:B]  # capacity B: the rest is dropped
+        tp[e, : ids.size] = ids
+    assert (c["mask"].sum(0) > B).any(), "the case must actually drop tokens"
+    b2e = np.arange(E, dtype=np.int32)
+    outs = _run_checkpointed(c, "shard_on_i_dropping", mode=mode, on_I=on_I, tp2id=tp.reshape(-1),
+                             b2e=np.zeros(E, np.int32))  # block_to_expert is ignored by this variant
+    assert len(outs) == (2 if on_I else 3)
+    g_out, g_gu, g_d = omoe.moe_blockwise_ref(c["hidden"], c["aff"], c["gate_up_w"], c["down_w"], tp.reshape(-1), b2e, B,
+                                              expert_affinities_scaling_mode=mode, checkpoint_activation=True)
+    assert tuple(outs[0].shape) == (T + 1, H)
+    _check(from_bf16_tensor(outs[0])[:T], g_out[:T], "dropping output")
+    _check(from_bf16_tensor(outs[1]), g_gu, "dropping gate_up_activations_T")
+    if not on_I:
+        _check(from_bf16_tensor(outs[2]), g_d, "dropping down_activations")
+
+
 def test_dense_conditions_stop():
     """Hybrid variant: blocks from the first conditions[b] == 0 on are skipped."""
     c = dense_case(256, 512, 256, 8, 2, 128, seed=4, hidden_std=1.0)
