@@ -115,7 +115,7 @@ int moe_router_topk(const void* x, const void* w, const void* w_bias, int bias_d
  * Writes token_position_to_id int32[N*B], block_to_expert int32[N], conditions int32[n_conditions]
  * (nullable; ones for the first N - n_padding_blocks entries... exactly: the trailing
  * n_padding_blocks + (n_conditions - N) entries are 0).  pad id = T, or -1 when skip_token.
- * workspace: >= moe_build_blocks_workspace_bytes(E) bytes.  Returns MOE_E_BAD_SHAPE through
+ * E <= 1024.  workspace: >= moe_build_blocks_workspace_bytes(E) bytes.  Returns MOE_E_BAD_SHAPE through
  * *status_out (device int32, nullable) == 1 when N is too small for the routing. */
 size_t moe_build_blocks_workspace_bytes(int64_t E);
 int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,

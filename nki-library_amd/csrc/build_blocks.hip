@@ -2,14 +2,16 @@
 // generate_token_position_to_id_and_experts,
 // test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:199-264).
 //
-// A stable counting sort of the routed (token, expert) pairs by expert:
-//   1. count_kernel    one workgroup per expert counts the tokens that selected it; the grid also
-//                      fills token_position_to_id with the pad id
-//   2. layout_kernel   one workgroup: blocks per expert, padding blocks to the last expert (or
-//                      split), exclusive scan -> first slot of every expert, block_to_expert,
-//                      conditions
-//   3. scatter_kernel  one workgroup per expert ranks its tokens in ascending token id with a
-//                      block-wide scan and writes their ids
+// A stable counting sort of the routed (token, expert) pairs by expert that reads the ids twice and nothing
+// else: the tokens are cut into at most 64 slabs, one workgroup each.
+//   1. count_kernel    per slab, 256 tokens at a time: every token sets its bit in the LDS bitmap of each expert
+//                      it selected; population counts give the slab's tokens per expert.  The grid also fills
+//                      token_position_to_id with the pad id.
+//   2. layout_kernel   one workgroup: per expert the counts of the slabs become offsets (exclusive scan over
+//                      the slabs), their sum the expert's count; blocks per expert, padding blocks to the last
+//                      expert (or split), exclusive scan -> first slot of every expert, block_to_expert, conditions
+//   3. scatter_kernel  per slab, the same bitmaps again: a token's rank among the tokens of its expert is the
+//                      number of set bits below its own, plus the slab's offset; writes the token ids
 // The work is latency bound (a few hundred KB of int32), so each step is a single small launch.
 #include "common.hpp"
 
@@ -17,47 +19,73 @@ namespace moe {
 
 constexpr int BB_THREADS = 256;
 
-// 1 if token t lists expert e among its k choices.  k == 8 (two 16-byte loads) is the common case.
-__device__ __forceinline__ int token_selects(const int32_t* ids, int64_t t, int64_t k, int e) {
-  if (k == 8) {
-    const int4 a = ((const int4*)(ids + t * 8))[0], b = ((const int4*)(ids + t * 8))[1];
-    return (a.x == e) | (a.y == e) | (a.z == e) | (a.w == e) | (b.x == e) | (b.y == e) | (b.z == e) | (b.w == e);
+constexpr int BB_SLABS_MAX = 64;
+constexpr int BB_E_MAX = 1024;  // bitmaps and running counts of all experts in LDS: 36 bytes per expert
+
+// The bitmaps of 256 tokens: bit (tid & 31) of word bm[(tid >> 5) * E + e] says that token t0 + tid selected
+// expert e.  Ids outside [0, E) are ignored; an id listed twice sets its bit once.
+__device__ __forceinline__ void bb_mark(const int32_t* __restrict__ ids, int64_t t, bool live, int64_t k, int64_t E,
+                                        uint32_t* bm, int my[8]) {
+  const uint32_t bit = 1u << (threadIdx.x & 31);
+  uint32_t* row = bm + (threadIdx.x >> 5) * E;
+  if (k == 8) {  // two 16-byte loads
+    int4 a = make_int4(-1, -1, -1, -1), b = a;
+    if (live) {
+      a = ((const int4*)(ids + t * 8))[0];
+      b = ((const int4*)(ids + t * 8))[1];
+    }
+    my[0] = a.x; my[1] = a.y; my[2] = a.z; my[3] = a.w;
+    my[4] = b.x; my[5] = b.y; my[6] = b.z; my[7] = b.w;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (my[j] >= 0 && my[j] < E) atomicOr(&row[my[j]], bit);
+  } else if (live) {
+    for (int64_t j = 0; j < k; ++j) {
+      const int e = ids[t * k + j];
+      if (e >= 0 && e < E) atomicOr(&row[e], bit);
+    }
   }
-  int hit = 0;
-  for (int64_t j = 0; j < k; ++j) hit |= (ids[t * k + j] == e);
-  return hit;
 }
 
-// One workgroup per expert counts its tokens (a ballot and a population count per 64 tokens); all
-// workgroups together also fill token_position_to_id with the pad id, which the scatter overwrites
-// where tokens sit.
+__device__ __forceinline__ int bb_bits(const uint32_t* bm, int64_t E, int64_t e) {
+  int n = 0;
+#pragma unroll
+  for (int w = 0; w < 8; ++w) n += __popc(bm[w * E + e]);
+  return n;
+}
+
+// Workgroup = slab of slab_tokens tokens (a multiple of 256).  slab_counts[slab][e] = tokens of the slab that
+// selected e.  All workgroups together also fill token_position_to_id with the pad id, which the scatter
+// overwrites where tokens sit.
 __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
-                                                             int32_t* __restrict__ counts,
+                                                             int64_t E, int64_t slab_tokens,
+                                                             int32_t* __restrict__ slab_counts,
                                                              int32_t* __restrict__ tp2id, int64_t NB, int pad_id) {
-  __shared__ int red[BB_THREADS / 64];
-  const int e = blockIdx.x;
-  int c = 0;
-  for (int64_t t0 = 0; t0 < T; t0 += BB_THREADS) {
-    const int64_t t = t0 + threadIdx.x;
-    const int hit = (t < T) ? token_selects(ids, t, k, e) : 0;
-    c += __popcll(__ballot(hit));
+  extern __shared__ uint32_t bb_lds[];
+  uint32_t* bm = bb_lds;            // [8][E]
+  int* run = (int*)(bb_lds + 8 * E);  // [E]
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) run[e] = 0;
+  const int64_t t_begin = (int64_t)blockIdx.x * slab_tokens;
+  for (int64_t sub = 0; sub < slab_tokens && t_begin + sub < T; sub += BB_THREADS) {
+    for (int64_t i = threadIdx.x; i < 8 * E; i += BB_THREADS) bm[i] = 0;
+    __syncthreads();
+    const int64_t t = t_begin + sub + threadIdx.x;
+    int my[8];
+    bb_mark(ids, t, t < T, k, E, bm, my);
+    __syncthreads();
+    for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) run[e] += bb_bits(bm, E, e);
+    __syncthreads();
   }
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int s = 0;
-    for (int i = 0; i < BB_THREADS / 64; ++i) s += red[i];
-    counts[e] = s;
-  }
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) slab_counts[(int64_t)blockIdx.x * E + e] = run[e];
   for (int64_t i = (int64_t)blockIdx.x * BB_THREADS + threadIdx.x; i < NB; i += (int64_t)gridDim.x * BB_THREADS)
     tp2id[i] = pad_id;
 }
 
-// ws layout: counts[E] | first_slot[E] | n_padding[1]
+// ws layout: first_slot[E] | slab_counts[BB_SLABS_MAX][E]
 // One workgroup: blocks per expert (padding blocks to the last expert, or split), exclusive scan ->
 // first slot of every expert, block_to_expert, conditions; sums and scans over the experts are
 // workgroup-wide (shuffles + one exchange), a tile of BB_THREADS experts at a time.
-__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ counts,
+__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(int32_t* __restrict__ slab_counts, int64_t n_slabs,
                                                               int32_t* __restrict__ first_slot,
                                                               int32_t* __restrict__ block_to_expert,
                                                               int32_t* __restrict__ conditions, int64_t n_conditions,
@@ -70,7 +98,18 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __
   // blocks per expert and their sum
   int mine = 0;
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
-    const int nb = (int)((counts[e] + B - 1) / B);
+    // the slabs' counts of this expert -> where each slab's tokens start inside the expert's region
+    // (all loads first: one round trip to memory instead of one per slab)
+    int v[BB_SLABS_MAX];
+#pragma unroll
+    for (int sl = 0; sl < BB_SLABS_MAX; ++sl) v[sl] = (sl < n_slabs) ? slab_counts[sl * E + e] : 0;
+    int64_t count = 0;
+#pragma unroll
+    for (int sl = 0; sl < BB_SLABS_MAX; ++sl) {
+      if (sl < n_slabs) slab_counts[sl * E + e] = (int32_t)count;
+      count += v[sl];
+    }
+    const int nb = (int)((count + B - 1) / B);
     s_nb[e] = nb;
     mine += nb;
   }
@@ -113,35 +152,43 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __
   }
 }
 
-// One workgroup per expert ranks its tokens in ascending token id (ballot + population count below
-// the lane, plus the counts of the waves before) and writes their ids.
+// Workgroup = slab.  A token's slot for expert e: first slot of e + tokens of e in the slabs before (the layout
+// kernel turned the counts into these offsets) + tokens of e earlier in this slab.
 __global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
+                                                               int64_t E, int64_t slab_tokens,
+                                                               const int32_t* __restrict__ slab_offsets,
                                                                const int32_t* __restrict__ first_slot,
                                                                int32_t* __restrict__ tp2id, int64_t NB) {
-  __shared__ int wsum[2][BB_THREADS / 64];
-  const int e = blockIdx.x;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  int base = first_slot[e];
-  int buf = 0;
-  for (int64_t t0 = 0; t0 < T; t0 += BB_THREADS, buf ^= 1) {
-    const int64_t t = t0 + threadIdx.x;
-    const int hit = (t < T) ? token_selects(ids, t, k, e) : 0;
-    const unsigned long long m = __ballot(hit);
-    const int below = __popcll(m & ((1ull << lane) - 1ull));
-    if (lane == 0) wsum[buf][w] = __popcll(m);
-    __syncthreads();  // wsum[buf] is rewritten two iterations later, after the next barrier
-    int before = 0, total = 0;
-#pragma unroll
-    for (int i = 0; i < BB_THREADS / 64; ++i) {
-      const int v = wsum[buf][i];
-      before += (i < w) ? v : 0;
-      total += v;
+  extern __shared__ uint32_t bb_lds[];
+  uint32_t* bm = bb_lds;
+  int* run = (int*)(bb_lds + 8 * E);
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS)
+    run[e] = first_slot[e] + slab_offsets[(int64_t)blockIdx.x * E + e];
+  const int64_t t_begin = (int64_t)blockIdx.x * slab_tokens;
+  const int wd = threadIdx.x >> 5;
+  const uint32_t below = (1u << (threadIdx.x & 31)) - 1u;
+  for (int64_t sub = 0; sub < slab_tokens && t_begin + sub < T; sub += BB_THREADS) {
+    for (int64_t i = threadIdx.x; i < 8 * E; i += BB_THREADS) bm[i] = 0;
+    __syncthreads();
+    const int64_t t = t_begin + sub + threadIdx.x;
+    const bool live = t < T;
+    int my[8];
+    bb_mark(ids, t, live, k, E, bm, my);
+    __syncthreads();
+    if (live) {
+      const int64_t kk = (k == 8) ? 8 : k;
+      for (int64_t j = 0; j < kk; ++j) {
+        const int e = (k == 8) ? my[j] : ids[t * k + j];
+        if (e < 0 || e >= E) continue;
+        int r = __popc(bm[wd * E + e] & below);
+        for (int w = 0; w < wd; ++w) r += __popc(bm[w * E + e]);
+        const int64_t pos = (int64_t)run[e] + r;
+        if (pos < NB) tp2id[pos] = (int32_t)t;
+      }
     }
-    if (hit) {
-      const int64_t pos = (int64_t)base + before + below;
-      if (pos < NB) tp2id[pos] = (int32_t)t;
-    }
-    base += total;
+    __syncthreads();
+    for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) run[e] += bb_bits(bm, E, e);
+    __syncthreads();  // the bitmaps are cleared next
   }
 }
 
@@ -149,7 +196,9 @@ __global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* _
 
 using namespace moe;
 
-extern "C" size_t moe_build_blocks_workspace_bytes(int64_t E) { return (size_t)(2 * E + 4) * sizeof(int32_t); }
+extern "C" size_t moe_build_blocks_workspace_bytes(int64_t E) {
+  return (size_t)((1 + BB_SLABS_MAX) * E + 4) * sizeof(int32_t);
+}
 
 extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
                                 int skip_token, int use_split_padding, int32_t* token_position_to_id,
@@ -159,19 +208,25 @@ extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, i
   if (T < 0 || k <= 0 || E <= 0 || B <= 0 || N <= 0) return MOE_E_BAD_ARG;
   if (conditions && n_conditions < N) return MOE_E_BAD_SHAPE;
   if (workspace_bytes < moe_build_blocks_workspace_bytes(E)) return MOE_E_WORKSPACE;
-  if (N * B >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
-  int32_t* counts = (int32_t*)workspace;
-  int32_t* first_slot = counts + E;
+  if (N * B >= (int64_t)1 << 31 || E > BB_E_MAX) return MOE_E_BAD_SHAPE;
+  // at most BB_SLABS_MAX slabs of a multiple of 256 tokens
+  int64_t slab_tokens = (T + BB_SLABS_MAX - 1) / BB_SLABS_MAX;
+  slab_tokens = (slab_tokens + BB_THREADS - 1) / BB_THREADS * BB_THREADS;
+  if (slab_tokens == 0) slab_tokens = BB_THREADS;
+  int64_t n_slabs = (T + slab_tokens - 1) / slab_tokens;
+  if (n_slabs == 0) n_slabs = 1;  // T == 0: one slab with no tokens still fills the pad ids
+  int32_t* first_slot = (int32_t*)workspace;
+  int32_t* slab_counts = first_slot + E;
+  const size_t lds = (size_t)9 * E * sizeof(int32_t);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(bb_count_kernel, dim3((unsigned)E), dim3(BB_THREADS), 0, s, topk_ids, T, k, counts,
-                     token_position_to_id, N * B, skip_token ? -1 : (int)T);
+  hipLaunchKernelGGL(bb_count_kernel, dim3((unsigned)n_slabs), dim3(BB_THREADS), lds, s, topk_ids, T, k, E, slab_tokens,
+                     slab_counts, token_position_to_id, N * B, skip_token ? -1 : (int)T);
   MOE_CHECK_LAUNCH();
-  if (2 * E * sizeof(int) > 48 * 1024) return MOE_E_BAD_SHAPE;
-  hipLaunchKernelGGL(bb_layout_kernel, dim3(1), dim3(BB_THREADS), 2 * E * sizeof(int), s, counts, first_slot,
-                     block_to_expert, conditions, n_conditions, E, B, N, use_split_padding, status_out);
+  hipLaunchKernelGGL(bb_layout_kernel, dim3(1), dim3(BB_THREADS), 2 * E * sizeof(int), s, slab_counts, n_slabs,
+                     first_slot, block_to_expert, conditions, n_conditions, E, B, N, use_split_padding, status_out);
   MOE_CHECK_LAUNCH();
-  hipLaunchKernelGGL(bb_scatter_kernel, dim3((unsigned)E), dim3(BB_THREADS), 0, s, topk_ids, T, k, first_slot,
-                     token_position_to_id, N * B);
+  hipLaunchKernelGGL(bb_scatter_kernel, dim3((unsigned)n_slabs), dim3(BB_THREADS), lds, s, topk_ids, T, k, E,
+                     slab_tokens, slab_counts, first_slot, token_position_to_id, N * B);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
 }

@@ -19,7 +19,8 @@ __global__ __launch_bounds__(256) void prep_blocks_kernel(const int32_t* __restr
                                                           const int32_t* __restrict__ conditions, int64_t n_conditions,
                                                           int64_t N, int64_t B, int64_t E, int64_t n_real,
                                                           int32_t* __restrict__ n_active,
-                                                          int32_t* __restrict__ valid_rows) {
+                                                          int32_t* __restrict__ valid_rows,
+                                                          int32_t* __restrict__ cnt) {
   __shared__ int s_first_zero;
   __shared__ int s_red[4];
   if (threadIdx.x == 0) s_first_zero = (int)N;
@@ -38,7 +39,10 @@ __global__ __launch_bounds__(256) void prep_blocks_kernel(const int32_t* __restr
     if (b < na && e >= 0 && e < E) {
       for (int64_t r = threadIdx.x; r < B; r += blockDim.x) {
         const int id = tp2id[b * B + r];
-        if (id >= 0 && id < n_real) v = (int)r + 1;
+        if (id >= 0 && id < n_real) {
+          v = (int)r + 1;
+          atomicAdd(&cnt[id], 1);  // slots per token, for the token -> slot lists of the combine
+        }
       }
     }
 #pragma unroll
@@ -50,22 +54,17 @@ __global__ __launch_bounds__(256) void prep_blocks_kernel(const int32_t* __restr
   }
 }
 
-// Single workgroup of 1024 threads, run after prep_blocks_kernel.  A "run" is a maximal sequence of
+// One workgroup of 1024 threads.  A "run" is a maximal sequence of
 // consecutive active blocks of one expert; the thread that owns a run's first block measures the
 // run (slots up to its last real token) and, after a block-wide scan of the chunk counts, writes
 // the run's chunks.  Chunk order follows block order.
-__global__ __launch_bounds__(1024) void build_chunks_kernel(const int32_t* __restrict__ b2e,
-                                                            const int32_t* __restrict__ n_active,
-                                                            const int32_t* __restrict__ valid_rows, int64_t N,
-                                                            int64_t B, int64_t E, int32_t* __restrict__ n_chunks,
-                                                            int32_t* __restrict__ chunk_slot,
-                                                            int32_t* __restrict__ chunk_rows,
-                                                            int32_t* __restrict__ chunk_expert, int64_t max_chunks) {
-  __shared__ int s_scan[1024];
-  __shared__ int s_carry;
+__device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, const int32_t* __restrict__ n_active,
+                                             const int32_t* __restrict__ valid_rows, int64_t N, int64_t B, int64_t E,
+                                             int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
+                                             int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
+                                             int64_t max_chunks, int* s_ws) {
   const int64_t na = *n_active;
-  if (threadIdx.x == 0) s_carry = 0;
-  __syncthreads();
+  int carry = 0;
   for (int64_t b0 = 0; b0 < na; b0 += 1024) {
     const int64_t b = b0 + threadIdx.x;
     int nch = 0;
@@ -83,15 +82,8 @@ __global__ __launch_bounds__(1024) void build_chunks_kernel(const int32_t* __res
         if (len > 0) nch = (len <= CHUNK_ROWS_MAX) ? 1 : (int)((len - CHUNK_ROWS_MAX + CHUNK_ROWS - 1) / CHUNK_ROWS) + 1;
       }
     }
-    s_scan[threadIdx.x] = nch;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {
-      const int v = (threadIdx.x >= (unsigned)o) ? s_scan[threadIdx.x - o] : 0;
-      __syncthreads();
-      s_scan[threadIdx.x] += v;
-      __syncthreads();
-    }
-    const int base = s_carry + s_scan[threadIdx.x] - nch;
+    int total;
+    const int base = carry + block_excl_scan(nch, s_ws, &total);
     for (int k = 0; k < nch; ++k) {
       const int64_t s0 = b * B + (int64_t)k * CHUNK_ROWS;
       if (base + k < max_chunks) {
@@ -100,11 +92,9 @@ __global__ __launch_bounds__(1024) void build_chunks_kernel(const int32_t* __res
         chunk_expert[base + k] = e;
       }
     }
-    __syncthreads();
-    if (threadIdx.x == 1023) s_carry += s_scan[1023];
-    __syncthreads();
+    carry += total;
   }
-  if (threadIdx.x == 0) *n_chunks = (int32_t)((s_carry < max_chunks) ? s_carry : max_chunks);
+  if (threadIdx.x == 0) *n_chunks = (int32_t)((carry < max_chunks) ? carry : max_chunks);
 }
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* __restrict__ p, int64_t n) {
@@ -112,32 +102,43 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* __restrict__ p,
   if (i < n) p[i] = 0;
 }
 
-__global__ __launch_bounds__(256) void inv_count_kernel(const int32_t* __restrict__ tp2id,
-                                                        const int32_t* __restrict__ valid_rows, int64_t N, int64_t B,
-                                                        int64_t n_real, int32_t* __restrict__ cnt) {
-  const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (s >= N * B) return;
-  const int64_t b = s / B, r = s % B;
-  if (r >= valid_rows[b]) return;
-  const int id = tp2id[s];
-  if (id >= 0 && id < n_real) atomicAdd(&cnt[id], 1);
-}
-
-// Exclusive scan of cnt[0..n) into off[0..n], single workgroup of 1024 threads.
-__global__ __launch_bounds__(1024) void inv_scan_kernel(const int32_t* __restrict__ cnt, int32_t* __restrict__ off,
-                                                        int64_t n) {
-  __shared__ int s_ws[16];
-  // thread t owns elements t, t + 1024, ... of each 1024-element tile: coalesced, one scan per tile
+// Exclusive scan of cnt[0..n) into off[0..n] by one workgroup of 1024 threads: a thread owns 8 consecutive
+// elements of each 8192-element tile.
+__device__ __forceinline__ void inv_scan(const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n,
+                                         int* s_ws) {
   int carry = 0;
-  for (int64_t base = 0; base < n; base += 1024) {
-    const int64_t i = base + threadIdx.x;
-    const int v = (i < n) ? cnt[i] : 0;
+  for (int64_t base = 0; base < n; base += 8192) {
+    const int64_t i0 = base + 8 * (int64_t)threadIdx.x;
+    int v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (i0 + j < n) ? cnt[i0 + j] : 0;
+    int mine = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) mine += v[j];
     int total;
-    const int ex = block_excl_scan(v, s_ws, &total);
-    if (i < n) off[i] = carry + ex;
+    int run = carry + block_excl_scan(mine, s_ws, &total);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (i0 + j < n) off[i0 + j] = run;
+      run += v[j];
+    }
     carry += total;
   }
   if (threadIdx.x == 0) off[n] = carry;
+}
+
+// Two workgroups of 1024 threads, run after prep_blocks_kernel: workgroup 0 builds the expert chunks,
+// workgroup 1 turns the slots-per-token counts into list offsets.  They share no data.
+__global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
+    const int32_t* __restrict__ b2e, const int32_t* __restrict__ n_active, const int32_t* __restrict__ valid_rows,
+    int64_t N, int64_t B, int64_t E, int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
+    int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int64_t max_chunks,
+    const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n_real) {
+  __shared__ int s_ws[16];
+  if (blockIdx.x == 0)
+    build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, max_chunks, s_ws);
+  else
+    inv_scan(cnt, off, n_real, s_ws);
 }
 
 __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict__ tp2id,
@@ -253,18 +254,14 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
   MOE_CHECK_LAUNCH();
   const unsigned g = (unsigned)(a->N < 1024 ? a->N : 1024);
   hipLaunchKernelGGL(prep_blocks_kernel, dim3(g), dim3(256), 0, s, a->token_position_to_id, a->block_to_expert,
-                     a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows);
+                     a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows, k.cnt);
   MOE_CHECK_LAUNCH();
-  hipLaunchKernelGGL(build_chunks_kernel, dim3(1), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows, a->N,
-                     a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.max_chunks);
+  hipLaunchKernelGGL(chunks_and_offsets_kernel, dim3(2), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows,
+                     a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.max_chunks, k.cnt,
+                     k.off, n_real);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
   const unsigned gs = (unsigned)((slots + 255) / 256);
-  hipLaunchKernelGGL(inv_count_kernel, dim3(gs), dim3(256), 0, s, a->token_position_to_id, k.valid_rows, a->N, a->B,
-                     n_real, k.cnt);
-  MOE_CHECK_LAUNCH();
-  hipLaunchKernelGGL(inv_scan_kernel, dim3(1), dim3(1024), 0, s, k.cnt, k.off, n_real);
-  MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(inv_fill_kernel, dim3(gs), dim3(256), 0, s, a->token_position_to_id, k.valid_rows, a->N, a->B,
                      n_real, k.off, k.cursor, k.list);
   MOE_CHECK_LAUNCH();
