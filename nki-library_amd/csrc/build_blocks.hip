@@ -7,8 +7,7 @@
 //   1. count_kernel    per slab, 256 tokens at a time: every token sets its bit in the LDS bitmap of each expert
 //                      it selected; population counts give the slab's tokens per expert.  The grid also fills
 //                      token_position_to_id with the pad id.
-//   2. layout_kernel   one workgroup: per expert the counts of the slabs become offsets (exclusive scan over
-//                      the slabs), their sum the expert's count; blocks per expert, padding blocks to the last
+//   2. layout_kernel   one workgroup: per expert the sum of the slabs' counts; blocks per expert, padding blocks to the last
 //                      expert (or split), exclusive scan -> first slot of every expert, block_to_expert, conditions
 //   3. scatter_kernel  per slab, the same bitmaps again: a token's rank among the tokens of its expert is the
 //                      number of set bits below its own, plus the slab's offset; writes the token ids
@@ -85,7 +84,7 @@ __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __r
 // One workgroup: blocks per expert (padding blocks to the last expert, or split), exclusive scan ->
 // first slot of every expert, block_to_expert, conditions; sums and scans over the experts are
 // workgroup-wide (shuffles + one exchange), a tile of BB_THREADS experts at a time.
-__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(int32_t* __restrict__ slab_counts, int64_t n_slabs,
+__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
                                                               int32_t* __restrict__ first_slot,
                                                               int32_t* __restrict__ block_to_expert,
                                                               int32_t* __restrict__ conditions, int64_t n_conditions,
@@ -98,17 +97,9 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(int32_t* __restri
   // blocks per expert and their sum
   int mine = 0;
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
-    // the slabs' counts of this expert -> where each slab's tokens start inside the expert's region
-    // (all loads first: one round trip to memory instead of one per slab)
-    int v[BB_SLABS_MAX];
-#pragma unroll
-    for (int sl = 0; sl < BB_SLABS_MAX; ++sl) v[sl] = (sl < n_slabs) ? slab_counts[sl * E + e] : 0;
     int64_t count = 0;
-#pragma unroll
-    for (int sl = 0; sl < BB_SLABS_MAX; ++sl) {
-      if (sl < n_slabs) slab_counts[sl * E + e] = (int32_t)count;
-      count += v[sl];
-    }
+#pragma unroll 8
+    for (int64_t sl = 0; sl < n_slabs; ++sl) count += slab_counts[sl * E + e];
     const int nb = (int)((count + B - 1) / B);
     s_nb[e] = nb;
     mine += nb;
@@ -152,18 +143,22 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(int32_t* __restri
   }
 }
 
-// Workgroup = slab.  A token's slot for expert e: first slot of e + tokens of e in the slabs before (the layout
-// kernel turned the counts into these offsets) + tokens of e earlier in this slab.
+// Workgroup = slab.  A token's slot for expert e: first slot of e + tokens of e in the slabs before (summed here
+// from the slab counts) + tokens of e earlier in this slab.
 __global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
                                                                int64_t E, int64_t slab_tokens,
-                                                               const int32_t* __restrict__ slab_offsets,
+                                                               const int32_t* __restrict__ slab_counts,
                                                                const int32_t* __restrict__ first_slot,
                                                                int32_t* __restrict__ tp2id, int64_t NB) {
   extern __shared__ uint32_t bb_lds[];
   uint32_t* bm = bb_lds;
   int* run = (int*)(bb_lds + 8 * E);
-  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS)
-    run[e] = first_slot[e] + slab_offsets[(int64_t)blockIdx.x * E + e];
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
+    int before = first_slot[e];
+#pragma unroll 8
+    for (int64_t sl = 0; sl < blockIdx.x; ++sl) before += slab_counts[sl * E + e];
+    run[e] = before;
+  }
   const int64_t t_begin = (int64_t)blockIdx.x * slab_tokens;
   const int wd = threadIdx.x >> 5;
   const uint32_t below = (1u << (threadIdx.x & 31)) - 1u;
