@@ -435,3 +435,124 @@ def moe_mx_token_ref(x_row, e_list, aff_row, gate_up_proj_weight, gate_up_proj_s
         wd = mx_dequant_down(down_proj_weight[e], down_proj_scale[e]).astype(np.float64)
         total += float(to_bf16(np.asarray([aff_row[e]], dtype=np.float32))[0]) * (yk.astype(np.float64) @ wd)
     return total
+
+
+# ---------------------------------------------------------------------------------------------------
+# Token-generation MoE (moe_tkg): restates moe_tkg_torch_ref
+# (src/nkilib_src/nkilib/core/moe/moe_tkg/moe_tkg_torch.py:35-226 dense, :320-442 MX).
+# ---------------------------------------------------------------------------------------------------
+def _tkg_expert_mlp(x, w_gu, w_d, b_gu, b_d, activation_function, gate_hi, up_hi, up_lo, s_gu, s_d):
+    """One expert's MLP on rows x, result rounded to bf16 (moe_tkg_torch.py:242-317; like the golden, the
+    gate projection is only clamped from above)."""
+    gw, uw = w_gu[:, 0, :].astype(np.float32), w_gu[:, 1, :].astype(np.float32)
+    if s_gu is not None:
+        gw = gw * np.asarray(s_gu, dtype=np.float32)[0:1, :]
+        uw = uw * np.asarray(s_gu, dtype=np.float32)[1:2, :]
+    g = x @ gw
+    if b_gu is not None:
+        g = g + np.asarray(b_gu, dtype=np.float32)[0]
+    if gate_hi is not None:
+        g = np.minimum(g, gate_hi)
+    g = act_fn(g, activation_function)
+    u = x @ uw
+    if b_gu is not None:
+        u = u + np.asarray(b_gu, dtype=np.float32)[1]
+    u = _clip(u.copy(), up_lo, up_hi)
+    dw = np.asarray(w_d, dtype=np.float32)
+    if s_d is not None:
+        dw = dw * np.asarray(s_d, dtype=np.float32).reshape(1, -1)
+    y = (g * u) @ dw
+    if b_d is not None:
+        y = y + np.asarray(b_d, dtype=np.float32)
+    return to_bf16(y.astype(np.float32))
+
+
+def moe_tkg_ref(hidden_input, expert_gate_up_weights, expert_down_weights, expert_affinities, expert_index,
+                is_all_expert, expert_gate_up_bias=None, expert_down_bias=None, expert_gate_up_weights_scale=None,
+                expert_down_weights_scale=None, expert_affinities_scaling_mode=NO_SCALE,
+                activation_function=ACT_SILU, gate_clamp_upper_limit=None, up_clamp_upper_limit=None,
+                up_clamp_lower_limit=None):
+    """Dense (bf16 / fp8-row-weight) token-generation MoE.  hidden_input [T, H]; weights [E, H, 2, I], [E, I, H]
+    (fp32 values); row scales [E, 2, I], [E, H]; expert_affinities [T, E] (already sliced / masked for the
+    all-expert mode); expert_index [T, K].  Every expert output is rounded to bf16, multiplied by the bf16 affinity
+    (POST_SCALE) and added to the bf16 output: all experts in ascending order (all-expert, experts whose affinity
+    column sums to zero are skipped, moe_tkg_torch.py:158-161), or the token's experts in the order expert_index
+    lists them (:187-214).  Returns bf16-valued fp32 [T, H]."""
+    x = np.asarray(hidden_input, dtype=np.float32)
+    T, H = x.shape
+    E = expert_gate_up_weights.shape[0]
+    aff = to_bf16(np.asarray(expert_affinities, dtype=np.float32))
+    out = np.zeros((T, H), dtype=np.float32)
+
+    def mlp(rows, e):
+        return _tkg_expert_mlp(
+            rows, np.asarray(expert_gate_up_weights[e]), expert_down_weights[e],
+            None if expert_gate_up_bias is None else expert_gate_up_bias[e],
+            None if expert_down_bias is None else expert_down_bias[e], activation_function, gate_clamp_upper_limit,
+            up_clamp_upper_limit, up_clamp_lower_limit,
+            None if expert_gate_up_weights_scale is None else expert_gate_up_weights_scale[e],
+            None if expert_down_weights_scale is None else expert_down_weights_scale[e])
+
+    if is_all_expert:
+        for e in range(E):
+            if aff[:, e].sum() == 0:
+                continue
+            y = mlp(x, e)
+            if expert_affinities_scaling_mode == POST_SCALE:
+                y = to_bf16(aff[:, e:e + 1] * y)
+            out = to_bf16(out + y)
+    else:
+        idx = np.asarray(expert_index)
+        for t in range(T):
+            for k in range(idx.shape[1]):
+                e = int(idx[t, k])
+                y = mlp(x[t:t + 1], e)[0]
+                if expert_affinities_scaling_mode == POST_SCALE:
+                    y = to_bf16(aff[t, e] * y)
+                out[t] = to_bf16(out[t] + y)
+    return out
+
+
+def moe_tkg_mx_ref(hidden_input, gate_up_proj_weight, down_proj_weight, gate_up_proj_scale, down_proj_scale,
+                   expert_affinities, expert_index, is_all_expert, gate_up_proj_bias=None, down_proj_bias=None,
+                   expert_affinities_scaling_mode=NO_SCALE, activation_function=ACT_SILU, weight_format="e4m3"):
+    """MX token-generation MoE (moe_tkg_torch.py:320-442): the hidden rows are quantised to MXFP8 with the same
+    8x4 blocks as the context-encoding path (:375-379), gate / up / down use the projection goldens of that path
+    (gate_up_proj_mx / down_proj_mx above restate the same functions, mlp_proj_mxfp4_torch.py:52-190), the product
+    act(gate) * up goes to the down projection unrounded, and the expert outputs are summed in fp32, times the
+    affinity with POST_SCALE; the result is rounded to bf16 once (:425-442).  Layouts as moe_blockwise_mx_ref."""
+    x = np.asarray(hidden_input, dtype=np.float32)
+    T, H = x.shape
+    E = gate_up_proj_weight.shape[0]
+    I = gate_up_proj_weight.shape[4]
+    aff = np.asarray(expert_affinities, dtype=np.float32)
+    res = np.zeros((T, H), dtype=np.float32)
+
+    def one(rows, e):
+        n = rows.shape[0]
+        gb = ub = None
+        if gate_up_proj_bias is not None:
+            gb = np.asarray(gate_up_proj_bias, dtype=np.float32)[e][:, 0]
+            ub = np.asarray(gate_up_proj_bias, dtype=np.float32)[e][:, 1]
+        g = gate_up_proj_mx(rows, gate_up_proj_weight[e][:, 0], gate_up_proj_scale[e][:, 0], gb, H, I, n, weight_format)
+        u = gate_up_proj_mx(rows, gate_up_proj_weight[e][:, 1], gate_up_proj_scale[e][:, 1], ub, H, I, n, weight_format)
+        y = (act_fn(g, activation_function) * u).astype(np.float32)
+        db = None if down_proj_bias is None else np.asarray(down_proj_bias, dtype=np.float32)[e]
+        return down_proj_mx(y, down_proj_weight[e], down_proj_scale[e], db, H, I, n, weight_format).reshape(n, H)
+
+    if is_all_expert:
+        for e in range(E):
+            y = one(x, e)
+            if expert_affinities_scaling_mode == POST_SCALE:
+                y = y * aff[:, e:e + 1]
+            res += y
+    else:
+        idx = np.asarray(expert_index)
+        for t in range(T):
+            for k in range(idx.shape[1]):
+                e = int(idx[t, k])
+                y = one(x[t:t + 1], e)[0]
+                if expert_affinities_scaling_mode == POST_SCALE:
+                    y = y * aff[t, e]
+                res[t] += y
+    return to_bf16(res)
