@@ -119,6 +119,76 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
   else if (KIND == MOE_KIND_BF16) nks = (int)((a.K + 63) / 64);
   else nks = (int)((a.K + 127) / 128);
 
+  if constexpr (KIND == MOE_KIND_FP8_ROW) {
+    // Both operands are plain 16-byte copies here (the weights were transposed beforehand), so the loop is
+    // software pipelined: the global loads of k-step ks+1 are in flight while the MFMAs of k-step ks run.
+    constexpr int PB = NCOLS * 8 / GT;
+    uint4 ra[4], rb[PB];
+    auto fetch = [&](int ks) {
+      const int64_t a_off = (int64_t)ks * 128;
+      const int a_valid = (int)((a.K - a_off < 128) ? (a.K - a_off) : 128);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = (tid >> 3) + 32 * j, ch = tid & 7;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        const uint8_t* src = nullptr;
+        if (STAGE == 1) {
+          const int tok = s_tok[row];
+          if (tok >= 0) src = a.A + (int64_t)tok * a.a_stride;
+        } else {
+          if (r0 + row < vr) src = a.A + (slot0 + row) * a.a_stride;
+        }
+        if (src != nullptr && ch * 16 + 16 <= a_valid) {
+          src += a_off + ch * 16;
+          if (STAGE == 1) {  // rows of H + 4 bytes are only 4-byte aligned
+            const uint32_t* s4 = (const uint32_t*)src;
+            val = make_uint4(s4[0], s4[1], s4[2], s4[3]);
+          } else {
+            val = *(const uint4*)src;
+          }
+        }
+        ra[j] = val;
+      }
+#pragma unroll
+      for (int j = 0; j < PB; ++j) {
+        const int idx = tid + GT * j;
+        const int col = idx >> 3, ch = idx & 7;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (STAGE == 1) {
+          const int gu = col >> 7;
+          const int64_t i = c0 + (col & 127);
+          if (i < a.I) val = *(const uint4*)(a.W + (((int64_t)e * 2 + gu) * a.I + i) * a.Kp + a_off + ch * 16);
+        } else {
+          const int64_t h = c0 + col;
+          if (h < a.H) val = *(const uint4*)(a.W + ((int64_t)e * a.H + h) * a.Kp + a_off + ch * 16);
+        }
+        rb[j] = val;
+      }
+    };
+    fetch(0);
+    for (int ks = 0; ks < nks; ++ks) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *(uint4*)(sA + ((tid >> 3) + 32 * j) * LROW + (tid & 7) * 16) = ra[j];
+#pragma unroll
+      for (int j = 0; j < PB; ++j) {
+        const int idx = tid + GT * j;
+        *(uint4*)(sB + (idx >> 3) * LROW + (idx & 7) * 16) = rb[j];
+      }
+      __syncthreads();
+      if (ks + 1 < nks) fetch(ks + 1);
+      v8i af[2];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) af[mt] = lds_read_frag(sA + (m0 + 16 * mt + c) * LROW, g);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const v8i bf = lds_read_frag(sB + (nt * 16 + c) * LROW, g);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, 127, 0, 127);
+      }
+      __syncthreads();
+    }
+  } else
   for (int ks = 0; ks < nks; ++ks) {
     // position of this k-step
     int kt = 0, pb = 0, Ptk = 128;      // MX: K tile (H or I tile), partition group, valid partitions
@@ -247,26 +317,22 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
           *(uint16_t*)(sB + col * LROW + kr * 2) = v;
         }
       }
-    } else {  // FP8_ROW: 128 k-rows x NCOLS byte columns, byte transpose
-      constexpr int CG = NCOLS / 4;
-      constexpr int RSTEP = GT / CG;
-      const int cg = tid % CG, kr0 = tid / CG;
-#pragma unroll 4
-      for (int j = 0; j < 128 / RSTEP; ++j) {
-        const int kr = kr0 + RSTEP * j;
-        const int64_t k = (int64_t)ks * 128 + kr;
-        uint32_t v = 0;
-        const int col = 4 * cg;
+    } else {  // FP8_ROW: the weights were transposed to K-contiguous rows of Kp bytes beforehand; staged like A
+      constexpr int PER = NCOLS * 8 / GT;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const int idx = tid + GT * j;
+        const int col = idx >> 3, ch = idx & 7;
+        uint4 val = make_uint4(0, 0, 0, 0);
         if (STAGE == 1) {
           const int gu = col >> 7;
           const int64_t i = c0 + (col & 127);
-          if (k < a.H && i < a.I) v = *(const uint32_t*)(a.W + (((int64_t)e * a.H + k) * 2 + gu) * a.I + i);
+          if (i < a.I) val = *(const uint4*)(a.W + (((int64_t)e * 2 + gu) * a.I + i) * a.Kp + (int64_t)ks * 128 + ch * 16);
         } else {
           const int64_t h = c0 + col;
-          if (k < a.I && h < a.H) v = *(const uint32_t*)(a.W + ((int64_t)e * a.I_pad + k) * a.H + h);
+          if (h < a.H) val = *(const uint4*)(a.W + ((int64_t)e * a.H + h) * a.Kp + (int64_t)ks * 128 + ch * 16);
         }
-#pragma unroll
-        for (int cc = 0; cc < 4; ++cc) sB[(col + cc) * LROW + kr] = (uint8_t)((v >> (8 * cc)) & 0xff);
+        *(uint4*)(sB + col * LROW + ch * 16) = val;
       }
     }
     __syncthreads();
@@ -465,6 +531,57 @@ __global__ __launch_bounds__(256) void row_requant_kernel(const float* __restric
     for (int k = 0; k < 4; ++k) v[k] = (i + k < I) ? y[i + k] / sc : 0.f;
     *(uint32_t*)(q + i) = pack4_e4m3(v[0], v[1], v[2], v[3]);
   }
+}
+
+// Byte-matrix transpose for the fp8 weights: batches of [R, C] (row stride src_row_stride) -> [C, Kp] with
+// Kp >= R a multiple of 64, the tail of every output row zero.  The GEMM wants K-contiguous weight rows (both
+// MFMA operands are read along K), the reference stores them N-contiguous.  64 x 64 tiles through LDS.
+__global__ __launch_bounds__(256) void transpose_fp8_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                            int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
+                                                            int nb1, int64_t src_bs0, int64_t src_bs1, int64_t dst_bs) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[64][80];
+  const int b = blockIdx.z;
+  const uint8_t* S = src + (int64_t)(b / nb1) * src_bs0 + (int64_t)(b % nb1) * src_bs1;
+  uint8_t* D = dst + (int64_t)b * dst_bs;
+  const int64_t n0 = (int64_t)blockIdx.x * 64, k0 = (int64_t)blockIdx.y * 64;
+  {
+    const int r = threadIdx.x >> 2, c16 = (threadIdx.x & 3) * 16;
+    const int64_t k = k0 + r, n = n0 + c16;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (k < R) {
+      const uint8_t* p = S + k * src_row_stride + n;
+      if (n + 16 <= C && (((uintptr_t)p) & 15) == 0) {
+        v = *(const uint4*)p;
+      } else {
+        uint8_t t[16];
+        for (int j = 0; j < 16; ++j) t[j] = (n + j < C) ? p[j] : (uint8_t)0;
+        __builtin_memcpy(&v, t, 16);
+      }
+    }
+    *(uint4*)(&tile[r][c16]) = v;
+  }
+  __syncthreads();
+  const int nn = threadIdx.x >> 2, kc = (threadIdx.x & 3) * 16;
+  if (n0 + nn < C) {
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      w[q] = (uint32_t)tile[kc + 4 * q][nn] | ((uint32_t)tile[kc + 4 * q + 1][nn] << 8) |
+             ((uint32_t)tile[kc + 4 * q + 2][nn] << 16) | ((uint32_t)tile[kc + 4 * q + 3][nn] << 24);
+    }
+    *(uint4*)(D + (n0 + nn) * Kp + k0 + kc) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
+                         int64_t nb0, int nb1, int64_t src_bs0, int64_t src_bs1, hipStream_t s) {
+  if ((Kp & 63) != 0 || Kp < R || (((uintptr_t)dst) & 15) != 0) return MOE_E_BAD_ARG;
+  const int64_t gx = (C + 63) / 64, gy = Kp / 64, gz = nb0 * nb1;
+  if (gy > 65535 || gz > 65535) return MOE_E_BAD_SHAPE;
+  hipLaunchKernelGGL(transpose_fp8_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s, src, dst, R,
+                     C, src_row_stride, Kp, nb1, src_bs0, src_bs1, C * Kp);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
 }
 
 template <int KIND, int STAGE>

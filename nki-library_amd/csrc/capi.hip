@@ -37,7 +37,8 @@ namespace {
 inline size_t al256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Plan {
-  size_t book, xq, xs, y, yq, ys, d, total;
+  size_t book, xq, xs, y, yq, ys, d, wt1, wt2, total;
+  int64_t Hk;      // FP8_ROW: H padded to the K step, row length of the transposed gate/up weights
   int64_t Iw;      // padded intermediate width (elements) of the stage-2 A operand
   int64_t pI, nI;  // MXFP8
 };
@@ -121,6 +122,10 @@ Plan make_plan(const moe_bwmm_args* a) {
     p.y = off; off += al256(slots * (size_t)a->I * 4);
     p.yq = off; off += al256(slots * (size_t)p.Iw);
     p.ys = off; off += al256(slots * 4);
+    // K-contiguous copies of the fp8 weights: [E, 2, I, Hk] and [E, H, Iw]
+    p.Hk = (a->H + 127) / 128 * 128;
+    p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk);
+    p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw);
   }
   p.d = off; off += al256(slots * (size_t)a->H * 2);
   p.total = off;
@@ -215,6 +220,20 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     g1.out = ws + p.y; g1.out_stride = a->I * 4;
     g2.A = ws + p.yq; g2.a_stride = p.Iw; g2.K = p.Iw; g2.A_scale = ws + p.ys;
     gx1 = (unsigned)((a->I + 127) / 128);
+    // the reference stores the weights N-contiguous ([E, H, 2, I], [E, I_pad, H]); both MFMA operands are read
+    // along K, so each stage first writes a K-contiguous copy of its weights
+    g1.W = ws + p.wt1; g1.Kp = p.Hk;
+    g2.W = ws + p.wt2; g2.Kp = p.Iw;
+    if (stages & MOE_STAGE_GATE_UP) {
+      rc = launch_transpose_fp8((const uint8_t*)a->gate_up_proj_weight, ws + p.wt1, a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
+                                a->H * 2 * a->I, a->I, s);
+      if (rc != MOE_OK) return rc;
+    }
+    if (stages & MOE_STAGE_DOWN) {
+      rc = launch_transpose_fp8((const uint8_t*)a->down_proj_weight, ws + p.wt2, a->I, a->H, a->H, p.Iw, a->E, 1,
+                                g.I_pad * a->H, 0, s);
+      if (rc != MOE_OK) return rc;
+    }
   }
 
   const bool mx_fast = a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I);
