@@ -10,6 +10,11 @@
 // K-slice of both operands in LDS in K-contiguous order and lets each of the four waves run
 // 2 x (8|16) MFMA tiles over it.  Rows are gathered through token_position_to_id while the A
 // operand is staged (the gather is fused into the load, no gathered copy exists in HBM).
+// The bf16 and fp8-row weights arrive N-contiguous ([E, H, 2, I], [E, I, H]); both MFMA operands
+// are read along K, so a transposition kernel first writes K-contiguous copies of them, after
+// which both operands are 16-byte copies into LDS and the K loop is software pipelined (loads
+// of step k+1 in flight under the MFMAs of step k).  MXFP8 weights outside the large-tile path
+// keep the reference's x4 layouts and a plain loop.
 //
 // Reference semantics: generate_blockwise_numpy_golden,
 //   test/integration/nkilib/core/moe/moe_cte/test_moe_cte_common.py:267-447 (bf16 / fp8 weight),
@@ -119,14 +124,16 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
   else if (KIND == MOE_KIND_BF16) nks = (int)((a.K + 63) / 64);
   else nks = (int)((a.K + 127) / 128);
 
-  if constexpr (KIND == MOE_KIND_FP8_ROW) {
-    // Both operands are plain 16-byte copies here (the weights were transposed beforehand), so the loop is
-    // software pipelined: the global loads of k-step ks+1 are in flight while the MFMAs of k-step ks run.
+  if constexpr (KIND == MOE_KIND_FP8_ROW || KIND == MOE_KIND_BF16) {
+    // Both operands are plain 16-byte copies here (the weights were transposed to K-contiguous rows of Kp bytes
+    // beforehand), so the loop is software pipelined: the global loads of k-step ks+1 are in flight while the
+    // MFMAs of k-step ks run.  A k-step is 128 bytes of K: 128 fp8 or 64 bf16 elements.
+    const int64_t kbytes = (KIND == MOE_KIND_BF16) ? a.K * 2 : a.K;
     constexpr int PB = NCOLS * 8 / GT;
     uint4 ra[4], rb[PB];
     auto fetch = [&](int ks) {
       const int64_t a_off = (int64_t)ks * 128;
-      const int a_valid = (int)((a.K - a_off < 128) ? (a.K - a_off) : 128);
+      const int a_valid = (int)((kbytes - a_off < 128) ? (kbytes - a_off) : 128);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int row = (tid >> 3) + 32 * j, ch = tid & 7;
@@ -140,7 +147,7 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
         }
         if (src != nullptr && ch * 16 + 16 <= a_valid) {
           src += a_off + ch * 16;
-          if (STAGE == 1) {  // rows of H + 4 bytes are only 4-byte aligned
+          if (KIND == MOE_KIND_FP8_ROW && STAGE == 1) {  // rows of H + 4 bytes are only 4-byte aligned
             const uint32_t* s4 = (const uint32_t*)src;
             val = make_uint4(s4[0], s4[1], s4[2], s4[3]);
           } else {
@@ -176,38 +183,47 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
       }
       __syncthreads();
       if (ks + 1 < nks) fetch(ks + 1);
-      v8i af[2];
+      if constexpr (KIND == MOE_KIND_BF16) {
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) af[mt] = lds_read_frag(sA + (m0 + 16 * mt + c) * LROW, g);
+        for (int sub = 0; sub < 2; ++sub) {
+          v8bf af[2];
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const v8i bf = lds_read_frag(sB + (nt * 16 + c) * LROW, g);
+          for (int mt = 0; mt < 2; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * LROW + sub * 64 + g * 16);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, 127, 0, 127);
+          for (int nt = 0; nt < NT; ++nt) {
+            const v8bf bf = *(const v8bf*)(sB + (nt * 16 + c) * LROW + sub * 64 + g * 16);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+              acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bf, acc[nt][mt], 0, 0, 0);
+          }
+        }
+      } else {
+        v8i af[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) af[mt] = lds_read_frag(sA + (m0 + 16 * mt + c) * LROW, g);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const v8i bf = lds_read_frag(sB + (nt * 16 + c) * LROW, g);
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt)
+            acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, 127, 0, 127);
+        }
       }
       __syncthreads();
     }
   } else
-  for (int ks = 0; ks < nks; ++ks) {
-    // position of this k-step
-    int kt = 0, pb = 0, Ptk = 128;      // MX: K tile (H or I tile), partition group, valid partitions
-    int64_t a_off;                      // byte offset of the slice inside an A row
+  for (int ks = 0; ks < nks; ++ks) {  // MXFP8: the weights stay in the reference's x4 layouts
+    // position of this k-step: K tile (H or I tile), partition group, valid partitions
+    const int kt = ks >> 2, pb = ks & 3;
+    int Ptk = 128;
     int a_valid = 128;                  // valid bytes of the slice
-    if (KIND == MOE_KIND_MXFP8) {
-      kt = ks >> 2; pb = ks & 3;
-      if (STAGE == 2) {
-        const int rows_t = (int)((a.I - (int64_t)kt * 512 < 512) ? (a.I - (int64_t)kt * 512) : 512);
-        Ptk = rows_t / 4;
-        if (pb * 32 >= Ptk) continue;
-        a_valid = (Ptk - pb * 32) * 4 < 128 ? (Ptk - pb * 32) * 4 : 128;
-      }
-      a_off = (int64_t)kt * 512 + pb * 128;
-    } else {
-      a_off = (int64_t)ks * 128;
-      const int64_t kbytes = (KIND == MOE_KIND_BF16) ? a.K * 2 : a.K;
-      a_valid = (int)((kbytes - a_off < 128) ? (kbytes - a_off) : 128);
+    if (STAGE == 2) {
+      const int rows_t = (int)((a.I - (int64_t)kt * 512 < 512) ? (a.I - (int64_t)kt * 512) : 512);
+      Ptk = rows_t / 4;
+      if (pb * 32 >= Ptk) continue;
+      a_valid = (Ptk - pb * 32) * 4 < 128 ? (Ptk - pb * 32) * 4 : 128;
     }
+    const int64_t a_off = (int64_t)kt * 512 + pb * 128;  // byte offset of the slice inside an A row
 
     // ---- stage A: 128 rows x 128 bytes, 8 threads per row ---------------------------------
 #pragma unroll
@@ -223,17 +239,11 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
         if (r0 + row < vr) src = a.A + (slot0 + row) * a.a_stride;
       }
       if (src != nullptr && ch * 16 + 16 <= a_valid) {
-        src += a_off + ch * 16;
-        if (KIND == MOE_KIND_FP8_ROW && STAGE == 1) {  // rows are only 4-byte aligned
-          const uint32_t* s4 = (const uint32_t*)src;
-          val = make_uint4(s4[0], s4[1], s4[2], s4[3]);
-        } else {
-          val = *(const uint4*)src;
-        }
+        val = *(const uint4*)(src + a_off + ch * 16);
       }
       *(uint4*)(sA + row * LROW + ch * 16) = val;
     }
-    if (KIND == MOE_KIND_MXFP8 && tid < TM) {
+    if (tid < TM) {
       uint32_t sv = 0;
       if (STAGE == 1) {
         const int tok = s_tok[tid];
@@ -290,82 +300,24 @@ __global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
           sBs[col] = sv;
         }
       }
-    } else if (KIND == MOE_KIND_BF16) {
-      // 64 k-rows x NCOLS columns of bf16 (or fp8 widened to bf16)
-      constexpr int CP = NCOLS / 2;        // column pairs
-      constexpr int RSTEP = GT / CP;       // k-rows covered per pass
-      const int cp = tid % CP, kr0 = tid / CP;
-      const bool w8 = a.weight_dtype == MOE_DT_FP8_E4M3;
-#pragma unroll 4
-      for (int j = 0; j < 64 / RSTEP; ++j) {
-        const int kr = kr0 + RSTEP * j;
-        const int64_t k = (int64_t)ks * 64 + kr;
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          const int col = 2 * cp + cc;
-          uint16_t v = 0;
-          int64_t idx = -1;
-          if (STAGE == 1) {
-            const int gu = col >> 7;
-            const int64_t i = c0 + (col & 127);
-            if (k < a.H && i < a.I) idx = (((int64_t)e * a.H + k) * 2 + gu) * a.I + i;
-          } else {
-            const int64_t h = c0 + col;
-            if (k < a.I && h < a.H) idx = ((int64_t)e * a.I_pad + k) * a.H + h;
-          }
-          if (idx >= 0) v = w8 ? f32_to_bf16_bits(e4m3_to_f32(a.W[idx])) : ((const uint16_t*)a.W)[idx];
-          *(uint16_t*)(sB + col * LROW + kr * 2) = v;
-        }
-      }
-    } else {  // FP8_ROW: the weights were transposed to K-contiguous rows of Kp bytes beforehand; staged like A
-      constexpr int PER = NCOLS * 8 / GT;
-#pragma unroll
-      for (int j = 0; j < PER; ++j) {
-        const int idx = tid + GT * j;
-        const int col = idx >> 3, ch = idx & 7;
-        uint4 val = make_uint4(0, 0, 0, 0);
-        if (STAGE == 1) {
-          const int gu = col >> 7;
-          const int64_t i = c0 + (col & 127);
-          if (i < a.I) val = *(const uint4*)(a.W + (((int64_t)e * 2 + gu) * a.I + i) * a.Kp + (int64_t)ks * 128 + ch * 16);
-        } else {
-          const int64_t h = c0 + col;
-          if (h < a.H) val = *(const uint4*)(a.W + ((int64_t)e * a.H + h) * a.Kp + (int64_t)ks * 128 + ch * 16);
-        }
-        *(uint4*)(sB + col * LROW + ch * 16) = val;
-      }
     }
     __syncthreads();
 
     // ---- MFMA ------------------------------------------------------------------------------
-    if (KIND == MOE_KIND_BF16) {
-#pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
-        v8bf af[2];
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * LROW + sub * 64 + g * 16);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const v8bf bf = *(const v8bf*)(sB + (nt * 16 + c) * LROW + sub * 64 + g * 16);
-#pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
-            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bf, acc[nt][mt], 0, 0, 0);
-        }
-      }
-    } else {
+    {
       v8i af[2];
       int sa[2];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         const int row = m0 + 16 * mt + c;
         af[mt] = lds_read_frag(sA + row * LROW, g);
-        sa[mt] = (KIND == MOE_KIND_MXFP8) ? (int)((sAs[row] >> (8 * g)) & 0xffu) : 127;
+        sa[mt] = (int)((sAs[row] >> (8 * g)) & 0xffu);
       }
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
         const int col = nt * 16 + c;
         const v8i bf = lds_read_frag(sB + col * LROW, g);
-        const int sb = (KIND == MOE_KIND_MXFP8) ? (int)((sBs[col] >> (8 * g)) & 0xffu) : 127;
+        const int sb = (int)((sBs[col] >> (8 * g)) & 0xffu);
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
           acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, sa[mt], 0, sb);
@@ -571,6 +523,74 @@ __global__ __launch_bounds__(256) void transpose_fp8_kernel(const uint8_t* __res
     }
     *(uint4*)(D + (n0 + nn) * Kp + k0 + kc) = make_uint4(w[0], w[1], w[2], w[3]);
   }
+}
+
+// The same for the bf16 kind: batches of [R, C] bf16 (W8 == false) or fp8-e4m3 widened to bf16 (W8 == true)
+// -> bf16 [C, Kp] with Kp (elements) a multiple of 64.
+template <bool W8>
+__global__ __launch_bounds__(256) void transpose_w16_kernel(const uint8_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                            int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
+                                                            int nb1, int64_t src_bs0, int64_t src_bs1, int64_t dst_bs) {
+  __shared__ __attribute__((aligned(16))) uint16_t tile[64][72];
+  constexpr int ES = W8 ? 1 : 2;
+  const int b = blockIdx.z;
+  const uint8_t* S = src + ((int64_t)(b / nb1) * src_bs0 + (int64_t)(b % nb1) * src_bs1) * ES;
+  uint16_t* D = dst + (int64_t)b * dst_bs;
+  const int64_t n0 = (int64_t)blockIdx.x * 64, k0 = (int64_t)blockIdx.y * 64;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int idx = threadIdx.x + 256 * j;
+    const int r = idx >> 3, c8 = (idx & 7) * 8;
+    const int64_t k = k0 + r, n = n0 + c8;
+    uint16_t v[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) v[q] = 0;
+    if (k < R) {
+      const uint8_t* p = S + (k * src_row_stride + n) * ES;
+      if (n + 8 <= C && (((uintptr_t)p) & (8 * ES - 1)) == 0) {
+        if (W8) {
+          const uint2 raw = *(const uint2*)p;
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            v[q] = f32_to_bf16_bits(e4m3_to_f32(((q < 4 ? raw.x : raw.y) >> (8 * (q & 3))) & 0xffu));
+        } else {
+          *(uint4*)v = *(const uint4*)p;
+        }
+      } else {
+        for (int q = 0; q < 8; ++q)
+          if (n + q < C) v[q] = W8 ? f32_to_bf16_bits(e4m3_to_f32(p[q])) : ((const uint16_t*)p)[q];
+      }
+    }
+    *(uint4*)(&tile[r][c8]) = *(const uint4*)v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int idx = threadIdx.x + 256 * j;
+    const int nn = idx >> 3, kc = (idx & 7) * 8;
+    if (n0 + nn < C) {
+      uint32_t w[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[q] = (uint32_t)tile[kc + 2 * q][nn] | ((uint32_t)tile[kc + 2 * q + 1][nn] << 16);
+      *(uint4*)(D + (n0 + nn) * Kp + k0 + kc) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+}
+
+int launch_transpose_w16(const void* src, int w8, uint16_t* dst, int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
+                         int64_t nb0, int nb1, int64_t src_bs0, int64_t src_bs1, hipStream_t s) {
+  if ((Kp & 63) != 0 || Kp < R || (((uintptr_t)dst) & 15) != 0) return MOE_E_BAD_ARG;
+  const int64_t gx = (C + 63) / 64, gy = Kp / 64, gz = nb0 * nb1;
+  if (gy > 65535 || gz > 65535) return MOE_E_BAD_SHAPE;
+  const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)gz);
+  if (w8)
+    hipLaunchKernelGGL(transpose_w16_kernel<true>, grid, dim3(256), 0, s, (const uint8_t*)src, dst, R, C, src_row_stride,
+                       Kp, nb1, src_bs0, src_bs1, C * Kp);
+  else
+    hipLaunchKernelGGL(transpose_w16_kernel<false>, grid, dim3(256), 0, s, (const uint8_t*)src, dst, R, C, src_row_stride,
+                       Kp, nb1, src_bs0, src_bs1, C * Kp);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
 }
 
 int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,

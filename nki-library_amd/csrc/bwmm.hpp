@@ -35,7 +35,7 @@ struct GemmArgs {
   int32_t act_fn, scaling_mode, clamp_mask;
   float clamp[4];          // gate hi, gate lo, up hi, up lo
   int32_t pI, nI;          // MXFP8: partitions per intermediate tile in the down weight, number of tiles
-  int64_t Kp;              // FP8_ROW: bytes per row of the transposed (K-contiguous) weights W points to
+  int64_t Kp;              // BF16 / FP8_ROW: bytes per row of the transposed (K-contiguous) weights W points to
   uint16_t* ckpt;          // BF16 kind, nullable: stage 1 gate/up checkpoint [N, 2, I, B], stage 2 down checkpoint [N, B, H]
 };
 
@@ -78,6 +78,9 @@ int launch_mx_gemm(int stage, const MxArgs& m, unsigned gx, unsigned gy, hipStre
 
 int launch_gemm_stage(int kind, int stage, const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s);
 // batches [nb0][nb1] of byte matrices [R, C] -> [C, Kp] (K-contiguous, zero tail), see bwmm.hip
+// the bf16 kind: [R, C] bf16 (or fp8 widened to bf16 when w8) -> bf16 [C, Kp], Kp in elements, a multiple of 64
+int launch_transpose_w16(const void* src, int w8, uint16_t* dst, int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
+                         int64_t nb0, int nb1, int64_t src_bs0, int64_t src_bs1, hipStream_t s);
 int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
                          int64_t nb0, int nb1, int64_t src_bs0, int64_t src_bs1, hipStream_t s);
 int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,

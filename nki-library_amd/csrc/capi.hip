@@ -38,7 +38,7 @@ inline size_t al256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Plan {
   size_t book, xq, xs, y, yq, ys, d, wt1, wt2, total;
-  int64_t Hk;      // FP8_ROW: H padded to the K step, row length of the transposed gate/up weights
+  int64_t Hk;      // BF16 / FP8_ROW: H padded to the K step, row length (elements) of the transposed gate/up weights
   int64_t Iw;      // padded intermediate width (elements) of the stage-2 A operand
   int64_t pI, nI;  // MXFP8
 };
@@ -117,6 +117,10 @@ Plan make_plan(const moe_bwmm_args* a) {
   } else if (a->kind == MOE_KIND_BF16) {
     p.Iw = (a->I + 63) / 64 * 64;
     p.y = off; off += al256(slots * (size_t)p.Iw * 2);
+    // K-contiguous bf16 copies of the weights: [E, 2, I, Hk] and [E, H, Iw]
+    p.Hk = (a->H + 63) / 64 * 64;
+    p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk * 2);
+    p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw * 2);
   } else {
     p.Iw = (a->I + 127) / 128 * 128;
     p.y = off; off += al256(slots * (size_t)a->I * 4);
@@ -215,6 +219,20 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     g1.out = ws + p.y; g1.out_stride = p.Iw * 2;
     g2.A = ws + p.y; g2.a_stride = p.Iw * 2; g2.K = p.Iw;
     gx1 = (unsigned)((a->I + 127) / 128);
+    // K-contiguous bf16 copies of the weights (fp8 weights are widened on the way), as for the fp8-row kind below
+    g1.W = ws + p.wt1; g1.Kp = p.Hk * 2;
+    g2.W = ws + p.wt2; g2.Kp = p.Iw * 2;
+    const int w8 = a->weight_dtype == MOE_DT_FP8_E4M3;
+    if (stages & MOE_STAGE_GATE_UP) {
+      rc = launch_transpose_w16(a->gate_up_proj_weight, w8, (uint16_t*)(ws + p.wt1), a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
+                                a->H * 2 * a->I, a->I, s);
+      if (rc != MOE_OK) return rc;
+    }
+    if (stages & MOE_STAGE_DOWN) {
+      rc = launch_transpose_w16(a->down_proj_weight, w8, (uint16_t*)(ws + p.wt2), a->I, a->H, a->H, p.Iw, a->E, 1,
+                                g.I_pad * a->H, 0, s);
+      if (rc != MOE_OK) return rc;
+    }
   } else {
     g1.A = (const uint8_t*)a->hidden_states; g1.a_stride = a->H + 4; g1.K = a->H;
     g1.out = ws + p.y; g1.out_stride = a->I * 4;
