@@ -9,7 +9,10 @@ GEMM with fused affinity scaling, and the per-token combine into bf16 rows.
 Default workload: BASELINE config 4, DeepSeek-V3-shaped routed experts (T=8192, H=7168, I=2048,
 E=256, top-8, block 128, MXFP8 weights ~11 GB).  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c5-<T>] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c5-<T>|c2] [--no-cpu-baseline]
+
+`--workload c2` times BASELINE config 2 instead (fp8 activations with a per-row scale from RMSNorm-Quant, fp8
+weights with per-channel scales, Mixtral-8x7B shape) through the same entry points.
 """
 
 import argparse
@@ -130,12 +133,125 @@ def cpu_baseline(cfg, t, tp2id, b2e, n_blocks):
     }
 
 
+def bench_fp8_row(args):
+    """BASELINE config 2: RMSNorm-Quant (fp8 rows + fp32 row scale) -> block build -> fp8-row blockwise layer."""
+    import numpy as np
+    import torch
+    from nkilib import _native as nv
+    from nkilib import synthetic as syn
+    from nkilib.core.moe.moe_cte import (MoECTEImplementation, MoECTESpec, QuantizationConfig, build_token_blocks,
+                                         get_n_blocks, moe_cte)
+    from nkilib.core.moe.moe_cte import _launch
+    from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+
+    dev = torch.device("cuda:0")
+    nv.check(nv.lib().moe_check_device(), "device check")
+    cfg = dict(syn.CONFIGS["c2"])
+    T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
+    gu_q, gu_s, d_q, d_s = syn.fp8_channel_weights(E, H, I, 0.02, dev, seed=0)
+    ids, aff = syn.route(T, E, k, dev, seed=0, mode="softmax")
+    x = syn.hidden_states(T, H, dev, seed=0)
+    gamma = torch.ones((1, H), dtype=torch.bfloat16, device=dev)
+    N = get_n_blocks(T, k, E, B)
+    spec = MoECTESpec(implementation=MoECTEImplementation.shard_on_block)
+    qcfg = QuantizationConfig(gu_s, d_s)
+    gu8, d8 = gu_q.view(torch.float8_e4m3fn), d_q.view(torch.float8_e4m3fn)
+    names = ["norm_quant", "build_blocks", "prep", "gate_up", "requant", "down", "combine"]
+    events = []
+
+    def rec():
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        events[-1].append(ev)
+
+    def step(timed):
+        if timed:
+            events.append([])
+            rec()
+        recs = rmsnorm_quant_kernel(x, gamma, RmsNormQuantKernelArgs())
+        if timed:
+            rec()
+        tp2id, b2e, cond = build_token_blocks(ids, E, B, N)
+        if timed:
+            rec()
+        _launch.stage_callback = (lambda name: rec()) if timed else None
+        out = moe_cte[2](recs, aff.reshape(-1, 1), gu8, d8, tp2id, b2e, B, spec, quantization_config=qcfg)
+        _launch.stage_callback = None
+        return out, recs, tp2id, b2e
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, recs, tp2id, b2e = step(True)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    stage_ms = {n: 0.0 for n in names}
+    for evs in events:
+        assert len(evs) == len(names) + 1, (len(evs), names)
+        for i, n in enumerate(names):
+            stage_ms[n] += evs[i].elapsed_time(evs[i + 1]) / args.steps
+    routed = int((tp2id.reshape(-1) < T).sum().item())
+    flops_layer, flops_gu = 6.0 * routed * H * I, 4.0 * routed * H * I
+    tflops = flops_layer / (ms_per_step * 1e-3) / 1e12
+    gu_tflops = flops_gu / (stage_ms["gate_up"] * 1e-3) / 1e12
+    # gate/up stage: the K-contiguous copy of the expert weights (read + write) and the GEMM
+    gu_bytes = E * 2 * H * I * 3 + routed * (H + 4) + routed * I * 4
+    roofline = {"bound": "mfma", "achieved": round(gu_tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(gu_tflops / PEAK_FP8_TFLOPS, 4), "traffic": None,
+                "kernel": "moe::transpose_fp8_kernel + moe::bwmm_kernel<1, 1> (gate/up stage of the fp8-row kind: "
+                          "K-contiguous weight copy, then the blockwise GEMM with fused act*up)",
+                "algorithmic_bytes": int(gu_bytes), "algorithmic_flops": int(flops_gu),
+                "avg_launch_ms": round(stage_ms["gate_up"], 4)}
+    res = {
+        "metric": METRIC, "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp8_e4m3 (per-row activation scale, per-channel weight scale, fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"c2: fp8-row blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} (N={N} blocks, "
+                               f"{routed} routed rows), RMSNorm-Quant front end + block build + gate/up + row re-quantise "
+                               f"+ down + combine",
+                   "T": T, "H": H, "I": I, "E": E, "top_k": k, "block_size": B},
+        "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
+        "pct_of_fp8_mfma_peak": round(100.0 * tflops / PEAK_FP8_TFLOPS, 2),
+        "stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        from oracle import moe as omoe
+
+        tpb = tp2id.cpu().numpy().reshape(-1, B)
+        be = b2e.cpu().numpy()
+        keep = [b for b in range(tpb.shape[0]) if (tpb[b] < T).any()][:24]
+        experts = sorted(set(int(be[b]) for b in keep))
+        remap = {e: i for i, e in enumerate(experts)}
+        sel = torch.tensor(experts, device=dev)
+        raw = recs.view(torch.uint8).cpu().numpy()
+        codes, scale = raw[:, :H], raw[:, H:].copy().view(np.float32).reshape(-1)
+        aff_np = aff.float().cpu().numpy()[:, experts]
+        tp_s = np.concatenate([tpb[b] for b in keep])
+        be_s = np.array([remap[int(be[b])] for b in keep], dtype=np.int32)
+        rows = int(sum((tpb[b] < T).sum() for b in keep))
+        wq = [w[sel].cpu().numpy() for w in (gu_q, d_q, gu_s, d_s)]
+        t0 = time.perf_counter()
+        omoe.moe_blockwise_fp8_row_ref(codes, scale, aff_np, wq[0], wq[1], wq[2], wq[3], tp_s, be_s, B)
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": 6.0 * rows * H * I / dt / 1e12, "unit": "TFLOP/s", "cores": os.cpu_count(),
+                               "kind": "port",
+                               "sample": f"first {len(keep)} non-empty blocks ({rows} routed rows) of the same workload, "
+                                         f"numpy oracle, {dt:.1f} s"}
+    print(json.dumps(res), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "c2":
+        return bench_fp8_row(args)
     import torch
 
     from nkilib import _native as nv

@@ -50,8 +50,11 @@ __device__ __forceinline__ v8i lds_read_frag(const uint8_t* row, int g) {
   return r;
 }
 
+// (the bf16 and fp8-row kinds are held to 256 registers so that two workgroups share a CU and cover each other's
+// barriers: their 128 x 256 stage-1 tile alone needs 128 accumulator registers)
 template <int KIND, int STAGE>
-__global__ __launch_bounds__(GT) void bwmm_kernel(const GemmArgs a) {
+__global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_KIND_MXFP8 ? 1 : 2, 8))) void bwmm_kernel(
+    const GemmArgs a) {
   constexpr int NCOLS = (STAGE == 1) ? 256 : 128;
   constexpr int NT = NCOLS / 16;
   __shared__ __attribute__((aligned(16))) uint8_t sA[TM * LROW];
