@@ -232,6 +232,11 @@ typedef struct moe_bwmm_args {
    * blocks that conditions stops are zero. */
   void* gate_up_activations_T;
   void* down_activations;
+  /* Optional K-contiguous copies of the bf16 / fp8 weights of the BF16 and FP8_ROW kinds, made once by
+   * moe_prepare_kmajor_weights (they depend on the weights only).  Both NULL: every call makes its own copies
+   * in the workspace.  Ignored by the MXFP8 kind, whose x4 layouts are K-major already. */
+  const void* gate_up_proj_weight_kmajor;
+  const void* down_proj_weight_kmajor;
 } moe_bwmm_args;
 
 /* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /
@@ -257,6 +262,15 @@ int moe_blockwise(const moe_bwmm_args* args, void* stream);
 #define MOE_STAGE_COMBINE 32u  /* per-token accumulation of the contributions into the output        */
 #define MOE_STAGE_ALL 63u
 int moe_blockwise_stages(const moe_bwmm_args* args, unsigned stages, void* stream);
+
+/* No counterpart in the reference, whose dense weights are consumed N-contiguous ([E, H, 2, I], [E, I_pad, H]):
+ * the MFMA operands of the BF16 and FP8_ROW kinds are read along K, so the GEMMs run on K-contiguous copies
+ * ([E, 2, I, Hk] and [E, H, Ik]; bf16 for the BF16 kind, fp8 weights widened; fp8 for FP8_ROW; tails zero).
+ * A caller whose weights do not change (inference) makes the copies once and passes them in
+ * moe_bwmm_args.*_kmajor.  moe_kmajor_weights_bytes: bytes of the gate/up (which == 0) or down (which == 1)
+ * copy for these args, 0 if the kind has none.  moe_prepare_kmajor_weights fills both (256-byte aligned). */
+size_t moe_kmajor_weights_bytes(const moe_bwmm_args* args, int which);
+int moe_prepare_kmajor_weights(const moe_bwmm_args* args, void* gate_up_kmajor, void* down_kmajor, void* stream);
 
 #ifdef __cplusplus
 }

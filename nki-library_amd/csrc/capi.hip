@@ -22,7 +22,7 @@ extern "C" const char* moe_error_string(int code) {
   }
 }
 
-extern "C" int moe_abi_version(void) { return 2; }
+extern "C" int moe_abi_version(void) { return 3; }
 
 extern "C" int moe_check_device(void) {
   int dev = 0;
@@ -119,8 +119,8 @@ Plan make_plan(const moe_bwmm_args* a) {
     p.y = off; off += al256(slots * (size_t)p.Iw * 2);
     // K-contiguous bf16 copies of the weights: [E, 2, I, Hk] and [E, H, Iw]
     p.Hk = (a->H + 63) / 64 * 64;
-    p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk * 2);
-    p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw * 2);
+    if (!a->gate_up_proj_weight_kmajor) { p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk * 2); }
+    if (!a->down_proj_weight_kmajor) { p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw * 2); }
   } else {
     p.Iw = (a->I + 127) / 128 * 128;
     p.y = off; off += al256(slots * (size_t)a->I * 4);
@@ -128,15 +128,51 @@ Plan make_plan(const moe_bwmm_args* a) {
     p.ys = off; off += al256(slots * 4);
     // K-contiguous copies of the fp8 weights: [E, 2, I, Hk] and [E, H, Iw]
     p.Hk = (a->H + 127) / 128 * 128;
-    p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk);
-    p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw);
+    if (!a->gate_up_proj_weight_kmajor) { p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk); }
+    if (!a->down_proj_weight_kmajor) { p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw); }
   }
   p.d = off; off += al256(slots * (size_t)a->H * 2);
   p.total = off;
   return p;
 }
 
+// K-contiguous copy of the gate/up (which == 0) or down (which == 1) weights of the BF16 / FP8_ROW kinds.
+int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hipStream_t s) {
+  const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
+  if (a->kind == MOE_KIND_BF16) {
+    const int w8 = a->weight_dtype == MOE_DT_FP8_E4M3;
+    if (which == 0)
+      return launch_transpose_w16(a->gate_up_proj_weight, w8, (uint16_t*)dst, a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
+                                  a->H * 2 * a->I, a->I, s);
+    return launch_transpose_w16(a->down_proj_weight, w8, (uint16_t*)dst, a->I, a->H, a->H, p.Iw, a->E, 1, Ipad * a->H, 0, s);
+  }
+  if (which == 0)
+    return launch_transpose_fp8((const uint8_t*)a->gate_up_proj_weight, (uint8_t*)dst, a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
+                                a->H * 2 * a->I, a->I, s);
+  return launch_transpose_fp8((const uint8_t*)a->down_proj_weight, (uint8_t*)dst, a->I, a->H, a->H, p.Iw, a->E, 1,
+                              Ipad * a->H, 0, s);
+}
+
 }  // namespace
+
+extern "C" size_t moe_kmajor_weights_bytes(const moe_bwmm_args* a, int which) {
+  if (validate(a) != MOE_OK || a->kind == MOE_KIND_MXFP8 || which < 0 || which > 1) return 0;
+  const Plan p = make_plan(a);
+  const size_t es = a->kind == MOE_KIND_BF16 ? 2 : 1;
+  return which == 0 ? (size_t)a->E * 2 * a->I * p.Hk * es : (size_t)a->E * a->H * p.Iw * es;
+}
+
+extern "C" int moe_prepare_kmajor_weights(const moe_bwmm_args* a, void* gate_up_kmajor, void* down_kmajor, void* stream) {
+  int rc = validate(a);
+  if (rc != MOE_OK) return rc;
+  if (a->kind == MOE_KIND_MXFP8) return MOE_E_UNSUPPORTED;
+  if (!gate_up_kmajor || !down_kmajor) return MOE_E_BAD_ARG;
+  if ((((uintptr_t)gate_up_kmajor) & 255) != 0 || (((uintptr_t)down_kmajor) & 255) != 0) return MOE_E_BAD_ARG;
+  const Plan p = make_plan(a);
+  rc = kmajor_copy(a, p, 0, gate_up_kmajor, (hipStream_t)stream);
+  if (rc != MOE_OK) return rc;
+  return kmajor_copy(a, p, 1, down_kmajor, (hipStream_t)stream);
+}
 
 extern "C" size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* a) {
   if (validate(a) != MOE_OK) return 0;
@@ -220,17 +256,16 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     g2.A = ws + p.y; g2.a_stride = p.Iw * 2; g2.K = p.Iw;
     gx1 = (unsigned)((a->I + 127) / 128);
     // K-contiguous bf16 copies of the weights (fp8 weights are widened on the way), as for the fp8-row kind below
-    g1.W = ws + p.wt1; g1.Kp = p.Hk * 2;
-    g2.W = ws + p.wt2; g2.Kp = p.Iw * 2;
-    const int w8 = a->weight_dtype == MOE_DT_FP8_E4M3;
-    if (stages & MOE_STAGE_GATE_UP) {
-      rc = launch_transpose_w16(a->gate_up_proj_weight, w8, (uint16_t*)(ws + p.wt1), a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
-                                a->H * 2 * a->I, a->I, s);
+    g1.W = a->gate_up_proj_weight_kmajor ? (const uint8_t*)a->gate_up_proj_weight_kmajor : ws + p.wt1;
+    g2.W = a->down_proj_weight_kmajor ? (const uint8_t*)a->down_proj_weight_kmajor : ws + p.wt2;
+    g1.Kp = p.Hk * 2;
+    g2.Kp = p.Iw * 2;
+    if ((stages & MOE_STAGE_GATE_UP) && !a->gate_up_proj_weight_kmajor) {
+      rc = kmajor_copy(a, p, 0, ws + p.wt1, s);
       if (rc != MOE_OK) return rc;
     }
-    if (stages & MOE_STAGE_DOWN) {
-      rc = launch_transpose_w16(a->down_proj_weight, w8, (uint16_t*)(ws + p.wt2), a->I, a->H, a->H, p.Iw, a->E, 1,
-                                g.I_pad * a->H, 0, s);
+    if ((stages & MOE_STAGE_DOWN) && !a->down_proj_weight_kmajor) {
+      rc = kmajor_copy(a, p, 1, ws + p.wt2, s);
       if (rc != MOE_OK) return rc;
     }
   } else {
@@ -240,16 +275,16 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     gx1 = (unsigned)((a->I + 127) / 128);
     // the reference stores the weights N-contiguous ([E, H, 2, I], [E, I_pad, H]); both MFMA operands are read
     // along K, so each stage first writes a K-contiguous copy of its weights
-    g1.W = ws + p.wt1; g1.Kp = p.Hk;
-    g2.W = ws + p.wt2; g2.Kp = p.Iw;
-    if (stages & MOE_STAGE_GATE_UP) {
-      rc = launch_transpose_fp8((const uint8_t*)a->gate_up_proj_weight, ws + p.wt1, a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
-                                a->H * 2 * a->I, a->I, s);
+    g1.W = a->gate_up_proj_weight_kmajor ? (const uint8_t*)a->gate_up_proj_weight_kmajor : ws + p.wt1;
+    g2.W = a->down_proj_weight_kmajor ? (const uint8_t*)a->down_proj_weight_kmajor : ws + p.wt2;
+    g1.Kp = p.Hk;
+    g2.Kp = p.Iw;
+    if ((stages & MOE_STAGE_GATE_UP) && !a->gate_up_proj_weight_kmajor) {
+      rc = kmajor_copy(a, p, 0, ws + p.wt1, s);
       if (rc != MOE_OK) return rc;
     }
-    if (stages & MOE_STAGE_DOWN) {
-      rc = launch_transpose_fp8((const uint8_t*)a->down_proj_weight, ws + p.wt2, a->I, a->H, a->H, p.Iw, a->E, 1,
-                                g.I_pad * a->H, 0, s);
+    if ((stages & MOE_STAGE_DOWN) && !a->down_proj_weight_kmajor) {
+      rc = kmajor_copy(a, p, 1, ws + p.wt2, s);
       if (rc != MOE_OK) return rc;
     }
   }

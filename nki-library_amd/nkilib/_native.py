@@ -43,6 +43,8 @@ EXPORTED_SYMBOLS = (
     "moe_blockwise_workspace_bytes",
     "moe_blockwise",
     "moe_blockwise_stages",
+    "moe_kmajor_weights_bytes",
+    "moe_prepare_kmajor_weights",
 )
 
 
@@ -93,6 +95,8 @@ class BwmmArgs(ctypes.Structure):
         ("up_clamp_lower", c_float),
         ("gate_up_activations_T", c_void_p),
         ("down_activations", c_void_p),
+        ("gate_up_proj_weight_kmajor", c_void_p),
+        ("down_proj_weight_kmajor", c_void_p),
     ]
 
 
@@ -151,6 +155,10 @@ def lib():
     L.moe_blockwise_workspace_bytes.argtypes = [POINTER(BwmmArgs)]
     L.moe_blockwise.restype = c_int
     L.moe_blockwise.argtypes = [POINTER(BwmmArgs), c_void_p]
+    L.moe_kmajor_weights_bytes.restype = c_size_t
+    L.moe_kmajor_weights_bytes.argtypes = [POINTER(BwmmArgs), c_int]
+    L.moe_prepare_kmajor_weights.restype = c_int
+    L.moe_prepare_kmajor_weights.argtypes = [POINTER(BwmmArgs), c_void_p, c_void_p, c_void_p]
     L.moe_blockwise_stages.restype = c_int
     L.moe_blockwise_stages.argtypes = [POINTER(BwmmArgs), ctypes.c_uint, c_void_p]
     _lib = L

@@ -3,6 +3,7 @@ reference kernels do (kernel_assert), allocates the output in the reference's
 return shape, and calls ``moe_blockwise`` of libmoe_gfx950.so."""
 
 import ctypes
+import weakref
 from typing import Optional
 
 import torch
@@ -26,6 +27,44 @@ _STAGES = (
     ("down", nv.STAGE_DOWN),
     ("combine", nv.STAGE_COMBINE),
 )
+
+
+# K-contiguous copies of the dense (bf16 / fp8) expert weights, kept per weight tensor pair: the GEMMs of the bf16
+# and fp8-row kinds read both operands along K while the reference's layouts are N-contiguous, and the copies
+# depend on the weights only.  An entry lives as long as both weight tensor objects do and is remade when either
+# was modified in place (torch's version counter).  Costs one more copy of the weights in HBM (two for fp8 weights
+# of the bf16 kind, which are widened); ``kmajor_weight_cache = False`` makes every call build its copies in the
+# workspace instead.
+kmajor_weight_cache = True
+_KMAJOR_MAX_ENTRIES = 64
+_kmajor = {}
+
+
+def clear_kmajor_weight_cache():
+    _kmajor.clear()
+
+
+def _kmajor_weights(L, a, guw, dw, dev):
+    key = (id(guw), id(dw))
+    sig = (guw._version, dw._version, guw.data_ptr(), dw.data_ptr(), tuple(guw.shape), tuple(dw.shape), guw.dtype,
+           dw.dtype, int(a.kind), int(a.weight_dtype), int(a.I_pad))
+    ent = _kmajor.get(key)
+    if ent is not None and ent[0]() is guw and ent[1]() is dw and ent[2] == sig:
+        return ent[3], ent[4]
+    n0 = L.moe_kmajor_weights_bytes(ctypes.byref(a), 0)
+    n1 = L.moe_kmajor_weights_bytes(ctypes.byref(a), 1)
+    if n0 == 0 or n1 == 0:
+        return None, None
+    k0 = torch.empty(n0, dtype=torch.uint8, device=dev)
+    k1 = torch.empty(n1, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        nv.check(L.moe_prepare_kmajor_weights(ctypes.byref(a), nv.ptr(k0), nv.ptr(k1), nv.stream_ptr(dev)),
+                 "moe_cte (K-contiguous weight copies)")
+    if len(_kmajor) >= _KMAJOR_MAX_ENTRIES:
+        _kmajor.pop(next(iter(_kmajor)))
+    drop = lambda _ref, key=key: _kmajor.pop(key, None)
+    _kmajor[key] = (weakref.ref(guw, drop), weakref.ref(dw, drop), sig, k0, k1)
+    return k0, k1
 
 
 def run_blockwise(
@@ -154,6 +193,12 @@ def run_blockwise(
     if checkpoint_down:
         ck_down = torch.empty((N, B, H), dtype=torch.bfloat16, device=dev)
         a.down_activations = nv.ptr(ck_down)
+
+    kmajor = (None, None)
+    if kmajor_weight_cache and kind in (nv.KIND_BF16, nv.KIND_FP8_ROW):
+        kmajor = _kmajor_weights(L, a, gate_up_proj_weight, down_proj_weight, dev)
+        a.gate_up_proj_weight_kmajor = nv.ptr(kmajor[0])
+        a.down_proj_weight_kmajor = nv.ptr(kmajor[1])
 
     need = L.moe_blockwise_workspace_bytes(ctypes.byref(a))
     if need == 0:

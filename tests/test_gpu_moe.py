@@ -195,6 +195,55 @@ def test_dropping_variant(mode, on_I):
         _check(from_bf16_tensor(outs[2]), g_d, "dropping down_activations")
 
 
+@pytest.mark.parametrize("fp8_row", [False, True])
+def test_kmajor_weight_cache(fp8_row):
+    """The K-contiguous weight copies kept across calls give the same bits as the copies a call makes for itself,
+    and an in-place change of the weights remakes them."""
+    import torch
+    from nkilib.core.moe.moe_cte import MoECTEImplementation, MoECTESpec, QuantizationConfig, _launch, moe_cte
+    from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+
+    dev = torch.device("cuda:0")
+    c = dense_case(256, 512, 384, 4, 2, 128, seed=11, quant=fp8_row, hidden_std=1.0)
+    kw = {}
+    if fp8_row:
+        gu = u8_tensor(c["gate_up_q"], dev).view(torch.float8_e4m3fn)
+        dw = u8_tensor(c["down_q"], dev).view(torch.float8_e4m3fn)
+        kw["quantization_config"] = QuantizationConfig(f32_tensor(c["gate_up_scale"], dev), f32_tensor(c["down_scale"], dev))
+        x = rmsnorm_quant_kernel(bf16_tensor(c["hidden"], dev), bf16_tensor(np.ones((1, 512), np.float32), dev),
+                                 RmsNormQuantKernelArgs())
+    else:
+        gu, dw = bf16_tensor(c["gate_up_w"], dev), bf16_tensor(c["down_w"], dev)
+        x = bf16_tensor(c["hidden"], dev)
+    aff, tp, be = bf16_tensor(c["aff"].reshape(-1, 1), dev), i32_tensor(c["tp2id"], dev), i32_tensor(c["b2e"], dev)
+
+    def run():
+        o = moe_cte(x, aff, gu, dw, tp, be, 128, MoECTESpec(implementation=MoECTEImplementation.shard_on_i), **kw)
+        torch.cuda.synchronize()
+        return o.clone()
+
+    _launch.clear_kmajor_weight_cache()
+    try:
+        _launch.kmajor_weight_cache = False
+        plain = run()
+        _launch.kmajor_weight_cache = True
+        first, second = run(), run()
+        assert len(_launch._kmajor) == 1
+        assert torch.equal(first, plain) and torch.equal(second, plain)
+        # in-place change of one expert's down weights: the cached copies must not survive it
+        if fp8_row:
+            dw.view(torch.uint8)[0].bitwise_xor_(0x80)  # flips the sign of every weight of expert 0
+        else:
+            dw[0].neg_()
+        changed = run()
+        _launch.kmajor_weight_cache = False
+        assert torch.equal(changed, run())
+        assert not torch.equal(changed, plain)
+    finally:
+        _launch.kmajor_weight_cache = True
+        _launch.clear_kmajor_weight_cache()
+
+
 def test_dense_conditions_stop():
     """Hybrid variant: blocks from the first conditions[b] == 0 on are skipped."""
     c = dense_case(256, 512, 256, 8, 2, 128, seed=4, hidden_std=1.0)
