@@ -20,7 +20,8 @@
 // fragment reads are conflict free, and the token fragments into six register sets (five steps ahead:
 // that stream comes from HBM); loads and waits are written as instructions (a wave's loads complete in
 // issue order, so a wait names how many of the most recent ones may still be out), one barrier per
-// step.  What bounds a step is the LDS: every wave reads the whole 32 KB slice of wt for its 16 tokens.
+// step.  What bounds a step is what the CU's L1 can bring in: 40 KB per step and workgroup (the 32 KB slice
+// of wt from L2, 8 KB of token rows), about 16 bytes per cycle.
 #include <type_traits>
 
 #include "common.hpp"
