@@ -474,12 +474,32 @@ __global__ __launch_bounds__(256) void row_requant_kernel(const float* __restric
   const int64_t b = slot / B, r = slot % B;
   if (b >= *n_active || r >= valid_rows[b]) return;
   const float* y = Y + slot * I;
+  uint8_t* q = Yq + slot * Iw;
+  constexpr int MAXV = 16;  // float4 per thread kept in registers: rows of up to 16384 values are read once
+  if (I % 4 == 0 && I <= (int64_t)MAXV * 4 * 256) {
+    float4 v[MAXV];
+    float am = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+      const int64_t i = ((int64_t)j * 256 + threadIdx.x) * 4;
+      v[j] = (i < I) ? *(const float4*)(y + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+      am = fmaxf(fmaxf(am, fmaxf(fabsf(v[j].x), fabsf(v[j].y))), fmaxf(fabsf(v[j].z), fabsf(v[j].w)));
+    }
+    am = block_max(am, red);
+    const float sc = fmaxf(am / 240.0f, 1e-05f);
+    if (threadIdx.x == 0) ys[slot] = sc;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+      const int64_t i = ((int64_t)j * 256 + threadIdx.x) * 4;
+      if (i < Iw) *(uint32_t*)(q + i) = pack4_e4m3(v[j].x / sc, v[j].y / sc, v[j].z / sc, v[j].w / sc);
+    }
+    return;
+  }
   float am = 0.f;
   for (int64_t i = threadIdx.x; i < I; i += blockDim.x) am = fmaxf(am, fabsf(y[i]));
   am = block_max(am, red);
   const float sc = fmaxf(am / 240.0f, 1e-05f);
   if (threadIdx.x == 0) ys[slot] = sc;
-  uint8_t* q = Yq + slot * Iw;
   for (int64_t i = (int64_t)threadIdx.x * 4; i < Iw; i += (int64_t)blockDim.x * 4) {
     float v[4];
 #pragma unroll
