@@ -113,13 +113,26 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
 
   const int lane = tid & 63, w = tid >> 6;
   const int c = lane & 15, g = lane >> 4;
-  const int m0 = w * 32;
+  // MXFP8: a wave owns 32 rows and every column tile.  bf16 / fp8-row: the four waves form a 2 x 2 grid, a wave
+  // owns 64 rows and half the column tiles (stage 1: four gate tiles and the matching four up tiles), which
+  // takes a third fewer fragment bytes out of LDS per MFMA than 32 rows x all columns.
+  constexpr bool GRID2 = (KIND != MOE_KIND_MXFP8);
+  constexpr int MT = GRID2 ? 4 : 2;
+  constexpr int NTW = GRID2 ? NT / 2 : NT;
+  const int m0 = GRID2 ? (w >> 1) * 64 : w * 32;
+  const int wn = GRID2 ? (w & 1) : 0;
+  // column tile (16 staged columns) behind accumulator index nt
+  auto ctile = [&](int nt) -> int {
+    if constexpr (!GRID2) return nt;
+    else if constexpr (STAGE == 1) return (nt < 4) ? wn * 4 + nt : 4 + wn * 4 + nt;
+    else return wn * 4 + nt;
+  };
 
-  v4f acc[NT][2];
+  v4f acc[NTW][MT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
+  for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) acc[nt][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   // ---- K loop ---------------------------------------------------------------------------
   int nks;
@@ -189,26 +202,26 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
       if constexpr (KIND == MOE_KIND_BF16) {
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
-          v8bf af[2];
+          v8bf af[MT];
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * LROW + sub * 64 + g * 16);
+          for (int mt = 0; mt < MT; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * LROW + sub * 64 + g * 16);
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            const v8bf bf = *(const v8bf*)(sB + (nt * 16 + c) * LROW + sub * 64 + g * 16);
+          for (int nt = 0; nt < NTW; ++nt) {
+            const v8bf bf = *(const v8bf*)(sB + (ctile(nt) * 16 + c) * LROW + sub * 64 + g * 16);
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+            for (int mt = 0; mt < MT; ++mt)
               acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bf, acc[nt][mt], 0, 0, 0);
           }
         }
       } else {
-        v8i af[2];
+        v8i af[MT];
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) af[mt] = lds_read_frag(sA + (m0 + 16 * mt + c) * LROW, g);
+        for (int mt = 0; mt < MT; ++mt) af[mt] = lds_read_frag(sA + (m0 + 16 * mt + c) * LROW, g);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const v8i bf = lds_read_frag(sB + (nt * 16 + c) * LROW, g);
+        for (int nt = 0; nt < NTW; ++nt) {
+          const v8i bf = lds_read_frag(sB + (ctile(nt) * 16 + c) * LROW, g);
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
+          for (int mt = 0; mt < MT; ++mt)
             acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, 127, 0, 127);
         }
       }
@@ -331,9 +344,9 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
 
   // ---- epilogue ----------------------------------------------------------------------------
   // accumulator element r of tile (nt, mt) is (row m0 + 16*mt + 4*g + r, column nt*16 + c)
-  if (STAGE == 1) {
+  if constexpr (STAGE == 1) {
     const bool pre = (a.scaling_mode == MOE_SCALE_PRE || a.scaling_mode == MOE_SCALE_PRE_DELAYED);
-    if (KIND == MOE_KIND_MXFP8) {
+    if constexpr (KIND == MOE_KIND_MXFP8) {
       uint8_t* Yq = (uint8_t*)a.out;
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
@@ -385,8 +398,8 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
       const float* wsc = (const float*)a.W_scale;
       const int64_t wsb = (a.w_scale_experts > 1) ? (int64_t)e * 2 * a.I : 0;
 #pragma unroll
-      for (int nt = 0; nt < 8; ++nt) {
-        const int64_t i = c0 + nt * 16 + c;
+      for (int nt = 0; nt < NTW / 2; ++nt) {  // gate tile nt of this wave, its up tile is accumulator nt + NTW / 2
+        const int64_t i = c0 + ctile(nt) * 16 + c;
         const bool iv = i < a.I;
         float sg = 1.f, su = 1.f, bg = 0.f, bu = 0.f;
         if (iv && wsc) { sg = wsc[wsb + i]; su = wsc[wsb + a.I + i]; }
@@ -395,11 +408,11 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
           bu = load_bias(a.bias, a.bias_dtype, ((int64_t)e * 2 + 1) * a.I + i);
         }
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
+        for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int row = m0 + 16 * mt + 4 * g + r;
-            float gv = acc[nt][mt][r], uv = acc[nt + 8][mt][r];
+            float gv = acc[nt][mt][r], uv = acc[nt + NTW / 2][mt][r];
             if (KIND == MOE_KIND_BF16) {
               if (pre) { gv *= s_aff[row]; uv *= s_aff[row]; }
               gv *= sg; uv *= su;
@@ -436,13 +449,13 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
     const int64_t wsb = (a.w_scale_experts > 1) ? (int64_t)e * a.H : 0;
     const bool post = a.scaling_mode == MOE_SCALE_POST;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int64_t h = c0 + nt * 16 + c;
+    for (int nt = 0; nt < NTW; ++nt) {
+      const int64_t h = c0 + ctile(nt) * 16 + c;
       if (h >= a.H) continue;
       const float sd = wsc ? wsc[wsb + h] : 1.f;
       const float bd = a.bias ? load_bias(a.bias, a.bias_dtype, (int64_t)e * a.H + h) : 0.f;
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
+      for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int row = m0 + 16 * mt + 4 * g + r;
