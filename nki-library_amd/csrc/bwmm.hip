@@ -52,13 +52,28 @@ __device__ __forceinline__ v8i lds_read_frag(const uint8_t* row, int g) {
 
 // (the bf16 and fp8-row kinds are held to 256 registers so that two workgroups share a CU and cover each other's
 // barriers: their 128 x 256 stage-1 tile alone needs 128 accumulator registers)
+// The same fragment from a 128-byte row whose 16-byte pieces are swizzled with sw = row & 7.
+__device__ __forceinline__ v8i lds_read_frag_swz(const uint8_t* row, int g, int sw) {
+  const v4i lo = *(const v4i*)(row + ((g ^ sw) * 16));
+  const v4i hi = *(const v4i*)(row + (((g + 4) ^ sw) * 16));
+  v8i r;
+  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+  return r;
+}
+
 template <int KIND, int STAGE>
 __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_KIND_MXFP8 ? 1 : 2, 8))) void bwmm_kernel(
     const GemmArgs a) {
   constexpr int NCOLS = (STAGE == 1) ? 256 : 128;
   constexpr int NT = NCOLS / 16;
-  __shared__ __attribute__((aligned(16))) uint8_t sA[TM * LROW];
-  __shared__ __attribute__((aligned(16))) uint8_t sB[NCOLS * LROW];
+  // bf16 / fp8-row: 128-byte rows whose 16-byte pieces are XOR-swizzled with the row's low three bits (piece j of
+  // row r sits at j ^ (r & 7)): the 16 lanes that a 16-byte LDS read serves in one pass (lanes 0-3, 12-15, 20-23,
+  // 24-27 of a wave, and so on) then touch 64 different banks, which rows padded to 144 bytes do not achieve
+  // (a third of the LDS cycles were bank conflicts).  MXFP8: padded rows, staged by 4-byte transposing stores.
+  constexpr int SROW = (KIND == MOE_KIND_MXFP8) ? LROW : 128;
+  __shared__ __attribute__((aligned(16))) uint8_t sA[TM * SROW];
+  __shared__ __attribute__((aligned(16))) uint8_t sB[NCOLS * SROW];
   __shared__ uint32_t sAs[TM];   // MX: the 4 E8M0 bytes of this k-step; FP8_ROW: fp32 row scale bits
   __shared__ uint32_t sBs[NCOLS];
   __shared__ int s_tok[TM];
@@ -191,11 +206,11 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
     fetch(0);
     for (int ks = 0; ks < nks; ++ks) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) *(uint4*)(sA + ((tid >> 3) + 32 * j) * LROW + (tid & 7) * 16) = ra[j];
+      for (int j = 0; j < 4; ++j) *(uint4*)(sA + ((tid >> 3) + 32 * j) * SROW + (((tid & 7) ^ ((tid >> 3) & 7)) * 16)) = ra[j];
 #pragma unroll
       for (int j = 0; j < PB; ++j) {
-        const int idx = tid + GT * j;
-        *(uint4*)(sB + (idx >> 3) * LROW + (idx & 7) * 16) = rb[j];
+        const int idx = tid + GT * j;  // row idx >> 3 has the low bits of tid >> 3 as well
+        *(uint4*)(sB + (idx >> 3) * SROW + (((tid & 7) ^ ((tid >> 3) & 7)) * 16)) = rb[j];
       }
       __syncthreads();
       if (ks + 1 < nks) fetch(ks + 1);
@@ -204,10 +219,10 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
         for (int sub = 0; sub < 2; ++sub) {
           v8bf af[MT];
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * LROW + sub * 64 + g * 16);
+          for (int mt = 0; mt < MT; ++mt) af[mt] = *(const v8bf*)(sA + (m0 + 16 * mt + c) * SROW + (((sub * 4 + g) ^ (c & 7)) * 16));
 #pragma unroll
           for (int nt = 0; nt < NTW; ++nt) {
-            const v8bf bf = *(const v8bf*)(sB + (ctile(nt) * 16 + c) * LROW + sub * 64 + g * 16);
+            const v8bf bf = *(const v8bf*)(sB + (ctile(nt) * 16 + c) * SROW + (((sub * 4 + g) ^ (c & 7)) * 16));
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bf, acc[nt][mt], 0, 0, 0);
@@ -216,10 +231,10 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
       } else {
         v8i af[MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) af[mt] = lds_read_frag(sA + (m0 + 16 * mt + c) * LROW, g);
+        for (int mt = 0; mt < MT; ++mt) af[mt] = lds_read_frag_swz(sA + (m0 + 16 * mt + c) * SROW, g, c & 7);
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
-          const v8i bf = lds_read_frag(sB + (ctile(nt) * 16 + c) * LROW, g);
+          const v8i bf = lds_read_frag_swz(sB + (ctile(nt) * 16 + c) * SROW, g, c & 7);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, 127, 0, 127);
