@@ -50,8 +50,9 @@ __device__ __forceinline__ v8i lds_read_frag(const uint8_t* row, int g) {
   return r;
 }
 
-// (the bf16 and fp8-row kinds are held to 256 registers so that two workgroups share a CU and cover each other's
-// barriers: their 128 x 256 stage-1 tile alone needs 128 accumulator registers)
+// (the bf16 and fp8-row kinds are held to 256 registers in stage 1 and 168 in stage 2 so that two / three workgroups
+// share a CU: each keeps the CU's loads flowing while the others wait at their barriers or run MFMAs; the
+// 128 x 256 stage-1 tile alone needs 128 accumulator registers)
 // The same fragment from a 128-byte row whose 16-byte pieces are swizzled with sw = row & 7.
 __device__ __forceinline__ v8i lds_read_frag_swz(const uint8_t* row, int g, int sw) {
   const v4i lo = *(const v4i*)(row + ((g ^ sw) * 16));
@@ -63,7 +64,7 @@ __device__ __forceinline__ v8i lds_read_frag_swz(const uint8_t* row, int g, int 
 }
 
 template <int KIND, int STAGE>
-__global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_KIND_MXFP8 ? 1 : 2, 8))) void bwmm_kernel(
+__global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_KIND_MXFP8 ? 1 : (STAGE == 2 ? 3 : 2), 8))) void bwmm_kernel(
     const GemmArgs a) {
   constexpr int NCOLS = (STAGE == 1) ? 256 : 128;
   constexpr int NT = NCOLS / 16;

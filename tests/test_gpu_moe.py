@@ -95,6 +95,11 @@ def test_c1_tiny_bf16():
         (256, 512, 256, 8, 2, 128, "shard_on_i", 1, 1, True, True, False),     # GELU, bias, skip_token
         (256, 512, 256, 4, 1, 128, "shard_on_block", 2, 1, False, False, False),  # top-1: non accumulating
         (200, 256, 128, 3, 2, 64, "shard_on_i", 0, 0, False, False, False),    # NO_SCALE, B < 128
+        # many rows per expert: the 256-row chunk tiles (a chunk of 300 rows = a full tile and a 44-row one; H and I
+        # that are no multiples of the column tiles)
+        (300, 512, 384, 2, 2, 128, "shard_on_block", 0, 1, True, False, False),
+        (640, 576, 520, 2, 2, 128, "shard_on_i", 3, 2, False, False, True),
+        (600, 512, 384, 2, 2, 128, "shard_on_block", 1, 1, True, True, False),
     ],
 )
 def test_dense_variants(T, H, I, E, k, B, impl, act, mode, bias, skip, clamp):
@@ -276,7 +281,8 @@ def _run_fp8_row(c, gamma):
     return rec, out
 
 
-@pytest.mark.parametrize("T,H,I,E,k,B", [(256, 512, 512, 4, 2, 128), (384, 1024, 896, 8, 2, 128)])
+@pytest.mark.parametrize("T,H,I,E,k,B", [(256, 512, 512, 4, 2, 128), (384, 1024, 896, 8, 2, 128),
+                                         (300, 512, 640, 2, 2, 128), (768, 1024, 896, 2, 2, 128)])  # 256-row chunk tiles
 def test_fp8_row_pipeline(T, H, I, E, k, B):
     """RMSNorm-Quant ROW -> fp8 x fp8 blockwise MoE with per-row / per-channel scales (BASELINE config 2 shape family)."""
     import torch
