@@ -42,7 +42,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-blocks", type=int, default=6, help="blocks of the workload timed on the CPU oracle")
+    ap.add_argument("--cpu-blocks", type=int, default=48, help="blocks of the workload timed on the CPU oracle (48: 10-20 s)")
     ap.add_argument("--with-router", action="store_true",
                     help="start from hidden states: time the router top-k front end (synthetic router weights) as a "
                          "stage of its own and route with its output; the headline metric stays the MoE layer")
