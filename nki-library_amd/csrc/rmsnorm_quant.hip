@@ -50,6 +50,32 @@ __device__ __forceinline__ void load8(const void* base, int dtype, int64_t i, in
   }
 }
 
+// The same for 8 elements known to lie inside the tensor at a 16-byte aligned address: no bounds checks, one branch
+// on the (uniform) dtype.
+__device__ __forceinline__ void load8_vec(const void* base, int dtype, int64_t i, float* v) {
+  if (dtype == MOE_DT_FP32) {
+    const float* p = (const float*)base + i;
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    return;
+  }
+  const uint4 a = *(const uint4*)((const uint16_t*)base + i);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+  if (dtype == MOE_DT_BF16) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = __uint_as_float(w[k] << 16);
+      v[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = fp16_bits_to_f32((uint16_t)(w[k] & 0xffffu));
+      v[2 * k + 1] = fp16_bits_to_f32((uint16_t)(w[k] >> 16));
+    }
+  }
+}
+
 // MODE 0: per-row scale appended to the row ([H+4] record).  MODE 1: static scale.
 template <int MODE>
 __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
@@ -70,7 +96,8 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
     if (j < nchunk) {
       const int64_t i = ((int64_t)j * RQ_THREADS + threadIdx.x) * 8;
       if (i < H) {
-        load8(xr, x_dtype, i, H, vec_ok, v[j]);
+        if (vec_ok) load8_vec(xr, x_dtype, i, v[j]);  // H % 8 == 0: the 8 elements lie inside the row
+        else load8(xr, x_dtype, i, H, false, v[j]);
       } else {
 #pragma unroll
         for (int k = 0; k < 8; ++k) v[j][k] = 0.f;
@@ -91,7 +118,8 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
         const int64_t i = ((int64_t)j * RQ_THREADS + threadIdx.x) * 8;
         if (i < H) {
           float g[8];
-          load8(gamma, gamma_dtype, i, H, vec_ok, g);
+          if (vec_ok) load8_vec(gamma, gamma_dtype, i, g);
+          else load8(gamma, gamma_dtype, i, H, false, g);
 #pragma unroll
           for (int k = 0; k < 8; ++k) v[j][k] = (v[j][k] * inv) * g[k];
         }
@@ -184,7 +212,7 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
       const int tile = blk >> 4, p8 = blk & 15;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        load8(xr, x_dtype, q * Hq + tile * 128 + p8 * 8, H, true, v[j][q]);
+        load8_vec(xr, x_dtype, q * Hq + tile * 128 + p8 * 8, v[j][q]);
 #pragma unroll
         for (int r = 0; r < 8; ++r) ss += (double)v[j][q][r] * (double)v[j][q][r];
       }
@@ -205,7 +233,7 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         float g[8];
-        if (do_norm) load8(gamma, gamma_dtype, q * Hq + tile * 128 + p8 * 8, H, true, g);
+        if (do_norm) load8_vec(gamma, gamma_dtype, q * Hq + tile * 128 + p8 * 8, g);
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
           float t = v[j][q][r];
