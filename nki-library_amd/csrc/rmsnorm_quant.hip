@@ -235,12 +235,16 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
         float g[8];
         if (do_norm) load8_vec(gamma, gamma_dtype, q * Hq + tile * 128 + p8 * 8, g);
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          float t = v[j][q][r];
-          if (do_norm) t = (t * inv) * g[r];
-          t = round_to_bf16(t);
-          v[j][q][r] = t;
-          am = fmaxf(am, fabsf(t));
+        for (int r = 0; r < 8; r += 2) {
+          float t0 = v[j][q][r], t1 = v[j][q][r + 1];
+          if (do_norm) {
+            t0 = (t0 * inv) * g[r];
+            t1 = (t1 * inv) * g[r + 1];
+          }
+          round2_to_bf16(t0, t1);
+          v[j][q][r] = t0;
+          v[j][q][r + 1] = t1;
+          am = fmaxf(am, fmaxf(fabsf(t0), fabsf(t1)));
         }
       }
       if (out_norm != nullptr) {
