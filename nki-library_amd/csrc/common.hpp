@@ -34,15 +34,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
-// Two values rounded to bf16 (round to nearest even) and widened again, with the hardware's packed conversion.
-__device__ __forceinline__ void round2_to_bf16(float& a, float& b) {
+// Two values rounded to bf16 (round to nearest even) with the hardware's packed conversion: a in the low half.
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
   typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
   typedef float v2f_t __attribute__((ext_vector_type(2)));
   const v2bf_t h = __builtin_convertvector((v2f_t){a, b}, v2bf_t);
-  const uint32_t u = __builtin_bit_cast(uint32_t, h);
-  a = __uint_as_float(u << 16);
-  b = __uint_as_float(u & 0xffff0000u);
+  return __builtin_bit_cast(uint32_t, h);
 }
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
 __device__ __forceinline__ float fp16_bits_to_f32(uint16_t b) {
   _Float16 h;

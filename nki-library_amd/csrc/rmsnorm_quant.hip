@@ -188,22 +188,39 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
 // contiguous elements at h = q*(H/4) + tile*128 + p8*8 + r.
 constexpr int MXQ_MAX_BLK = RQ_MAX_H / 32 / RQ_THREADS;  // 2
 
-// MAXB = MX blocks per thread (1 for H <= 32 * RQ_THREADS: half the registers, twice the rows in flight per CU:
-// a row is one load round trip, one reduction and one store, so rows in flight are what fills the memory pipeline).
-template <int MAXB>
-__global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? 5 : 3, 8))) void rmsnorm_quant_mx_kernel(
+// Eight 16-bit elements (bf16 or fp16) as loaded, widened.
+__device__ __forceinline__ void unpack8(const uint4& a, int dtype, float* v) {
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (dtype == MOE_DT_BF16) {
+      v[2 * k] = bf16_lo(w[k]);
+      v[2 * k + 1] = bf16_hi(w[k]);
+    } else {
+      v[2 * k] = fp16_bits_to_f32((uint16_t)(w[k] & 0xffffu));
+      v[2 * k + 1] = fp16_bits_to_f32((uint16_t)(w[k] >> 16));
+    }
+  }
+}
+
+// MAXB = MX blocks per thread (1 for H <= 32 * RQ_THREADS).  A row is one load round trip, one reduction and one
+// store, so the rows in flight per CU are what fills the memory pipeline, and registers decide how many those are:
+// 16-bit inputs (X16) stay packed as loaded (16 registers per MX block instead of 32) and the normalised values,
+// which are bf16 by definition, are kept as bf16 pairs.
+template <int MAXB, bool X16>
+__global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? (X16 ? 6 : 5) : 3, 8))) void rmsnorm_quant_mx_kernel(
     const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
     uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, uint16_t* __restrict__ out_norm, int64_t rows,
     int64_t H, float eps, float hidden_actual, int do_norm, int layout) {
   __shared__ double redd[16];
   const int64_t row = blockIdx.x;
-  const int es = (x_dtype == MOE_DT_FP32) ? 4 : 2;
+  const int es = X16 ? 2 : 4;
   const void* xr = (const uint8_t*)x + row * H * es;
   const int nblk = (int)(H / 32);
   const int nT = (int)(H / 512);
   const int64_t Hq = H / 4;
 
-  float v[MAXB][4][8];
+  uint4 raw[MAXB][X16 ? 4 : 8];  // the thread's inputs as loaded: [block][q] (fp32: [block][2 q + half])
   double ss = 0.0;
 #pragma unroll
   for (int j = 0; j < MAXB; ++j) {
@@ -212,9 +229,18 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
       const int tile = blk >> 4, p8 = blk & 15;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        load8_vec(xr, x_dtype, q * Hq + tile * 128 + p8 * 8, v[j][q]);
+        const int64_t i = q * Hq + tile * 128 + p8 * 8;
+        float t[8];
+        if constexpr (X16) {
+          raw[j][q] = *(const uint4*)((const uint16_t*)xr + i);
+          unpack8(raw[j][q], x_dtype, t);
+        } else {
+          raw[j][2 * q] = *(const uint4*)((const float*)xr + i);
+          raw[j][2 * q + 1] = *(const uint4*)((const float*)xr + i + 4);
+          __builtin_memcpy(t, &raw[j][2 * q], 32);
+        }
 #pragma unroll
-        for (int r = 0; r < 8; ++r) ss += (double)v[j][q][r] * (double)v[j][q][r];
+        for (int r = 0; r < 8; ++r) ss += (double)t[r] * (double)t[r];
       }
     }
   }
@@ -230,21 +256,23 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
     if (blk < nblk) {
       const int tile = blk >> 4, p8 = blk & 15;
       float am = 0.f;
+      uint32_t nv[4][4];  // normalised values, rounded to bf16: [q][pair of r]
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        float g[8];
+        float t[8], g[8];
+        if constexpr (X16) unpack8(raw[j][q], x_dtype, t);
+        else __builtin_memcpy(t, &raw[j][2 * q], 32);
         if (do_norm) load8_vec(gamma, gamma_dtype, q * Hq + tile * 128 + p8 * 8, g);
 #pragma unroll
         for (int r = 0; r < 8; r += 2) {
-          float t0 = v[j][q][r], t1 = v[j][q][r + 1];
+          float t0 = t[r], t1 = t[r + 1];
           if (do_norm) {
             t0 = (t0 * inv) * g[r];
             t1 = (t1 * inv) * g[r + 1];
           }
-          round2_to_bf16(t0, t1);
-          v[j][q][r] = t0;
-          v[j][q][r + 1] = t1;
-          am = fmaxf(am, fmaxf(fabsf(t0), fabsf(t1)));
+          const uint32_t u = pack2_bf16(t0, t1);
+          nv[q][r >> 1] = u;
+          am = fmaxf(am, fmaxf(fabsf(bf16_lo(u)), fabsf(bf16_hi(u))));
         }
       }
       if (out_norm != nullptr) {
@@ -253,16 +281,19 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
 #pragma unroll
           for (int r = 0; r < 8; ++r) {
             const int64_t p = p8 * 8 + r, h1 = (int64_t)q * nT + tile;
-            out_norm[(p * rows + row) * (H / 128) + h1] = f32_to_bf16_bits(v[j][q][r]);
+            out_norm[(p * rows + row) * (H / 128) + h1] = (uint16_t)((r & 1) ? (nv[q][r >> 1] >> 16) : (nv[q][r >> 1] & 0xffffu));
           }
       }
       const uint32_t sb = mx_scale_byte(am);
       const float is = mx_inv_scale(sb);
       uint32_t d[8];
 #pragma unroll
-      for (int r = 0; r < 8; ++r)
-        d[r] = pack4_e4m3(clip448(v[j][0][r] * is), clip448(v[j][1][r] * is), clip448(v[j][2][r] * is),
-                          clip448(v[j][3][r] * is));
+      for (int r = 0; r < 8; ++r) {
+        float e[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) e[q] = ((r & 1) ? bf16_hi(nv[q][r >> 1]) : bf16_lo(nv[q][r >> 1])) * is;
+        d[r] = pack4_e4m3(clip448(e[0]), clip448(e[1]), clip448(e[2]), clip448(e[3]));
+      }
       if (layout == MOE_MX_LAYOUT_TOKEN_MAJOR) {
         uint4* o = (uint4*)(out_q + row * H + (int64_t)blk * 32);
         o[0] = make_uint4(d[0], d[1], d[2], d[3]);
@@ -327,14 +358,19 @@ extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* g
     return MOE_E_BAD_ARG;
   if (rows == 0) return MOE_OK;
   const float ha = (float)(hidden_actual > 0 ? hidden_actual : H);
-  if (H <= 32 * RQ_THREADS)
-    hipLaunchKernelGGL(rmsnorm_quant_mx_kernel<1>, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
-                       x_dtype, gamma, gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H,
-                       eps, ha, do_norm, layout);
-  else
-    hipLaunchKernelGGL(rmsnorm_quant_mx_kernel<MXQ_MAX_BLK>, dim3((unsigned)rows), dim3(RQ_THREADS), 0,
-                       (hipStream_t)stream, x, x_dtype, gamma, gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale,
-                       (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout);
+  const bool x16 = x_dtype != MOE_DT_FP32;
+  const dim3 grid((unsigned)rows), block(RQ_THREADS);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, x, x_dtype, gamma, gamma_dtype, (uint8_t*)out_q,
+                       (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout);
+  };
+  if (H <= 32 * RQ_THREADS) {
+    if (x16) launch(rmsnorm_quant_mx_kernel<1, true>);
+    else launch(rmsnorm_quant_mx_kernel<1, false>);
+  } else {
+    if (x16) launch(rmsnorm_quant_mx_kernel<MXQ_MAX_BLK, true>);
+    else launch(rmsnorm_quant_mx_kernel<MXQ_MAX_BLK, false>);
+  }
   MOE_CHECK_LAUNCH();
   return MOE_OK;
 }
