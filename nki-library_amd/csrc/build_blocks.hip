@@ -19,6 +19,8 @@ namespace moe {
 constexpr int BB_THREADS = 256;
 
 constexpr int BB_SLABS_MAX = 64;
+constexpr int64_t BB_SINGLE_MAX_TOKENS = 1024;  // up to this many tokens form one slab, built by a single launch
+constexpr int64_t BB_SINGLE_MAX_SLOTS = 1 << 17;  // one workgroup fills the pad ids of up to this many slots itself
 constexpr int BB_E_MAX = 1024;  // bitmaps and running counts of all experts in LDS: 36 bytes per expert
 
 // The bitmaps of 256 tokens: bit (tid & 31) of word bm[(tid >> 5) * E + e] says that token t0 + tid selected
@@ -56,15 +58,15 @@ __device__ __forceinline__ int bb_bits(const uint32_t* bm, int64_t E, int64_t e)
 // Workgroup = slab of slab_tokens tokens (a multiple of 256).  slab_counts[slab][e] = tokens of the slab that
 // selected e.  All workgroups together also fill token_position_to_id with the pad id, which the scatter
 // overwrites where tokens sit.
-__global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
-                                                             int64_t E, int64_t slab_tokens,
-                                                             int32_t* __restrict__ slab_counts,
-                                                             int32_t* __restrict__ tp2id, int64_t NB, int pad_id) {
-  extern __shared__ uint32_t bb_lds[];
+// (slab = this workgroup's slab, n_wg = workgroups that share the pad fill; bb_lds = 9 E words of LDS)
+__device__ __forceinline__ void bb_count_body(const int32_t* __restrict__ ids, int64_t T, int64_t k, int64_t E,
+                                              int64_t slab_tokens, int32_t* __restrict__ slab_counts,
+                                              int32_t* __restrict__ tp2id, int64_t NB, int pad_id, int64_t slab,
+                                              int64_t n_wg, uint32_t* bb_lds) {
   uint32_t* bm = bb_lds;            // [8][E]
   int* run = (int*)(bb_lds + 8 * E);  // [E]
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) run[e] = 0;
-  const int64_t t_begin = (int64_t)blockIdx.x * slab_tokens;
+  const int64_t t_begin = slab * slab_tokens;
   for (int64_t sub = 0; sub < slab_tokens && t_begin + sub < T; sub += BB_THREADS) {
     for (int64_t i = threadIdx.x; i < 8 * E; i += BB_THREADS) bm[i] = 0;
     __syncthreads();
@@ -75,22 +77,28 @@ __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __r
     for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) run[e] += bb_bits(bm, E, e);
     __syncthreads();
   }
-  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) slab_counts[(int64_t)blockIdx.x * E + e] = run[e];
-  for (int64_t i = (int64_t)blockIdx.x * BB_THREADS + threadIdx.x; i < NB; i += (int64_t)gridDim.x * BB_THREADS)
-    tp2id[i] = pad_id;
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) slab_counts[slab * E + e] = run[e];
+  for (int64_t i = slab * BB_THREADS + threadIdx.x; i < NB; i += n_wg * BB_THREADS) tp2id[i] = pad_id;
+}
+
+__global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
+                                                             int64_t E, int64_t slab_tokens,
+                                                             int32_t* __restrict__ slab_counts,
+                                                             int32_t* __restrict__ tp2id, int64_t NB, int pad_id) {
+  extern __shared__ uint32_t bb_lds[];
+  bb_count_body(ids, T, k, E, slab_tokens, slab_counts, tp2id, NB, pad_id, blockIdx.x, gridDim.x, bb_lds);
 }
 
 // ws layout: first_slot[E] | slab_counts[BB_SLABS_MAX][E]
 // One workgroup: blocks per expert (padding blocks to the last expert, or split), exclusive scan ->
 // first slot of every expert, block_to_expert, conditions; sums and scans over the experts are
 // workgroup-wide (shuffles + one exchange), a tile of BB_THREADS experts at a time.
-__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
-                                                              int32_t* __restrict__ first_slot,
-                                                              int32_t* __restrict__ block_to_expert,
-                                                              int32_t* __restrict__ conditions, int64_t n_conditions,
-                                                              int64_t E, int64_t B, int64_t N, int use_split_padding,
-                                                              int32_t* __restrict__ status) {
-  extern __shared__ int s_nb[];  // [E] blocks per expert, then [E] first block of every expert
+__device__ __forceinline__ void bb_layout_body(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
+                                               int32_t* __restrict__ first_slot, int32_t* __restrict__ block_to_expert,
+                                               int32_t* __restrict__ conditions, int64_t n_conditions, int64_t E,
+                                               int64_t B, int64_t N, int use_split_padding,
+                                               int32_t* __restrict__ status, int* s_nb) {
+  // s_nb: [E] blocks per expert, then [E] first block of every expert
   int* s_first = s_nb + E;
   __shared__ int s_npad;
   __shared__ int s_ws[16];
@@ -143,23 +151,32 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __
   }
 }
 
+__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
+                                                              int32_t* __restrict__ first_slot,
+                                                              int32_t* __restrict__ block_to_expert,
+                                                              int32_t* __restrict__ conditions, int64_t n_conditions,
+                                                              int64_t E, int64_t B, int64_t N, int use_split_padding,
+                                                              int32_t* __restrict__ status) {
+  extern __shared__ int s_nb_dyn[];
+  bb_layout_body(slab_counts, n_slabs, first_slot, block_to_expert, conditions, n_conditions, E, B, N,
+                 use_split_padding, status, s_nb_dyn);
+}
+
 // Workgroup = slab.  A token's slot for expert e: first slot of e + tokens of e in the slabs before (summed here
 // from the slab counts) + tokens of e earlier in this slab.
-__global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
-                                                               int64_t E, int64_t slab_tokens,
-                                                               const int32_t* __restrict__ slab_counts,
-                                                               const int32_t* __restrict__ first_slot,
-                                                               int32_t* __restrict__ tp2id, int64_t NB) {
-  extern __shared__ uint32_t bb_lds[];
+__device__ __forceinline__ void bb_scatter_body(const int32_t* __restrict__ ids, int64_t T, int64_t k, int64_t E,
+                                                int64_t slab_tokens, const int32_t* __restrict__ slab_counts,
+                                                const int32_t* __restrict__ first_slot, int32_t* __restrict__ tp2id,
+                                                int64_t NB, int64_t slab, uint32_t* bb_lds) {
   uint32_t* bm = bb_lds;
   int* run = (int*)(bb_lds + 8 * E);
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
     int before = first_slot[e];
 #pragma unroll 8
-    for (int64_t sl = 0; sl < blockIdx.x; ++sl) before += slab_counts[sl * E + e];
+    for (int64_t sl = 0; sl < slab; ++sl) before += slab_counts[sl * E + e];
     run[e] = before;
   }
-  const int64_t t_begin = (int64_t)blockIdx.x * slab_tokens;
+  const int64_t t_begin = slab * slab_tokens;
   const int wd = threadIdx.x >> 5;
   const uint32_t below = (1u << (threadIdx.x & 31)) - 1u;
   for (int64_t sub = 0; sub < slab_tokens && t_begin + sub < T; sub += BB_THREADS) {
@@ -187,6 +204,32 @@ __global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* _
   }
 }
 
+__global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
+                                                               int64_t E, int64_t slab_tokens,
+                                                               const int32_t* __restrict__ slab_counts,
+                                                               const int32_t* __restrict__ first_slot,
+                                                               int32_t* __restrict__ tp2id, int64_t NB) {
+  extern __shared__ uint32_t bb_lds[];
+  bb_scatter_body(ids, T, k, E, slab_tokens, slab_counts, first_slot, tp2id, NB, blockIdx.x, bb_lds);
+}
+
+// Few tokens (one slab): the three steps in one launch by one workgroup.  What one step leaves in global memory
+// (the slab's counts, the first slots, the pad ids under the tokens' slots) the next reads or overwrites after a
+// workgroup barrier: all of it goes through this CU's L1.
+__global__ __launch_bounds__(BB_THREADS) void bb_single_slab_kernel(
+    const int32_t* __restrict__ ids, int64_t T, int64_t k, int64_t E, int64_t slab_tokens,
+    int32_t* __restrict__ slab_counts, int32_t* __restrict__ first_slot, int32_t* __restrict__ tp2id, int64_t NB,
+    int pad_id, int32_t* __restrict__ block_to_expert, int32_t* __restrict__ conditions, int64_t n_conditions, int64_t B,
+    int64_t N, int use_split_padding, int32_t* __restrict__ status) {
+  extern __shared__ uint32_t bb_lds[];  // 9 E words of the count / scatter steps, then 2 E of the layout step
+  bb_count_body(ids, T, k, E, slab_tokens, slab_counts, tp2id, NB, pad_id, 0, 1, bb_lds);
+  __syncthreads();
+  bb_layout_body(slab_counts, 1, first_slot, block_to_expert, conditions, n_conditions, E, B, N, use_split_padding,
+                 status, (int*)(bb_lds + 9 * E));
+  __syncthreads();
+  bb_scatter_body(ids, T, k, E, slab_tokens, slab_counts, first_slot, tp2id, NB, 0, bb_lds);
+}
+
 }  // namespace moe
 
 using namespace moe;
@@ -208,12 +251,22 @@ extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, i
   int64_t slab_tokens = (T + BB_SLABS_MAX - 1) / BB_SLABS_MAX;
   slab_tokens = (slab_tokens + BB_THREADS - 1) / BB_THREADS * BB_THREADS;
   if (slab_tokens == 0) slab_tokens = BB_THREADS;
+  if (T <= BB_SINGLE_MAX_TOKENS) slab_tokens = (T + BB_THREADS - 1) / BB_THREADS * BB_THREADS;  // one slab
+  if (slab_tokens == 0) slab_tokens = BB_THREADS;
   int64_t n_slabs = (T + slab_tokens - 1) / slab_tokens;
   if (n_slabs == 0) n_slabs = 1;  // T == 0: one slab with no tokens still fills the pad ids
   int32_t* first_slot = (int32_t*)workspace;
   int32_t* slab_counts = first_slot + E;
   const size_t lds = (size_t)9 * E * sizeof(int32_t);
   hipStream_t s = (hipStream_t)stream;
+  if (n_slabs == 1 && N * B <= BB_SINGLE_MAX_SLOTS) {
+    hipLaunchKernelGGL(bb_single_slab_kernel, dim3(1), dim3(BB_THREADS), lds + 2 * E * sizeof(int32_t), s, topk_ids, T,
+                       k, E, slab_tokens, slab_counts, first_slot, token_position_to_id, N * B,
+                       skip_token ? -1 : (int)T, block_to_expert, conditions, n_conditions, B, N, use_split_padding,
+                       status_out);
+    MOE_CHECK_LAUNCH();
+    return MOE_OK;
+  }
   hipLaunchKernelGGL(bb_count_kernel, dim3((unsigned)n_slabs), dim3(BB_THREADS), lds, s, topk_ids, T, k, E, slab_tokens,
                      slab_counts, token_position_to_id, N * B, skip_token ? -1 : (int)T);
   MOE_CHECK_LAUNCH();
