@@ -38,14 +38,14 @@ def build_token_blocks(topk_ids: torch.Tensor, E: int, B: int, N: int = None, sk
     if n_conditions is None:
         n_conditions = N + 1
     dev = ids.device
-    tp2id = torch.empty(N * B, dtype=torch.int32, device=dev)
-    b2e = torch.empty(N, dtype=torch.int32, device=dev)
-    cond = torch.empty(n_conditions, dtype=torch.int32, device=dev)
-    status = torch.zeros(1, dtype=torch.int32, device=dev)
-    ws = torch.empty(L.moe_build_blocks_workspace_bytes(E), dtype=torch.uint8, device=dev)
+    # one allocation for the three outputs, the status word (always written by the layout step) and the int32
+    # workspace: at decode sizes the host side of this call costs more than its kernels
+    ws_words = (L.moe_build_blocks_workspace_bytes(E) + 3) // 4
+    buf = torch.empty(N * B + N + n_conditions + 1 + ws_words, dtype=torch.int32, device=dev)
+    tp2id, b2e, cond, status, ws = torch.split(buf, [N * B, N, n_conditions, 1, ws_words])
     with torch.cuda.device(dev):
         rc = L.moe_build_blocks(nv.ptr(ids), T, k, E, B, N, 1 if skip_token else 0, 1 if use_split_padding else 0,
-                                nv.ptr(tp2id), nv.ptr(b2e), nv.ptr(cond), n_conditions, nv.ptr(ws), ws.numel(),
+                                nv.ptr(tp2id), nv.ptr(b2e), nv.ptr(cond), n_conditions, nv.ptr(ws), ws.numel() * 4,
                                 nv.ptr(status), nv.stream_ptr(dev))
     nv.check(rc, "build_token_blocks")
     if check:
