@@ -113,6 +113,20 @@ __device__ __forceinline__ double block_sum_f64(double v, double* red) {
   for (int i = 0; i < nw; ++i) t += red[i];
   return t;
 }
+// The same over groups of `group` consecutive threads (64, 128 or 256 of a 256-thread workgroup): every thread gets
+// the sum of its group.
+__device__ __forceinline__ double group_sum_f64(double v, double* red, int group) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  const int w = threadIdx.x >> 6, gw = group >> 6;  // gw is 1, 2 or 4
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  const int w0 = w & ~(gw - 1);
+  double t = 0.0;
+  for (int i = 0; i < gw; ++i) t += red[w0 + i];
+  return t;
+}
 __device__ __forceinline__ float block_max(float v, float* red) {
   v = wave_max(v);
   const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;

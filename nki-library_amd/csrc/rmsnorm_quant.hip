@@ -211,12 +211,17 @@ template <int MAXB, bool X16>
 __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? (X16 ? 6 : 5) : 3, 8))) void rmsnorm_quant_mx_kernel(
     const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
     uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, uint16_t* __restrict__ out_norm, int64_t rows,
-    int64_t H, float eps, float hidden_actual, int do_norm, int layout) {
+    int64_t H, float eps, float hidden_actual, int do_norm, int layout, int tpr) {
   __shared__ double redd[16];
-  const int64_t row = blockIdx.x;
+  // tpr = threads per row (64, 128 or 256): short rows share a workgroup, RQ_THREADS / tpr of them
+  const int tpr_lg = (tpr == 64) ? 6 : ((tpr == 128) ? 7 : 8);
+  const int lt = threadIdx.x & (tpr - 1);
+  const int64_t row_raw = ((int64_t)blockIdx.x << (8 - tpr_lg)) + (threadIdx.x >> tpr_lg);
+  const bool row_ok = row_raw < rows;
+  const int64_t row = row_ok ? row_raw : rows - 1;
   const int es = X16 ? 2 : 4;
   const void* xr = (const uint8_t*)x + row * H * es;
-  const int nblk = (int)(H / 32);
+  const int nblk = row_ok ? (int)(H / 32) : 0;  // threads of a row past the end own no block
   const int nT = (int)(H / 512);
   const int64_t Hq = H / 4;
 
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
   double ss = 0.0;
 #pragma unroll
   for (int j = 0; j < MAXB; ++j) {
-    const int blk = j * RQ_THREADS + threadIdx.x;
+    const int blk = j * tpr + lt;
     if (blk < nblk) {
       const int tile = blk >> 4, p8 = blk & 15;
 #pragma unroll
@@ -246,13 +251,13 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
   }
   float inv = 1.0f;
   if (do_norm) {
-    const float total = (float)block_sum_f64(ss, redd);
+    const float total = (float)group_sum_f64(ss, redd, tpr);
     const float rms = sqrtf(total / hidden_actual + eps);
     inv = 1.0f / rms;
   }
 #pragma unroll
   for (int j = 0; j < MAXB; ++j) {
-    const int blk = j * RQ_THREADS + threadIdx.x;
+    const int blk = j * tpr + lt;
     if (blk < nblk) {
       const int tile = blk >> 4, p8 = blk & 15;
       float am = 0.f;
@@ -359,10 +364,13 @@ extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* g
   if (rows == 0) return MOE_OK;
   const float ha = (float)(hidden_actual > 0 ? hidden_actual : H);
   const bool x16 = x_dtype != MOE_DT_FP32;
-  const dim3 grid((unsigned)rows), block(RQ_THREADS);
+  const int nblk = (int)(H / 32);
+  const int tpr = nblk <= 64 ? 64 : (nblk <= 128 ? 128 : RQ_THREADS);
+  const int rpw = RQ_THREADS / tpr;  // rows per workgroup
+  const dim3 grid((unsigned)((rows + rpw - 1) / rpw)), block(RQ_THREADS);
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, x, x_dtype, gamma, gamma_dtype, (uint8_t*)out_q,
-                       (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout);
+                       (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout, tpr);
   };
   if (H <= 32 * RQ_THREADS) {
     if (x16) launch(rmsnorm_quant_mx_kernel<1, true>);
