@@ -134,7 +134,10 @@ def test_zero_row_follows_kernel_rule():
 
 
 @pytest.mark.parametrize("T,H,do_norm", [(4, 512, True), (64, 2048, True), (33, 7168, True), (16, 16384, True),
-                                          (40, 1024, False)])
+                                          (40, 1024, False),
+                                          # short rows share a workgroup (four of up to 64 MX blocks, two of up to
+                                          # 128): row counts that leave the last workgroup partly empty
+                                          (5, 1536, True), (7, 4096, True), (3, 3072, True)])
 def test_mx_front_end(T, H, do_norm):
     """RMSNorm -> MXFP8 (token-major and the reference's [128, H/512, T] layouts) vs the oracle."""
     import torch
