@@ -111,3 +111,16 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(nv, "LIB_PATH", str(tmp_path / "absent.so"))
     with pytest.raises(nv.NativeLibraryError, match="no CPU fallback"):
         nv.lib()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: --gpus N with N > 1 exits with a message that says so (before touching a GPU)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in res.stderr and res.stdout.strip() == ""
