@@ -163,22 +163,40 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
     const int64_t kbytes = (KIND == MOE_KIND_BF16) ? a.K * 2 : a.K;
     constexpr int PB = NCOLS * 8 / GT;
     uint4 ra[4], rb[PB];
+    // What a thread stages does not change over the K loop: 16-byte piece tid & 7 of rows / columns (tid >> 3) + 32 j.
+    // The addresses are worked out once: the A rows as 32-bit offsets (in units of 4 bytes) from a.A, the weight
+    // rows as one pointer plus offsets that are the same for the whole workgroup.
+    const int pc = tid & 7, rl = tid >> 3;
+    uint32_t ao[4];  // ~0: no such row
+    unsigned b_ok = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = rl + 32 * j;
+      int64_t off = -1;
+      if (STAGE == 1) {
+        const int tok = s_tok[row];
+        if (tok >= 0) off = (int64_t)tok * a.a_stride;
+      } else {
+        if (r0 + row < vr) off = (slot0 + row) * a.a_stride;
+      }
+      ao[j] = (off >= 0) ? (uint32_t)((off + pc * 16) >> 2) : ~0u;
+    }
+    const uint8_t* wb;
+    if (STAGE == 1) wb = a.W + (((int64_t)e * 2) * a.I + c0 + rl) * a.Kp + pc * 16;
+    else wb = a.W + ((int64_t)e * a.H + c0 + rl) * a.Kp + pc * 16;
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+      const int64_t cj = c0 + rl + 32 * (STAGE == 1 ? (j & 3) : j);  // stage 1: j < 4 gate columns, j >= 4 up columns
+      if (cj < (STAGE == 1 ? a.I : a.H)) b_ok |= 1u << j;
+    }
     auto fetch = [&](int ks) {
       const int64_t a_off = (int64_t)ks * 128;
-      const int a_valid = (int)((kbytes - a_off < 128) ? (kbytes - a_off) : 128);
+      const bool a_in = pc * 16 + 16 <= kbytes - a_off;  // A rows end at K; the weight rows are zero padded to Kp
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int row = (tid >> 3) + 32 * j, ch = tid & 7;
         uint4 val = make_uint4(0, 0, 0, 0);
-        const uint8_t* src = nullptr;
-        if (STAGE == 1) {
-          const int tok = s_tok[row];
-          if (tok >= 0) src = a.A + (int64_t)tok * a.a_stride;
-        } else {
-          if (r0 + row < vr) src = a.A + (slot0 + row) * a.a_stride;
-        }
-        if (src != nullptr && ch * 16 + 16 <= a_valid) {
-          src += a_off + ch * 16;
+        if (ao[j] != ~0u && a_in) {
+          const uint8_t* src = a.A + ((int64_t)ao[j] << 2) + a_off;
           if (KIND == MOE_KIND_FP8_ROW && STAGE == 1) {  // rows of H + 4 bytes are only 4-byte aligned
             const uint32_t* s4 = (const uint32_t*)src;
             val = make_uint4(s4[0], s4[1], s4[2], s4[3]);
@@ -190,17 +208,9 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
       }
 #pragma unroll
       for (int j = 0; j < PB; ++j) {
-        const int idx = tid + GT * j;
-        const int col = idx >> 3, ch = idx & 7;
+        const int64_t wj = (STAGE == 1) ? ((int64_t)(j >> 2) * a.I + 32 * (j & 3)) * a.Kp : (int64_t)(32 * j) * a.Kp;
         uint4 val = make_uint4(0, 0, 0, 0);
-        if (STAGE == 1) {
-          const int gu = col >> 7;
-          const int64_t i = c0 + (col & 127);
-          if (i < a.I) val = *(const uint4*)(a.W + (((int64_t)e * 2 + gu) * a.I + i) * a.Kp + a_off + ch * 16);
-        } else {
-          const int64_t h = c0 + col;
-          if (h < a.H) val = *(const uint4*)(a.W + ((int64_t)e * a.H + h) * a.Kp + a_off + ch * 16);
-        }
+        if ((b_ok >> j) & 1u) val = *(const uint4*)(wb + wj + a_off);
         rb[j] = val;
       }
     };
