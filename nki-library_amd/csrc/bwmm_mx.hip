@@ -42,9 +42,6 @@
 
 #include "bwmm.hpp"
 
-#ifndef MX_DBG_WAIT0
-#define MX_DBG_WAIT0 0
-#endif
 namespace moe {
 
 constexpr int MXT = 256;                       // threads
@@ -220,7 +217,11 @@ __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, 
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen nt" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
-// 16 bytes per lane straight into LDS at lds + 16 * lane (no destination registers).
+// 16 bytes per lane straight into LDS at lds + 16 * lane (no destination registers).  The instruction takes its
+// LDS base from M0, which is set in the same statement.  M0 is declared clobbered: the compiler warns that it
+// does not save reserved registers around a statement, which is what is wanted here -- on this target it never
+// carries a value in M0 from one instruction to the next (it writes M0 itself immediately before each instruction
+// of its own that reads it), so there is nothing to save.
 __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
@@ -520,7 +521,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
     asm volatile("" ::: "memory");
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + (D - 2) * N1) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NLB + (D - 2) * N1) : "memory");
     if constexpr (U == D - 1) {  // activation scales of slices ks+1 .. ks+D
       asm volatile("" : "+v"(asr));
       if constexpr (BIG) asm volatile("" : "+v"(asr2));
@@ -605,7 +606,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     const SliceAddr sa = slice_addr(u, u);
     static_for<0, N0>([&](auto i_) { issue_load(i_, sa, br[u], asr, asr2, std::integral_constant<bool, u == 0>{}); });
   });
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(MX_DBG_WAIT0 ? 0 : NLB + (D - 1) * N1) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NLB + (D - 1) * N1) : "memory");
   asm volatile("" : "+v"(asr));
   if constexpr (BIG) asm volatile("" : "+v"(asr2));
 #pragma unroll

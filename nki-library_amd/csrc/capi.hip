@@ -95,6 +95,28 @@ int validate(const moe_bwmm_args* a) {
       break;
     }
   }
+  // Address ranges.  The kernels form per-lane offsets in 32 bits; a shape whose tensors outgrow what those
+  // offsets reach would read wrong rows without any error, so it is refused here (the reference states its
+  // own size limits the same way, bwmm_shard_on_block_mx.py:586-633).
+  const int64_t slots = a->N * a->B;
+  if (a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I)) {
+    // large-tile kernels: byte offsets (row * row stride, added to a 64-bit base) and buffer descriptors of at most
+    // 2^32 - 1 bytes for the activations, the intermediate and their scales; signed 32-bit byte offsets inside one
+    // expert's weights
+    const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
+    const int64_t Iw = (a->I + 511) / 512 * 512;
+    const int64_t es = a->weight_dtype == MOE_DT_FP4_E2M1 ? 2 : 4;  // bytes of an x4 weight element
+    const int64_t pI = a->I > 512 ? 128 : a->I / 4, nI = (a->I + 511) / 512;
+    if (a->T1 * a->H >= lim32 || slots * Iw >= lim32) return MOE_E_BAD_SHAPE;
+    if (128 * 2 * (a->H / 512) * a->I * es >= lim31 || pI * nI * a->H * es >= lim31) return MOE_E_BAD_SHAPE;
+  } else if (a->kind != MOE_KIND_MXFP8) {
+    // general tiled kernel, dense kinds: row offsets are kept in units of 4 bytes in 32 bits (the value ~0 is
+    // reserved for "no such row"), i.e. each A operand must stay below 2^34 - 4 bytes = 16 GiB
+    const int64_t lim34 = ((int64_t)1 << 34) - 4;
+    const int64_t a1 = a->kind == MOE_KIND_BF16 ? a->H * 2 : a->H + 4;
+    const int64_t a2 = a->kind == MOE_KIND_BF16 ? (a->I + 63) / 64 * 64 * 2 : (a->I + 127) / 128 * 128;
+    if (a->T1 * a1 >= lim34 || slots * a2 >= lim34) return MOE_E_BAD_SHAPE;
+  }
   return MOE_OK;
 }
 

@@ -161,6 +161,16 @@ def moe_blockwise_ref(
     return out
 
 
+def fp8_row_requant(y):
+    """Per-row re-quantisation of the intermediate of the fp8-row pipeline (perform_row_quant without clipping,
+    test/integration/nkilib/core/mlp/test_mlp_common.py:978-986, applied at :1114-1116):
+    ``scale = max(amax / 240, 1e-5)``, codes = e4m3(y / scale).  Returns (uint8 codes, fp32 scale [rows, 1])."""
+    y = np.asarray(y, dtype=np.float32)
+    amax = np.abs(y).max(axis=-1, keepdims=True)
+    ys = np.maximum(amax / np.float32(NEURON_E4M3_MAX), np.float32(1e-05)).astype(np.float32)
+    return e4m3fn_encode(y / ys), ys
+
+
 def moe_blockwise_fp8_row_ref(
     hidden_q,
     hidden_row_scale,
@@ -218,9 +228,8 @@ def moe_blockwise_fp8_row_ref(
             g += np.asarray(gate_up_proj_bias, dtype=np.float32)[e, 0, :]
             u += np.asarray(gate_up_proj_bias, dtype=np.float32)[e, 1, :]
         y = (act_fn(g, activation_function) * u).astype(np.float32)
-        amax = np.abs(y).max(axis=-1, keepdims=True)
-        ys = np.maximum(amax / np.float32(NEURON_E4M3_MAX), np.float32(1e-05)).astype(np.float32)
-        yq = e4m3fn_decode(e4m3fn_encode(y / ys))
+        yc, ys = fp8_row_requant(y)
+        yq = e4m3fn_decode(yc)
         wd = e4m3fn_decode(down_w_q[e])[:I]
         sd = np.asarray(down_w_scale, dtype=np.float32)[e].reshape(-1)
         d = (np.matmul(yq, wd) * sd) * ys
@@ -434,6 +443,67 @@ def moe_mx_token_ref(x_row, e_list, aff_row, gate_up_proj_weight, gate_up_proj_s
         yk = quantize_vec32(y[i_of_kk])
         wd = mx_dequant_down(down_proj_weight[e], down_proj_scale[e]).astype(np.float64)
         total += float(to_bf16(np.asarray([aff_row[e]], dtype=np.float32))[0]) * (yk.astype(np.float64) @ wd)
+    return total
+
+
+def mx_expert_mlp_rows(x_rows, gate_up_proj_weight_e, gate_up_proj_scale_e, down_proj_weight_e, down_proj_scale_e,
+                       activation_function=ACT_SILU):
+    """Rows ``x_rows`` [n, H] (bf16-valued) through ONE expert's MXFP8 (e4m3) MLP; fp64 rows [n, H], no affinity.
+
+    The same index formulas as ``moe_mx_token_ref`` with each block's E8M0 weight scale taken out of the block's
+    sum -- ``sum_k x_k w_k 2^s = 2^s sum_k x_k w_k`` over the 32 k of a block -- so the expert's weights are
+    decoded once for all rows and never scaled element by element (what makes the full-size experts of
+    BASELINE configs 4 / 5 affordable on a CPU).  Products are exact in fp32; a block's 32-term sum is taken in
+    fp32 (relative error below 2^-19 of its largest term), the sums over blocks in fp64.  I % 512 == 0.
+    Pinned against ``moe_mx_token_ref`` in tests/test_oracle_moe.py.
+    """
+    x_rows = np.asarray(x_rows, dtype=np.float32)
+    n, H = x_rows.shape
+    nH = H // 512
+    I = gate_up_proj_weight_e.shape[3]
+    assert I % 512 == 0 and gate_up_proj_weight_e.shape == (128, 2, nH, I, 4)
+    nI = I // 512
+    kp = np.arange(H)
+    tile, p, q = kp // 512, (kp % 512) // 4, kp % 4
+    xk = np.stack([quantize_vec32(r[q * (H // 4) + tile * 128 + p]) for r in x_rows])          # [n, K']
+    xk = xk.reshape(n, nH, 16, 8, 4)                                                             # [n, t, pb, p8, q]
+    w = e4m3fn_decode(gate_up_proj_weight_e).reshape(16, 8, 2, nH, I, 4)                          # [pb, p8, g, t, i, q]
+    part = np.einsum("bpgtiq,ntbpq->nbgti", w, xk)                                               # fp32 block sums
+    sc = np.power(2.0, gate_up_proj_scale_e.astype(np.float64) - 127.0)                          # [pb, g, t, i]
+    gu = np.einsum("nbgti,bgti->ngi", part.astype(np.float64), sc)
+    g, u = gu[:, 0].astype(np.float32), gu[:, 1].astype(np.float32)
+    y = (act_fn(g, activation_function) * u).astype(np.float32)                                  # [n, I]
+    kk = np.arange(I)
+    ti, pi, qi = kk // 512, (kk % 512) // 4, kk % 4
+    yk = np.stack([quantize_vec32(r[ti * 512 + qi * 128 + pi]) for r in y]).reshape(n, nI, 16, 8, 4)
+    wd = e4m3fn_decode(down_proj_weight_e).reshape(16, 8, nI, H, 4)                               # [pb, p8, t, h, q]
+    partd = np.einsum("bpthq,ntbpq->nbth", wd, yk)
+    scd = np.power(2.0, down_proj_scale_e.astype(np.float64) - 127.0)                            # [pb, t, h]
+    return np.einsum("nbth,bth->nh", partd.astype(np.float64), scd)
+
+
+def moe_mx_tokens_ref(x_rows, experts_per_row, aff_per_row, expert_weights, activation_function=ACT_SILU, map_fn=map):
+    """Several tokens through their experts, grouped by expert so that each expert is decoded once.
+
+    x_rows [n, H]; experts_per_row: n lists of expert ids; aff_per_row: n lists of (bf16-valued) affinities in
+    the same order; ``expert_weights(e)`` returns that expert's (gate_up_q, gate_up_s, down_q, down_s).
+    Returns fp64 [n, H] = sum over a row's experts of aff * MLP_e(x) (``mx_expert_mlp_rows``).  ``map_fn`` may
+    be a thread pool's ``map`` (numpy releases the interpreter lock inside the einsums).
+    """
+    x_rows = np.asarray(x_rows, dtype=np.float32)
+    users = {}
+    for r, es in enumerate(experts_per_row):
+        for j, e in enumerate(es):
+            users.setdefault(int(e), []).append((r, j))
+
+    def one(e):
+        rows = [r for r, _ in users[e]]
+        return e, mx_expert_mlp_rows(x_rows[rows], *expert_weights(e), activation_function=activation_function)
+
+    total = np.zeros(x_rows.shape, dtype=np.float64)
+    for e, out in map_fn(one, sorted(users)):
+        for (r, j), o in zip(users[e], out):
+            total[r] += float(to_bf16(np.asarray([aff_per_row[r][j]], dtype=np.float32))[0]) * o
     return total
 
 

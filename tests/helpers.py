@@ -90,8 +90,49 @@ def mx_weights(rng, E, H, I, std=0.02, fmt="e4m3"):
     return gu_q, gu_s, d_q, d_s
 
 
+def _random_codes(rng, shape, fmt):
+    """Uniformly random element codes of an MX format without the NaN / infinity patterns."""
+    if fmt == "e2m1":
+        return rng.integers(0, 16, size=shape, dtype=np.uint8)
+    b = rng.integers(0, 256, size=shape, dtype=np.uint8)
+    if fmt == "e4m3":
+        b[(b & 0x7F) == 0x7F] &= 0xFE           # 0x7f / 0xff are NaN
+    else:
+        b[(b & 0x7C) == 0x7C] &= 0xFB           # e5m2: exponent 31 is infinity / NaN
+    return b
+
+
+def mx_weights_random_codes(rng, E, H, I, fmt="e4m3", gate_rms=3.0):
+    """Expert weights drawn directly in the quantised domain, the way the reference's generator does it
+    (generate_stabilized_mx_data, test/integration/nkilib/utils/tensor_generators.py:351-418: random element
+    codes, random E8M0 scales over a window of 11 exponents below an upper bound).  The upper bound is chosen so
+    that a projection of unit-variance inputs has a root mean square of about ``gate_rms``.  Fast enough for the
+    reference's own table shapes (no floating-point quantisation pass over hundreds of millions of elements)."""
+    from oracle.numerics import e2m1_decode, e5m2_decode
+
+    nH, nI = H // 512, math.ceil(I / 512)
+    pI = 128 if I > 512 else I // 4
+    pI8 = math.ceil(pI / 8) * 8
+    table = {"e4m3": e4m3fn_decode, "e5m2": e5m2_decode, "e2m1": e2m1_decode}[fmt]
+    vals = table(np.arange(16 if fmt == "e2m1" else 256, dtype=np.uint8)).astype(np.float64)
+    rms_code = float(np.sqrt(np.mean(vals[np.isfinite(vals)] ** 2)))
+
+    def scales(shape, K):
+        hi = int(round(127 + math.log2(gate_rms / (rms_code * 0.348 * math.sqrt(K)))))
+        return rng.integers(hi - 10, hi + 1, size=shape, dtype=np.uint8)
+
+    gu_q = _random_codes(rng, (E, 128, 2, nH, I, 4), fmt)
+    gu_s = scales((E, 16, 2, nH, I), H)
+    d_q = _random_codes(rng, (E, pI, nI, H, 4), fmt)
+    d_s = scales((E, pI8 // 8, nI, H), I)
+    tail = I % 512
+    if tail and I > 512:
+        d_q[:, tail // 4:, nI - 1] = 0
+    return gu_q, gu_s, d_q, d_s
+
+
 def mx_case(T, H, I, E, k, B, seed=0, skip_token=False, bias=False, alpha=None, hidden_std=1.0, weight_std=0.05,
-            dynamic=False, weight_format="e4m3"):
+            dynamic=False, weight_format="e4m3", random_codes=False):
     rng = np.random.default_rng(seed)
     N, mask, tp2id, b2e, cond = routing(T, k, E, B, skip_token, alpha, n_block_per_iter=2, is_block_parallel=True,
                                         is_mx=True)
@@ -99,7 +140,10 @@ def mx_case(T, H, I, E, k, B, seed=0, skip_token=False, bias=False, alpha=None, 
     hs = to_bf16((rng.standard_normal((T1, H)) * hidden_std).astype(np.float32))
     if not skip_token:
         hs[T] = 0
-    gu_q, gu_s, d_q, d_s = mx_weights(rng, E, H, I, weight_std, weight_format)
+    if random_codes:
+        gu_q, gu_s, d_q, d_s = mx_weights_random_codes(rng, E, H, I, weight_format)
+    else:
+        gu_q, gu_s, d_q, d_s = mx_weights(rng, E, H, I, weight_std, weight_format)
     c = {"T": T, "T1": T1, "H": H, "I": I, "E": E, "k": k, "B": B, "N": N, "skip_token": skip_token,
          "hidden": hs, "aff": affinities(rng, T, E, mask, skip_token), "tp2id": tp2id, "b2e": b2e,
          "cond": cond if dynamic else None, "mask": mask, "weight_format": weight_format,

@@ -69,3 +69,52 @@ def test_argument_validation_runs_without_a_gpu():
     assert L.moe_build_blocks_workspace_bytes(256) >= 2 * 256 * 4
     with pytest.raises(AssertionError, match="NCC_INKI016"):
         nv.check(-2, "x")
+
+
+def _valid_args(nv, kind, T1, H, I, E, B, N, weight_dtype=0):
+    """An argument block that passes validation (pointers are never dereferenced by it)."""
+    a = nv.BwmmArgs()
+    fake = ctypes.c_void_p(4096)
+    for f in ("hidden_states", "expert_affinities_masked", "gate_up_proj_weight", "down_proj_weight",
+              "gate_up_proj_scale", "down_proj_scale", "token_position_to_id", "block_to_expert", "output"):
+        setattr(a, f, fake)
+    a.T1, a.H, a.I, a.E, a.B, a.N = T1, H, I, E, B, N
+    a.out_row_stride = H
+    a.scale_experts = E
+    a.kind = kind
+    a.weight_dtype = weight_dtype
+    a.scaling_mode = 1
+    return a
+
+
+def test_shapes_beyond_the_32_bit_offsets_are_refused():
+    """The kernels address rows with 32-bit offsets: tensors that outgrow them must be refused, not wrapped around
+    (the reference states explicit limits too, bwmm_shard_on_block_mx.py:586-633)."""
+    from nkilib import _native as nv
+
+    L = nv.lib()
+    ws = lambda a: L.moe_blockwise_workspace_bytes(ctypes.byref(a))
+    rc = lambda a: L.moe_blockwise(ctypes.byref(a), None)
+    BAD_SHAPE, WORKSPACE = -2, -3
+    # MXFP8, DeepSeek-V3 experts: BASELINE config 4 passes
+    ok = _valid_args(nv, nv.KIND_MXFP8, 8193, 7168, 2048, 256, 128, 766, nv.DT_FP8)
+    assert ws(ok) > 0 and rc(ok) == WORKSPACE
+    # hidden states of 2^32 bytes: (T+1) * H
+    big_t = _valid_args(nv, nv.KIND_MXFP8, 2**32 // 7168 + 1, 7168, 2048, 256, 128, 766, nv.DT_FP8)
+    assert ws(big_t) == 0 and rc(big_t) == BAD_SHAPE
+    just_below = _valid_args(nv, nv.KIND_MXFP8, 2**32 // 7168, 7168, 2048, 256, 128, 766, nv.DT_FP8)
+    assert ws(just_below) > 0
+    # intermediate of 2^32 bytes: N * B * I (about 262k tokens top-8 at I = 2048)
+    big_n = _valid_args(nv, nv.KIND_MXFP8, 8193, 7168, 2048, 256, 128, 2**32 // (128 * 2048), nv.DT_FP8)
+    assert ws(big_n) == 0 and rc(big_n) == BAD_SHAPE
+    # one expert's gate/up weights of 2 GiB: 2 * H * I bytes
+    big_w = _valid_args(nv, nv.KIND_MXFP8, 129, 16384, 65536, 2, 128, 2, nv.DT_FP8)
+    assert ws(big_w) == 0 and rc(big_w) == BAD_SHAPE
+    # ... which 4-bit weights (half the bytes) still fit
+    assert ws(_valid_args(nv, nv.KIND_MXFP8, 129, 16384, 65536, 2, 128, 2, nv.DT_FP4_E2M1)) > 0
+    # dense kinds: 16 GiB per A operand
+    assert ws(_valid_args(nv, nv.KIND_BF16, 4097, 4096, 14336, 8, 128, 71)) > 0
+    big_bf16 = _valid_args(nv, nv.KIND_BF16, 2**34 // (4096 * 2), 4096, 1024, 8, 128, 71)
+    assert ws(big_bf16) == 0 and rc(big_bf16) == BAD_SHAPE
+    big_row = _valid_args(nv, nv.KIND_FP8_ROW, 4097, 4096, 14336, 8, 128, 2**34 // (128 * 14336) + 1)
+    assert ws(big_row) == 0 and rc(big_row) == BAD_SHAPE

@@ -411,6 +411,128 @@ def test_mx_fp4_weights(T, H, I, E, k, B, bias, wd):
     _check(o[0, :T], g[:T], f"mx fp4 H={H} I={I} E={E}")
 
 
+def _run_mx_options(c, act, clamps, uint_containers, prequant=False):
+    """bwmm_shard_on_block_mx with every option of the reference's MX table: activation, clamps, bias, conditions,
+    skip_token, and the weights either in typed containers (1-byte float8 elements with a trailing axis of 4, or
+    2-byte elements for MXFP4: the format is read off the tensor) or in the uint32 / uint16 containers of
+    convert_mx_weights_to_uint_dtype (test_moe_bwmm_mx_cte.py:113-133) with the format in ``weight_dtype``."""
+    import torch
+    from nkilib.core.moe.moe_cte import SkipMode
+    from nkilib.core.moe.moe_cte.bwmm_shard_on_block_mx import bwmm_shard_on_block_mx
+    from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize
+    from nkilib.core.utils.common_types import ActFnType
+
+    dev = torch.device("cuda:0")
+    fmt = c["weight_format"]
+    kw = dict(clamps or {})
+    if "gate_up_bias" in c:
+        kw["gate_and_up_proj_bias"] = bf16_tensor(c["gate_up_bias"], dev)
+        kw["down_proj_bias"] = bf16_tensor(c["down_bias"], dev)
+    if c["cond"] is not None:
+        kw["conditions"] = i32_tensor(c["cond"], dev)
+    if fmt == "e2m1":
+        from oracle.numerics import pack_e2m1_x4
+        gu = torch.from_numpy(pack_e2m1_x4(c["gate_up_q"]).view(np.int16)).to(dev)
+        dw = torch.from_numpy(pack_e2m1_x4(c["down_q"]).view(np.int16)).to(dev)
+        if uint_containers:
+            gu, dw = gu.view(torch.uint16), dw.view(torch.uint16)
+            kw["weight_dtype"] = "float4_e2m1fn_x4"
+    elif uint_containers:
+        gu = torch.from_numpy(c["gate_up_q"].view(np.uint32).reshape(c["gate_up_q"].shape[:-1])).to(dev)
+        dw = torch.from_numpy(c["down_q"].view(np.uint32).reshape(c["down_q"].shape[:-1])).to(dev)
+        kw["weight_dtype"] = "float8_e5m2_x4" if fmt == "e5m2" else "float8_e4m3fn_x4"
+    else:
+        tdt = torch.float8_e5m2 if fmt == "e5m2" else torch.float8_e4m3fn
+        gu, dw = u8_tensor(c["gate_up_q"], dev).view(tdt), u8_tensor(c["down_q"], dev).view(tdt)
+    hs = bf16_tensor(c["hidden"], dev)
+    if prequant:
+        hs, kw["hidden_states_scale"] = rmsnorm_mx_quantize(hs, None, do_norm=False)
+    out = bwmm_shard_on_block_mx[2](
+        hs, bf16_tensor(c["aff"].reshape(-1, 1), dev), gu, dw, i32_tensor(c["tp2id"], dev),
+        i32_tensor(c["b2e"], dev), gate_up_proj_scale=u8_tensor(c["gate_up_s"], dev),
+        down_proj_scale=u8_tensor(c["down_s"], dev), block_size=c["B"], activation_function=ActFnType(act),
+        skip_dma=SkipMode(c["skip_token"], False), **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+def _golden_mx_options(c, act, clamps):
+    cl = clamps or {}
+    return omoe.moe_blockwise_mx_ref(
+        c["hidden"], c["aff"], c["gate_up_q"], c["down_q"], c["gate_up_s"], c["down_s"], c["tp2id"], c["b2e"], c["B"],
+        conditions=c["cond"], gate_up_proj_bias=c.get("gate_up_bias"), down_proj_bias=c.get("down_bias"),
+        activation_function=act, skip_token=c["skip_token"], weight_format=c["weight_format"],
+        gate_clamp_upper_limit=cl.get("gate_clamp_upper_limit"), gate_clamp_lower_limit=cl.get("gate_clamp_lower_limit"),
+        up_clamp_upper_limit=cl.get("up_clamp_upper_limit"), up_clamp_lower_limit=cl.get("up_clamp_lower_limit"))
+
+
+# The reference's own clamp set for every row of its MX tables (test_moe_bwmm_mx_cte.py:59-106).
+REF_MX_CLAMPS = dict(gate_clamp_upper_limit=7.0, up_clamp_upper_limit=7.0, up_clamp_lower_limit=-7.0)
+
+
+@pytest.mark.parametrize(
+    "H,T,I,E,B,k,act,fmt,skip,dynamic,uint",
+    [
+        # a covering selection of moe_bwmm_mx_cte_unit_perms (test_moe_bwmm_mx_cte.py:59-86) at the table's own small
+        # token count: H=3072, (I, E) in {(384, 128), (1536, 32)}, top-4 (top-2 in the uint-container rows), B in
+        # {256, 512}, Swish, bias, skip_token 0/1, static / dynamic conditions, MXFP4 / e4m3 / e5m2 weights
+        (3072, 1024, 384, 128, 256, 4, 3, "e2m1", True, False, False),
+        (3072, 1024, 384, 128, 512, 4, 3, "e4m3", False, True, False),
+        (3072, 1024, 384, 128, 256, 2, 3, "e5m2", True, False, True),
+        (3072, 1024, 1536, 32, 256, 4, 3, "e2m1", False, True, True),
+        (3072, 1024, 1536, 32, 512, 4, 3, "e4m3", True, False, True),
+        (3072, 1024, 1536, 32, 512, 4, 3, "e5m2", False, False, False),
+        (3072, 1024, 384, 128, 512, 4, 3, "e2m1", True, True, False),
+        (3072, 1024, 384, 128, 256, 4, 3, "e4m3", True, False, False),
+        (3072, 1024, 1536, 32, 256, 4, 3, "e5m2", True, True, False),
+        # the n_static_blocks rows (:83-85): few experts, so every expert holds several 256-row chunks
+        (4096, 1024, 1536, 2, 256, 2, 0, "e4m3", True, True, False),
+        (4096, 1024, 1024, 4, 256, 4, 0, "e4m3", True, True, False),
+        (3072, 1024, 384, 2, 256, 2, 0, "e4m3", True, True, False),
+    ],
+)
+def test_mx_reference_table(H, T, I, E, B, k, act, fmt, skip, dynamic, uint):
+    """The large-tile MX kernels on the reference's own shard-on-block MX configurations: clamps 7 / +-7, bias, Swish
+    (SiLU in the n_static_blocks rows), B = 256 / 512."""
+    c = mx_case(T, H, I, E, k, B, seed=21, skip_token=skip, bias=True, dynamic=dynamic, weight_format=fmt,
+                random_codes=True)
+    out = _run_mx_options(c, act, REF_MX_CLAMPS, uint)
+    o = from_bf16_tensor(out)
+    assert o.shape[0] == 2 and not o[1].any()
+    g = _golden_mx_options(c, act, REF_MX_CLAMPS)
+    rows = T  # row T (the padding token, absent with skip_token) stays zero here; the golden scatters the bias to it
+    if not skip:
+        assert not o[0, T].any()
+    _check(o[0, :rows], g[:rows], f"mx table H={H} I={I} E={E} B={B} {fmt}")
+
+
+@pytest.mark.parametrize("I", [512, 96, 544])  # large-tile kernels; general tiled kernel (I % 128 != 0), with a tail tile
+@pytest.mark.parametrize(
+    "act,clamps",
+    [
+        (0, None), (1, None), (2, None), (3, None),
+        (3, dict(gate_clamp_upper_limit=0.6)),
+        (3, dict(gate_clamp_lower_limit=-0.4)),
+        (3, dict(up_clamp_upper_limit=0.5)),
+        (3, dict(up_clamp_lower_limit=-0.3)),
+        (1, dict(gate_clamp_upper_limit=0.6, gate_clamp_lower_limit=-0.4, up_clamp_upper_limit=0.5, up_clamp_lower_limit=-0.3)),
+    ],
+)
+def test_mx_activation_and_clamp_options(I, act, clamps):
+    """Every ActFnType and every clamp limit on its own (limits small enough to cut a large share of the values)
+    through both MX code paths, with bias."""
+    T, H, E, k, B = 256, 512, 8, 2, 128
+    c = mx_case(T, H, I, E, k, B, seed=31, bias=True, weight_std=0.05)
+    out = _run_mx_options(c, act, clamps, uint_containers=False, prequant=(act == 2))
+    o = from_bf16_tensor(out)
+    g = _golden_mx_options(c, act, clamps)
+    assert not o[0, T].any()
+    _check(o[0, :T], g[:T], f"mx I={I} act={act} clamps={sorted((clamps or {}).keys())}")
+    if clamps and len(clamps) == 1:
+        # the limit must matter: without it the result is measurably different
+        assert max_abs_rel(_golden_mx_options(c, act, None)[:T], g[:T]) > 2 * RTOL
+
+
 def test_mx_prequantised_equals_online():
     """Quantise-then-gather == gather-then-quantise: MX blocks never span tokens, so both entry forms agree bit-wise."""
     c = mx_case(256, 1024, 512, 8, 2, 128, seed=8)

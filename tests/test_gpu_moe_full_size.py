@@ -46,18 +46,65 @@ def _bf16_np(tensor):
     return bf16_from_bits(tensor.contiguous().view(torch.int16).cpu().numpy().view(np.uint16))
 
 
+_C4 = {}
+
+
+def _c4_experts():
+    """BASELINE config 4's expert weights (11 GB on the GPU), generated once for the tests of this module."""
+    import torch
+    from nkilib import synthetic as syn
+
+    if not _C4:
+        dev = torch.device("cuda:0")
+        cfg = dict(syn.CONFIGS["c4"])
+        gu_q, gu_s, d_q, d_s = syn.mx_expert_weights(cfg["E"], cfg["H"], cfg["I"], 0.02, dev, seed=0)
+        _C4.update(cfg=cfg, t=dict(gu_q=gu_q, gu_s=gu_s, d_q=d_q, d_s=d_s,
+                                   gamma=torch.ones((1, cfg["H"]), dtype=torch.bfloat16, device=dev)))
+    return _C4["cfg"], _C4["t"]
+
+
+def _check_tokens_against_oracle(t, x, ids, aff, out_rows, toks, what):
+    """Rows `toks` of the layer's output against the grouped per-expert oracle (each expert decoded once for all
+    the tokens that use it, experts spread over a thread pool)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    import torch
+
+    H = x.shape[1]
+    sel = torch.tensor(list(toks), device=x.device)
+    x_np = _bf16_np(x[sel])
+    aff_np = _bf16_np(aff[sel])
+    ids_np = ids[sel].cpu().numpy()
+    out_rows = out_rows[sel]
+    experts = [sorted(int(e) for e in row) for row in ids_np]
+    affs = [[aff_np[i, e] for e in es] for i, es in enumerate(experts)]
+    normed = orn.to_bf16(orn.rms_norm(x_np, np.ones((1, H), np.float32)))
+
+    def weights(e):
+        return tuple(t[n][e].cpu().numpy() for n in ("gu_q", "gu_s", "d_q", "d_s"))
+
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        want = omoe.moe_mx_tokens_ref(normed, experts, affs, weights, map_fn=pool.map)
+    o = _bf16_np(out_rows)
+    worst = 0.0
+    for i, tok in enumerate(toks):
+        err = max_abs_rel(o[i], want[i])
+        worst = max(worst, err)
+        assert max_all_close(o[i], want[i].astype(np.float32), rtol=RTOL, atol=ATOL), \
+            f"{what} token {tok} (experts {experts[i]}): max-abs-rel {err:.3e}"
+    n_exp = len({e for es in experts for e in es})
+    print(f"{what}: {len(toks)} tokens over {n_exp} experts, worst max-abs-rel {worst:.3e} (rtol {RTOL})", flush=True)
+
+
 def test_c4_sampled_tokens_and_invariants():
     import torch
     from nkilib import synthetic as syn
 
     dev = torch.device("cuda:0")
-    cfg = dict(syn.CONFIGS["c4"])
+    cfg, t = _c4_experts()
     T, H, I, E, k = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["k"]
-    gu_q, gu_s, d_q, d_s = syn.mx_expert_weights(E, H, I, 0.02, dev, seed=0)
     ids, aff = syn.route(T, E, k, dev, seed=0, mode="sigmoid")
     x = syn.hidden_states(T, H, dev, seed=0)
-    t = dict(gu_q=gu_q, gu_s=gu_s, d_q=d_q, d_s=d_s, gamma=torch.ones((1, H), dtype=torch.bfloat16, device=dev))
-
     out = _layer(t, cfg, ids, aff, x)
     assert out.shape[0] == 2 and not bool(out[1].any()), "second output plane must stay zero"
     assert not bool(out[0, T].any()), "padding row must stay zero"
@@ -77,23 +124,49 @@ def test_c4_sampled_tokens_and_invariants():
     outp = _layer(t, cfg, ids[perm].contiguous(), affp, xp)
     assert torch.equal(outp[0, :T], out[0, :T][perm]), "token permutation changed some output row"
 
-    # sampled tokens against the per-token oracle
-    x_np = _bf16_np(x)
-    aff_np = _bf16_np(aff)
+    # Tokens against the oracle, chosen by construction: the first and the last token (in slot order) of
+    #   expert 0, expert 255 (the last; its gate/up weights start 6.97 GiB into the tensor), an expert just past the
+    #   4 GiB mark of the gate/up weights, an expert with more than 256 rows (one 320-row chunk: the last token sits in
+    #   the row tiles that accumulate outside the accumulation registers) and one with at most 256 rows.
     ids_np = ids.cpu().numpy()
-    o = _bf16_np(out[0])
-    for tok in (0, 4097):
-        experts = sorted(int(e) for e in ids_np[tok])
-        sel = torch.tensor(experts, device=dev)
-        remap = list(range(len(experts)))
-        normed = orn.to_bf16(orn.rms_norm(x_np[tok:tok + 1], np.ones((1, H), np.float32)))[0]
-        aff_row = aff_np[tok, experts]
-        want = omoe.moe_mx_token_ref(normed, remap, aff_row, gu_q[sel].view(torch.uint8).cpu().numpy(),
-                                     gu_s[sel].cpu().numpy(), d_q[sel].view(torch.uint8).cpu().numpy(),
-                                     d_s[sel].cpu().numpy())
-        err = max_abs_rel(o[tok], want)
-        print(f"c4 token {tok}: experts {experts} max-abs-rel {err:.3e} (rtol {RTOL})", flush=True)
-        assert max_all_close(o[tok], want.astype(np.float32), rtol=RTOL, atol=ATOL), f"token {tok}: {err:.3e}"
+    counts = np.bincount(ids_np.reshape(-1), minlength=E)
+    per_expert_bytes = 128 * 2 * (H // 512) * I * 4
+    e_4g = int(np.ceil(2**32 / per_expert_bytes))
+    e_big = int(np.flatnonzero((counts > 256) & (counts <= 320))[0])
+    e_small = int(np.flatnonzero((counts > 128) & (counts <= 256))[0])
+    targets = [0, E - 1, e_4g, e_big, e_small]
+    toks = []
+    for e in targets:
+        users = np.flatnonzero((ids_np == e).any(axis=1))  # ascending token id == slot order within the expert
+        toks += [int(users[0]), int(users[-1])]
+    toks = sorted(set(toks))
+    assert len(toks) >= 8
+    print(f"c4 targets: experts {targets} (rows {[int(counts[e]) for e in targets]}), tokens {toks}", flush=True)
+    _check_tokens_against_oracle(t, x, ids, aff, out[0], toks, "c4")
+
+
+@pytest.mark.parametrize("T", [1, 8, 32, 128])
+def test_c5_decode_shaped(T):
+    """BASELINE config 5: T in {1, 8, 32, 128} tokens on config 4's experts, uniform random top-8 (most experts
+    hold one partially filled block: the smallest row-tile variant, streamed weights, single-slab block build).
+    Every token for T <= 8, 8 tokens for T >= 32, against the per-expert oracle; padding row zero; reruns bit-equal."""
+    import torch
+    from nkilib import synthetic as syn
+
+    dev = torch.device("cuda:0")
+    cfg4, t = _c4_experts()
+    cfg = dict(cfg4, T=T)
+    H, E, k = cfg["H"], cfg["E"], cfg["k"]
+    ids, aff = syn.route(T, E, k, dev, seed=50 + T, uniform_random=True)
+    x = syn.hidden_states(T, H, dev, seed=50 + T)
+    out = _layer(t, cfg, ids, aff, x)
+    assert tuple(out.shape) == (2, T + 1, H)
+    assert not bool(out[1].any()), "second output plane must stay zero"
+    assert not bool(out[0, T].any()), "padding row must stay zero"
+    assert bool(out[0, :T].any(dim=1).all()), "every token must receive a contribution"
+    assert torch.equal(out, _layer(t, cfg, ids, aff, x)), "two runs of the same layer differ"
+    toks = list(range(T)) if T <= 8 else [int(v) for v in np.linspace(0, T - 1, 8).round()]
+    _check_tokens_against_oracle(t, x, ids, aff, out[0], toks, f"c5 T={T}")
 
 
 def _subset_problem(ids, aff, x, keep, experts=None):

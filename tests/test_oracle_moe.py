@@ -12,7 +12,7 @@ from helpers import dense_case, mx_case
 from oracle import moe as omoe
 from oracle import rmsnorm as orn
 from oracle.compare import fp8_codes_match_except_ties, max_abs_rel, max_all_close
-from oracle.numerics import bf16_bits, e4m3fn_decode, to_bf16
+from oracle.numerics import bf16_bits, e4m3fn_decode, e4m3fn_encode, to_bf16
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
 
@@ -109,6 +109,72 @@ def test_mx_block_golden_equals_independent_token_formulation():
         want = omoe.moe_mx_token_ref(c["hidden"][t], es, c["aff"][t], c["gate_up_q"], c["gate_up_s"], c["down_q"],
                                      c["down_s"])
         assert max_abs_rel(out[t], want) < 2.0**-7
+
+
+def test_grouped_expert_formulation_equals_token_formulation():
+    """mx_expert_mlp_rows / moe_mx_tokens_ref (block scales taken out of the block sums, experts decoded once
+    for all their rows) against moe_mx_token_ref (every weight scaled, fp64 throughout)."""
+    c = mx_case(64, 1024, 1024, 6, 3, 64, seed=9)
+    toks = [0, 5, 17, 40, 63]
+    es = [list(np.nonzero(c["mask"][t])[0]) for t in toks]
+    got = omoe.moe_mx_tokens_ref(c["hidden"][toks], es, [c["aff"][t][e] for t, e in zip(toks, es)],
+                                 lambda e: (c["gate_up_q"][e], c["gate_up_s"][e], c["down_q"][e], c["down_s"][e]))
+    for i, t in enumerate(toks):
+        want = omoe.moe_mx_token_ref(c["hidden"][t], es[i], c["aff"][t], c["gate_up_q"], c["gate_up_s"], c["down_q"],
+                                     c["down_s"])
+        # the two differ only by fp32 vs fp64 sums inside a 32-element block, except where that moves an
+        # intermediate value across an e4m3 rounding boundary of the re-quantisation (one step of one element)
+        assert max_abs_rel(got[i], want) < 2e-3, (t, max_abs_rel(got[i], want))
+    # one expert, activation other than SiLU
+    one = omoe.mx_expert_mlp_rows(c["hidden"][:2], c["gate_up_q"][1], c["gate_up_s"][1], c["down_q"][1], c["down_s"][1],
+                                  activation_function=omoe.ACT_SWISH)
+    ref = omoe.moe_mx_token_ref(c["hidden"][1], [1], np.ones(6, np.float32), c["gate_up_q"], c["gate_up_s"], c["down_q"],
+                                c["down_s"], activation_function=omoe.ACT_SWISH)
+    assert max_abs_rel(one[1], ref) < 2e-3
+
+
+def test_fp8_row_requant_known_answers():
+    """Known answers for the fp8-row intermediate re-quantisation (test_mlp_common.py:978-986,1114-1116):
+    the range is Neuron's 240, not OCP's 448, and the scale is floored at 1e-5."""
+    for s in (2.0**-6, 1.0, 2.0**5):
+        y = np.array([[240.0 * s, 9.0 * s, -120.0 * s, 0.0]], np.float32)
+        codes, scale = omoe.fp8_row_requant(y)
+        assert scale.dtype == np.float32 and scale[0, 0] == np.float32(s)
+        # 240 = 1.875 * 2^7 -> 0x77; with amax/448 the first code would be 448 = 0x7E and the second 16.8 -> 16
+        assert list(codes[0]) == [0x77, 0x51, 0xEF, 0x00]
+    # amax below 240e-5: the scale is exactly the floor and the codes are y / 1e-5
+    y = np.array([[1.2e-3, -6e-4, 0.0, 3e-4]], np.float32)
+    codes, scale = omoe.fp8_row_requant(y)
+    assert scale[0, 0] == np.float32(1e-5)
+    assert list(codes[0]) == [0x6F, 0xE7, 0x00, 0x5F]  # 120, -60, 0, 30
+    # an all-zero row does not divide by zero
+    codes, scale = omoe.fp8_row_requant(np.zeros((1, 8), np.float32))
+    assert scale[0, 0] == np.float32(1e-5) and not codes.any()
+
+
+def test_fp8_row_golden_uses_the_requant_rule():
+    """End to end through moe_blockwise_fp8_row_ref: one expert, gate = a constant, up = chosen values, down = a
+    selector matrix, so out[h] = code(y_h / scale) * scale.  The ratio out[1] / out[0] is 9/240 under the 240 rule
+    (9 is an e4m3 value) and 16/448 (5 % lower) had the range been 448."""
+    H = I = 16
+    x_codes = np.zeros((2, H), np.uint8)
+    x_codes[0, 0] = 0x38  # 1.0 in column 0; row 1 is the padding token
+    xs = np.array([1.0, 0.0], np.float32)
+    gu = np.zeros((1, H, 2, I), np.uint8)
+    gu[0, 0, 0, :] = 0x40  # gate = 2.0 everywhere
+    up_vals = np.zeros(I, np.float32)
+    up_vals[:3] = [240.0, 9.0, 120.0]
+    gu[0, 0, 1, :] = e4m3fn_encode(up_vals)
+    dw = np.zeros((1, I, H), np.uint8)
+    dw[0, np.arange(I), np.arange(H)] = 0x38
+    aff = np.array([[1.0], [0.0]], np.float32)
+    out = omoe.moe_blockwise_fp8_row_ref(x_codes, xs, aff, gu, dw, np.ones((1, 1, 2 * I), np.float32),
+                                         np.ones((1, 1, H), np.float32), np.array([0, 1], np.int32),
+                                         np.array([0], np.int32), 2)
+    silu2 = 2.0 / (1.0 + np.exp(-2.0))
+    assert abs(out[0, 0] / (240.0 * silu2) - 1) < 2.0**-8           # bf16 output rounding
+    assert abs(out[0, 1] / out[0, 0] - 9.0 / 240.0) < 9.0 / 240.0 * 2.0**-7
+    assert abs(out[0, 2] / out[0, 0] - 0.5) < 2.0**-8
 
 
 def test_fp8_row_reduces_to_dequantised_matmul():
