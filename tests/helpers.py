@@ -90,34 +90,37 @@ def mx_weights(rng, E, H, I, std=0.02, fmt="e4m3"):
     return gu_q, gu_s, d_q, d_s
 
 
+_CODE_POOLS = {}
+
+
 def _random_codes(rng, shape, fmt):
-    """Uniformly random element codes of an MX format without the NaN / infinity patterns."""
-    if fmt == "e2m1":
-        return rng.integers(0, 16, size=shape, dtype=np.uint8)
-    b = rng.integers(0, 256, size=shape, dtype=np.uint8)
-    if fmt == "e4m3":
-        b[(b & 0x7F) == 0x7F] &= 0xFE           # 0x7f / 0xff are NaN
-    else:
-        b[(b & 0x7C) == 0x7C] &= 0xFB           # e5m2: exponent 31 is infinity / NaN
-    return b
+    """Random element codes of an MX format whose VALUES are (nearly) uniform over the format's range, like the
+    reference's ``(np.random.random(shape) * 2 - 1) * max_val`` cast to the format (tensor_generators.py:381-384):
+    one random byte per element picks a sign and one of 128 magnitudes on an even grid over (0, max)."""
+    from oracle.numerics import e2m1_encode, e5m2_encode
+
+    if fmt not in _CODE_POOLS:
+        enc, vmax = {"e4m3": (e4m3fn_encode, 448.0), "e5m2": (e5m2_encode, 57344.0), "e2m1": (e2m1_encode, 6.0)}[fmt]
+        mag = enc(((np.arange(128, dtype=np.float64) + 0.5) * (vmax / 128)).astype(np.float32))
+        sign_bit = 0x08 if fmt == "e2m1" else 0x80
+        _CODE_POOLS[fmt] = np.concatenate([mag, mag | np.uint8(sign_bit)])
+    return _CODE_POOLS[fmt][rng.integers(0, 256, size=shape, dtype=np.uint8)]
 
 
 def mx_weights_random_codes(rng, E, H, I, fmt="e4m3", gate_rms=3.0):
     """Expert weights drawn directly in the quantised domain, the way the reference's generator does it
-    (generate_stabilized_mx_data, test/integration/nkilib/utils/tensor_generators.py:351-418: random element
-    codes, random E8M0 scales over a window of 11 exponents below an upper bound).  The upper bound is chosen so
-    that a projection of unit-variance inputs has a root mean square of about ``gate_rms``.  Fast enough for the
-    reference's own table shapes (no floating-point quantisation pass over hundreds of millions of elements)."""
-    from oracle.numerics import e2m1_decode, e5m2_decode
-
+    (generate_stabilized_mx_data, test/integration/nkilib/utils/tensor_generators.py:351-418: element values
+    uniform over the format's range, random E8M0 scales over a window of 11 exponents below an upper bound).  The
+    upper bound is chosen so that a projection of unit-variance inputs has a root mean square of about
+    ``gate_rms``.  Fast enough for the reference's own table shapes (no floating-point quantisation pass over
+    hundreds of millions of elements)."""
     nH, nI = H // 512, math.ceil(I / 512)
     pI = 128 if I > 512 else I // 4
     pI8 = math.ceil(pI / 8) * 8
-    table = {"e4m3": e4m3fn_decode, "e5m2": e5m2_decode, "e2m1": e2m1_decode}[fmt]
-    vals = table(np.arange(16 if fmt == "e2m1" else 256, dtype=np.uint8)).astype(np.float64)
-    rms_code = float(np.sqrt(np.mean(vals[np.isfinite(vals)] ** 2)))
+    rms_code = {"e4m3": 448.0, "e5m2": 57344.0, "e2m1": 6.0}[fmt] / math.sqrt(3.0)  # uniform over [-max, max]
 
     def scales(shape, K):
+        # E[4^(s - hi)] over the 11 exponents of the window = 0.1212: weights have rms_code * 2^(hi-127) * 0.348
         hi = int(round(127 + math.log2(gate_rms / (rms_code * 0.348 * math.sqrt(K)))))
         return rng.integers(hi - 10, hi + 1, size=shape, dtype=np.uint8)
 
