@@ -31,6 +31,7 @@ extern "C" {
 #define MOE_E_LAUNCH (-4)        /* hipLaunchKernel / hipMemsetAsync reported an error        */
 #define MOE_E_UNSUPPORTED (-5)   /* valid in the reference, not built here                    */
 #define MOE_E_NO_DEVICE (-6)     /* current device is not gfx950                              */
+#define MOE_E_STATIC_LIMIT (-7)  /* size beyond the built-in scratch of an entry point that allocates nothing */
 
 const char* moe_error_string(int code);
 /* ABI version of this header; bumped on any signature change. */
@@ -122,6 +123,22 @@ int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, i
                      int skip_token, int use_split_padding, int32_t* token_position_to_id,
                      int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
                      void* workspace, size_t workspace_bytes, int32_t* status_out, void* stream);
+
+/* moe_build_blocks for callers that cannot allocate or pass device scratch memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * the same results, bit for bit, as moe_build_blocks minus (workspace, workspace_bytes): the first slots and
+ * per-slab counts live in a device array built into the library, MOE_BUILD_BLOCKS_STATIC_BYTES per GPU for the
+ * life of the process.  Calls no hipMalloc / hipFree or any other allocating routine.  E above
+ * MOE_BUILD_BLOCKS_STATIC_MAX_E returns MOE_E_STATIC_LIMIT (use moe_build_blocks with a workspace instead).  The
+ * array is looked up once per device on the first call there (the device of `stream` must be current).  All calls
+ * on one GPU share that GPU's array: calls that overlap on one GPU (different streams, or threads) race; calls in
+ * stream order do not.  Nothing in the array has to be cleared between calls. */
+#define MOE_BUILD_BLOCKS_STATIC_MAX_E 512
+#define MOE_BUILD_BLOCKS_STATIC_BYTES (((1 + 64) * MOE_BUILD_BLOCKS_STATIC_MAX_E + 4) * 4) /* 133 136 bytes */
+int moe_build_blocks_static(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                            int skip_token, int use_split_padding, int32_t* token_position_to_id,
+                            int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
+                            int32_t* status_out, void* stream);
 
 /* The reference's device-side pieces of the same construction, as separate operators
  * (mask [T, E] -> per-expert token lists -> block offsets -> flat token_position_to_id).

@@ -12,6 +12,8 @@
 //   3. scatter_kernel  per slab, the same bitmaps again: a token's rank among the tokens of its expert is the
 //                      number of set bits below its own, plus the slab's offset; writes the token ids
 // The work is latency bound (a few hundred KB of int32), so each step is a single small launch.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace moe {
@@ -238,15 +240,15 @@ extern "C" size_t moe_build_blocks_workspace_bytes(int64_t E) {
   return (size_t)((1 + BB_SLABS_MAX) * E + 4) * sizeof(int32_t);
 }
 
-extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
-                                int skip_token, int use_split_padding, int32_t* token_position_to_id,
-                                int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions, void* workspace,
-                                size_t workspace_bytes, int32_t* status_out, void* stream) {
-  if (!topk_ids || !token_position_to_id || !block_to_expert || !workspace) return MOE_E_BAD_ARG;
-  if (T < 0 || k <= 0 || E <= 0 || B <= 0 || N <= 0) return MOE_E_BAD_ARG;
-  if (conditions && n_conditions < N) return MOE_E_BAD_SHAPE;
-  if (workspace_bytes < moe_build_blocks_workspace_bytes(E)) return MOE_E_WORKSPACE;
-  if (N * B >= (int64_t)1 << 31 || E > BB_E_MAX) return MOE_E_BAD_SHAPE;
+namespace {
+
+// Shared by the two entry points: `ws` is device memory of at least moe_build_blocks_workspace_bytes(E) bytes,
+// laid out as first_slot[E] | slab_counts[BB_SLABS_MAX][E].  Every word of it that a kernel reads was written
+// earlier in the same call (the count step writes the counts of every slab it launches, the layout step every
+// first slot), so stale contents of an earlier call are never seen and nothing has to be cleared.
+int build_blocks_launch(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N, int skip_token,
+                        int use_split_padding, int32_t* token_position_to_id, int32_t* block_to_expert,
+                        int32_t* conditions, int64_t n_conditions, int32_t* ws, int32_t* status_out, hipStream_t s) {
   // at most BB_SLABS_MAX slabs of a multiple of 256 tokens
   int64_t slab_tokens = (T + BB_SLABS_MAX - 1) / BB_SLABS_MAX;
   slab_tokens = (slab_tokens + BB_THREADS - 1) / BB_THREADS * BB_THREADS;
@@ -255,10 +257,9 @@ extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, i
   if (slab_tokens == 0) slab_tokens = BB_THREADS;
   int64_t n_slabs = (T + slab_tokens - 1) / slab_tokens;
   if (n_slabs == 0) n_slabs = 1;  // T == 0: one slab with no tokens still fills the pad ids
-  int32_t* first_slot = (int32_t*)workspace;
+  int32_t* first_slot = ws;
   int32_t* slab_counts = first_slot + E;
   const size_t lds = (size_t)9 * E * sizeof(int32_t);
-  hipStream_t s = (hipStream_t)stream;
   if (n_slabs == 1 && N * B <= BB_SINGLE_MAX_SLOTS) {
     hipLaunchKernelGGL(bb_single_slab_kernel, dim3(1), dim3(BB_THREADS), lds + 2 * E * sizeof(int32_t), s, topk_ids, T,
                        k, E, slab_tokens, slab_counts, first_slot, token_position_to_id, N * B,
@@ -277,4 +278,75 @@ extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, i
                      slab_tokens, slab_counts, first_slot, token_position_to_id, N * B);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
+}
+
+int build_blocks_check(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                       const int32_t* token_position_to_id, const int32_t* block_to_expert, const int32_t* conditions,
+                       int64_t n_conditions) {
+  if (!topk_ids || !token_position_to_id || !block_to_expert) return MOE_E_BAD_ARG;
+  if (T < 0 || k <= 0 || E <= 0 || B <= 0 || N <= 0) return MOE_E_BAD_ARG;
+  if (conditions && n_conditions < N) return MOE_E_BAD_SHAPE;
+  if (N * B >= (int64_t)1 << 31 || E > BB_E_MAX) return MOE_E_BAD_SHAPE;
+  return MOE_OK;
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------
+// Its scratch (first slots and per-slab counts, what moe_build_blocks takes as `workspace`) is a file-scope device
+// array sized for MOE_BUILD_BLOCKS_STATIC_MAX_E experts.  Every GPU holds its own copy of the array at its own
+// address for the life of the process; host code never uses the array's name as an address, only the per-device
+// pointer obtained once from hipGetSymbolAddress with that device current.
+}  // namespace
+
+constexpr size_t BB_STATIC_BYTES = (size_t)((1 + BB_SLABS_MAX) * MOE_BUILD_BLOCKS_STATIC_MAX_E + 4) * sizeof(int32_t);
+static_assert(BB_STATIC_BYTES == MOE_BUILD_BLOCKS_STATIC_BYTES, "the header states the size of the built-in scratch");
+static_assert(MOE_BUILD_BLOCKS_STATIC_MAX_E <= BB_E_MAX, "the built-in scratch covers a subset of moe_build_blocks");
+static __device__ __align__(256) unsigned char scratch[BB_STATIC_BYTES];
+
+namespace {
+
+constexpr int BB_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[BB_MAX_DEVICES];  // per device: address of that device's copy of `scratch`, null until first use
+
+// The current device's scratch, looked up on the first call on that device.
+int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= BB_MAX_DEVICES) return MOE_E_NO_DEVICE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MOE_E_LAUNCH;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return MOE_OK;
+}
+
+}  // namespace
+
+extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                                int skip_token, int use_split_padding, int32_t* token_position_to_id,
+                                int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions, void* workspace,
+                                size_t workspace_bytes, int32_t* status_out, void* stream) {
+  const int rc = build_blocks_check(topk_ids, T, k, E, B, N, token_position_to_id, block_to_expert, conditions, n_conditions);
+  if (rc != MOE_OK) return rc;
+  if (!workspace) return MOE_E_BAD_ARG;
+  if (workspace_bytes < moe_build_blocks_workspace_bytes(E)) return MOE_E_WORKSPACE;
+  return build_blocks_launch(topk_ids, T, k, E, B, N, skip_token, use_split_padding, token_position_to_id,
+                             block_to_expert, conditions, n_conditions, (int32_t*)workspace, status_out,
+                             (hipStream_t)stream);
+}
+
+extern "C" int moe_build_blocks_static(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                                       int skip_token, int use_split_padding, int32_t* token_position_to_id,
+                                       int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
+                                       int32_t* status_out, void* stream) {
+  int rc = build_blocks_check(topk_ids, T, k, E, B, N, token_position_to_id, block_to_expert, conditions, n_conditions);
+  if (rc != MOE_OK) return rc;
+  if (E > MOE_BUILD_BLOCKS_STATIC_MAX_E) return MOE_E_STATIC_LIMIT;  // checked before any device call
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != MOE_OK) return rc;
+  return build_blocks_launch(topk_ids, T, k, E, B, N, skip_token, use_split_padding, token_position_to_id,
+                             block_to_expert, conditions, n_conditions, (int32_t*)ws, status_out, (hipStream_t)stream);
 }

@@ -18,11 +18,13 @@ extern "C" const char* moe_error_string(int code) {
     case MOE_E_LAUNCH: return "HIP launch failed";
     case MOE_E_UNSUPPORTED: return "option not supported by the gfx950 implementation";
     case MOE_E_NO_DEVICE: return "current HIP device is not gfx950";
+    case MOE_E_STATIC_LIMIT:
+      return "size exceeds the built-in scratch of this entry point (it allocates nothing): use the variant that takes a workspace";
     default: return "unknown error code";
   }
 }
 
-extern "C" int moe_abi_version(void) { return 3; }
+extern "C" int moe_abi_version(void) { return 4; }
 
 extern "C" int moe_check_device(void) {
   int dev = 0;

@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "moe_rmsnorm_quant_mxfp8",
     "moe_build_blocks_workspace_bytes",
     "moe_build_blocks",
+    "moe_build_blocks_static",
     "moe_find_nonzero_indices_workspace_bytes",
     "moe_find_nonzero_indices",
     "moe_indexed_flatten",
@@ -135,6 +136,9 @@ def lib():
     L.moe_build_blocks.restype = c_int
     L.moe_build_blocks.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p,
                                    c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_void_p]
+    L.moe_build_blocks_static.restype = c_int
+    L.moe_build_blocks_static.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p,
+                                          c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
     L.moe_find_nonzero_indices_workspace_bytes.restype = c_size_t
     L.moe_find_nonzero_indices_workspace_bytes.argtypes = [c_int64, c_int64]
     L.moe_find_nonzero_indices.restype = c_int

@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported():
     for name in declared:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
     assert set(nv.EXPORTED_SYMBOLS) == set(declared)
-    assert L.moe_abi_version() == 3
+    assert L.moe_abi_version() == 4
     assert b"workspace" in L.moe_error_string(-3)
 
 
@@ -118,3 +118,15 @@ def test_shapes_beyond_the_32_bit_offsets_are_refused():
     assert ws(big_bf16) == 0 and rc(big_bf16) == BAD_SHAPE
     big_row = _valid_args(nv, nv.KIND_FP8_ROW, 4097, 4096, 14336, 8, 128, 2**34 // (128 * 14336) + 1)
     assert ws(big_row) == 0 and rc(big_row) == BAD_SHAPE
+
+
+def test_static_scratch_entry_point_rejects_sizes_beyond_its_scratch():
+    """moe_build_blocks_static checks its limit before it touches the device."""
+    from nkilib import _native as nv
+
+    L = nv.lib()
+    fake = ctypes.c_void_p(4096)
+    rc = L.moe_build_blocks_static(fake, 4, 2, 513, 128, 600, 0, 0, fake, fake, None, 0, None, None)
+    assert rc == -7 and b"allocates nothing" in L.moe_error_string(rc)
+    assert L.moe_build_blocks_static(None, 4, 2, 256, 128, 600, 0, 0, fake, fake, None, 0, None, None) == -1
+    assert L.moe_build_blocks_workspace_bytes(512) == 133136  # MOE_BUILD_BLOCKS_STATIC_BYTES in the header

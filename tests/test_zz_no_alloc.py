@@ -1,0 +1,71 @@
+"""The entry point that allocates nothing, moe_build_blocks_static, against moe_build_blocks: same bits, on two calls
+in a row (the second smaller, so that it runs on whatever the first left in the built-in scratch)."""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(L, nv, ids, E, B, N, skip_token, split, n_cond, dev):
+    import torch
+
+    T, k = ids.shape
+    outs = []
+    for static in (False, True):
+        # poison the outputs so that a slot the kernels leave unwritten shows
+        tp = torch.full((N * B,), -7, dtype=torch.int32, device=dev)
+        b2e = torch.full((N,), -7, dtype=torch.int32, device=dev)
+        cond = torch.full((n_cond,), -7, dtype=torch.int32, device=dev)
+        status = torch.zeros(1, dtype=torch.int32, device=dev)
+        s = nv.stream_ptr(dev)
+        if static:
+            rc = L.moe_build_blocks_static(nv.ptr(ids), T, k, E, B, N, int(skip_token), int(split), nv.ptr(tp),
+                                           nv.ptr(b2e), nv.ptr(cond), n_cond, nv.ptr(status), s)
+        else:
+            ws = torch.empty(L.moe_build_blocks_workspace_bytes(E), dtype=torch.uint8, device=dev)
+            rc = L.moe_build_blocks(nv.ptr(ids), T, k, E, B, N, int(skip_token), int(split), nv.ptr(tp), nv.ptr(b2e),
+                                    nv.ptr(cond), n_cond, nv.ptr(ws), ws.numel(), nv.ptr(status), s)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        outs.append((tp.cpu().numpy(), b2e.cpu().numpy(), cond.cpu().numpy(), int(status.item())))
+    return outs
+
+
+def test_static_scratch_entry_point_equals_workspace_entry_point():
+    import torch
+    from nkilib import _native as nv
+    from oracle import blocks as ob
+
+    L = nv.lib()
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    # first a many-slab call with the largest expert count the built-in scratch takes, then a smaller, single-slab one
+    for (T, k, E, B, skip, split) in [(8192, 8, 512, 128, False, False), (300, 4, 64, 128, True, True),
+                                      (8192, 8, 256, 128, False, False), (8, 8, 256, 128, False, False)]:
+        ids = torch.rand((T, E), generator=g, device=dev).topk(k, dim=1).indices.to(torch.int32).contiguous()
+        N = ob.get_n_blocks(T, k, E, B, n_block_per_iter=2)
+        ref, got = _both(L, nv, ids, E, B, N, skip, split, N + 2, dev)
+        for a, b, what in zip(ref, got, ("token_position_to_id", "block_to_expert", "conditions", "status")):
+            assert np.array_equal(a, b), f"T={T} E={E}: {what} differs"
+        assert ref[3] == 0 and (ref[0] != -7).all() and (ref[1] != -7).all()
+        # and both equal the oracle (the workspace entry point is checked against it elsewhere as well)
+        mask = ob.expert_mask_from_router(ids.cpu().numpy(), E)
+        tp_o, b2e_o, _ = ob.build_token_blocks(mask, B, N, skip, use_split_padding=split)[:3]
+        assert np.array_equal(got[0], tp_o) and np.array_equal(got[1], b2e_o)
+
+
+def test_static_scratch_limit_is_an_error():
+    import torch
+    from nkilib import _native as nv
+
+    L = nv.lib()
+    dev = torch.device("cuda:0")
+    ids = torch.zeros((4, 2), dtype=torch.int32, device=dev)
+    out = torch.zeros(1024 * 128, dtype=torch.int32, device=dev)
+    rc = L.moe_build_blocks_static(nv.ptr(ids), 4, 2, 513, 128, 600, 0, 0, nv.ptr(out), nv.ptr(out), None, 0, None,
+                                   nv.stream_ptr(dev))
+    assert rc == -7 and b"allocates nothing" in L.moe_error_string(rc)
