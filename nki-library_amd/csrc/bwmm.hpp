@@ -57,6 +57,8 @@ struct MxArgs {
   const int32_t* chunk_slot;
   const int32_t* chunk_rows;
   const int32_t* chunk_expert;
+  const int32_t* q_chunk;  // work queues: two words per chunk, per XCD grouped by class, see Bookkeeping
+  const int32_t* q_off;    // [8][CHUNK_CLASSES + 1]
   uint8_t* Yq;             // stage 1 output
   uint8_t* Ys;
   int64_t y_stride, ys_stride;

@@ -183,6 +183,14 @@ __device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const BOp& bf,
 #undef MX_MFMA_CASE
 #undef MX_MFMA_ASM
 
+// A vector memory instruction that reads a scalar register (descriptor, scalar offset) needs five wait states
+// after a vector ALU instruction that wrote that register (v_readfirstlane, v_readlane: the compiler reloads
+// spilled scalars with the latter right where they are used).  The compiler keeps that distance for instructions
+// of its own; for the instructions written out in this file it cannot (it does not see which operands an inline
+// statement reads when), so each of them carries the wait states itself.  They are issue slots in the shadow of
+// the MFMAs between which the loads sit.
+#define MX_SGPR_WAIT "s_nop 4\n\t"
+
 // Raw buffer descriptor over [p, p + bytes): loads take a per-lane 32-bit byte offset (VGPR) plus a
 // wave-uniform 32-bit byte offset (SGPR), which is exactly the shape of every address in this
 // kernel, so no 64-bit per-lane pointer is ever formed.
@@ -210,12 +218,12 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 template <bool NT>
 __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
   if constexpr (NT)
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile(MX_SGPR_WAIT "buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
   else
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile(MX_SGPR_WAIT "buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_store_dwordx2 %0, %1, %2, %3 offen nt" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile(MX_SGPR_WAIT "buffer_store_dwordx2 %0, %1, %2, %3 offen nt" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 // 16 bytes per lane straight into LDS at lds + 16 * lane (no destination registers).  The instruction takes its
 // LDS base from M0, which is set in the same statement.  M0 is declared clobbered: the compiler warns that it
@@ -223,35 +231,49 @@ __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& r
 // carries a value in M0 from one instruction to the next (it writes M0 itself immediately before each instruction
 // of its own that reads it), so there is nothing to save.
 __device__ __forceinline__ void ld_lds_b128(uint32_t lds, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile(MX_SGPR_WAIT "s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
 template <bool NT>
 __device__ __forceinline__ void ld_b64(v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
   if constexpr (NT)
-    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen nt" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile(MX_SGPR_WAIT "buffer_load_dwordx2 %0, %1, %2, %3 offen nt" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
   else
-    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile(MX_SGPR_WAIT "buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 typedef int v3i __attribute__((ext_vector_type(3)));
 __device__ __forceinline__ void ld_dwords(v3i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_dwordx3 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile(MX_SGPR_WAIT "buffer_load_dwordx3 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void ld_dwords(v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile(MX_SGPR_WAIT "buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void ld_b32(int& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile(MX_SGPR_WAIT "buffer_load_dword %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
-// NMT = number of 16-row tiles this instantiation multiplies (the chunk has at most NMT*16 rows).
+// A workgroup barrier that orders LDS traffic only.  (__syncthreads also makes the workgroup's global stores
+// visible, for which the compiler waits until every vector memory operation has completed -- the loads in flight
+// for the next tile included.)
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// NMT = number of 16-row tiles this instantiation multiplies (the chunks it takes have at most NMT*16 rows).
 // Keeping it a compile-time constant keeps the K loop free of branches around the MFMAs.
-// LASTUSE: this chunk is the last one of its expert, so its weights are streamed past the L2 (which
+// LASTUSE: the chunks are the last ones of their experts, so their weights are streamed past the L2 (which
 // then keeps the activation tiles that the sibling workgroups share); an earlier chunk loads them
 // normally, for the chunk after it to find.
+//
+// A workgroup stays on its CU and walks a list of tiles of one class (items L, L + Lstep, ... below endL of its
+// XCD's queue; an item is a chunk and one of its column tiles).  Between two tiles nothing is left to the
+// hardware's workgroup dispatch: as soon as the K loop of a tile has ended, the loads of the first D slices of the
+// next tile are issued, and only then does the tile's epilogue run -- the memory pipeline works through those
+// loads while the epilogue computes, and the next K loop starts on data that has arrived.  What the next tile
+// needs before its loads can be issued (token ids, affinities, bias) is read one tile earlier the same way:
+// requested before an epilogue, put in place after it.
 template <int STAGE, int NMT, bool LASTUSE, int WFMT>
-__device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int* s_tok, float* s_aff, int nrows, int e,
-                                             int64_t slot0, int xt) {
+__device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int (*s_tok)[MX_ROWS_MAX],
+                                             float (*s_aff)[MX_ROWS_MAX], float (*s_bias)[MXT], int L, const int endL,
+                                             const int Lstep, const int qbase) {
   using Cfg = MxCfg<NMT>;
   constexpr int D = Cfg::D, RING = Cfg::RING, SA = Cfg::SA, SS = Cfg::SS, SSP = Cfg::SSP;
   constexpr bool BIG = NMT > 16;  // row tiles 16.. accumulate in ordinary registers
@@ -265,38 +287,114 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
   const int c = lane & 15, g = lane >> 4;
   const int64_t nH = a.H / 512;
-
-  // ---- column tile ---------------------------------------------------------------------------
-  int tI = 0, p0 = 0, Pt = 128;
-  int64_t h0 = 0;
-  if (STAGE == 1) {
-    tI = xt >> 2;
-    p0 = (xt & 3) * 32;
-    const int64_t rows_t = (a.I - (int64_t)tI * 512 < 512) ? (a.I - (int64_t)tI * 512) : 512;
-    Pt = (int)(rows_t / 4);
-    if (p0 >= Pt) return;  // whole workgroup: Pt is a multiple of 32 on this path
-  } else {
-    h0 = (int64_t)xt * 256;
-  }
   const int q = w;
 
-  // ---- rows: token ids, affinities ---------------------------------------------------------------
-  for (int r = tid; r < NMT * 16; r += MXT) {
-    int id = -1;
-    if (r < nrows) {
-      id = a.tp2id[slot0 + r];
-      if (id < 0 || id >= a.n_real) id = -1;
+  // ---- tiles ------------------------------------------------------------------------------------
+  // Everything that says which tile: uniform values, kept in scalar registers.  A tile's queue entry (two words)
+  // is read through the scalar cache where it is needed, with an instruction of this file's own: a plain load is a
+  // vector load to the compiler (it cannot know that no store aliases the queue), and a vector load in the wrong
+  // place waits for every load in flight.
+  struct Tile {
+    int nrows, e, slot0, xt;
+  };
+  typedef int v2i_t __attribute__((ext_vector_type(2)));
+  auto tile_at = [&](int l) {
+    const int pos = l / a.col_tiles;
+    v2i_t raw;
+    asm volatile(MX_SGPR_WAIT "s_load_dwordx2 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                 : "=s"(raw) : "s"(a.q_chunk), "s"((qbase + pos) * 8) : "memory");
+    Tile t;
+    t.xt = l - pos * a.col_tiles;
+    t.slot0 = raw[0];
+    t.nrows = raw[1] & 0xffff;
+    t.e = raw[1] >> 16;
+    return t;
+  };
+  // gate/up: column tiles are numbered over the existing ones, 4 per full intermediate tile, then those of a
+  // short last tile (whose partitions per q are a multiple of 32 on this path): intermediate tile, first
+  // partition, partitions per q.  down: first hidden column.
+  auto tile_tI = [&](const Tile& t) { return t.xt >> 2; };
+  auto tile_p0 = [&](const Tile& t) { return (t.xt & 3) * 32; };
+  auto tile_Pt = [&](const Tile& t) {
+    const int64_t rows_t = (a.I - (int64_t)(t.xt >> 2) * 512 < 512) ? (a.I - (int64_t)(t.xt >> 2) * 512) : 512;
+    return (int)(rows_t / 4);
+  };
+  auto tile_h0 = [&](const Tile& t) { return (int64_t)t.xt * 256; };
+  // Rows: a thread looks after rows tid and 256 + tid of the chunk (token id, affinity), and after one of the
+  // tile's 256 bias values.  Each of these is fetched in two steps: `*_raw` issues loads (always from a valid
+  // address, no branch), `*_put` turns what arrived into the value and stores it in LDS.  Between the two lies an
+  // epilogue with a tile's first loads in flight.  The loads are instructions of this file's own, like those of
+  // the K loop: the compiler waits for a load of its own wherever it first touches the result or reuses the
+  // register, and such a wait would hold the epilogue until everything issued before it has arrived.
+  constexpr bool ROWS2 = NMT * 16 > 256;
+  auto ids_raw = [&](const Tile& t, int (&raw)[2]) {
+    const v4i rd = make_rsrc(a.tp2id, 0xffffffffu);
+#pragma unroll
+    for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
+      const int r = tid + 256 * j;
+      ld_b32(raw[j], (uint32_t)(t.slot0 + ((r < t.nrows) ? r : t.nrows - 1)) * 4u, rd, 0);
     }
-    s_tok[r] = id;
-    if (STAGE == 2) {
-      float af = 0.f;
-      if (id >= 0 && a.aff)
-        af = (a.aff_dtype == MOE_DT_BF16) ? bf16_bits_to_f32(((const uint16_t*)a.aff)[(int64_t)id * a.E + e])
-                                          : ((const float*)a.aff)[(int64_t)id * a.E + e];
-      s_aff[r] = af;
+  };
+  auto ids_put = [&](int buf, int nrows, const int (&raw)[2]) {
+#pragma unroll
+    for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
+      const int r = tid + 256 * j;
+      if (r < NMT * 16) s_tok[buf][r] = (r < nrows && raw[j] >= 0 && raw[j] < a.n_real) ? raw[j] : -1;
     }
-  }
-  __syncthreads();
+  };
+  // (No branch may surround such a load: where two paths that load into the same variable meet, the compiler
+  // copies the register right behind the load instruction, i.e. before the data has arrived.  So there is one
+  // load instruction for both element types -- the aligned word that holds the element, the half picked later --
+  // and a table that is absent is replaced by an address that is valid.)
+  auto elem_offset = [&](uint32_t idx, bool two_byte) { return two_byte ? ((idx << 1) & ~3u) : (idx << 2); };
+  auto elem_value = [&](int word, uint32_t idx, bool two_byte) {
+    return two_byte ? bf16_bits_to_f32((uint16_t)((uint32_t)word >> ((idx & 1u) * 16u))) : __builtin_bit_cast(float, word);
+  };
+  auto aff_index = [&](int e, int buf, int r) {
+    const int id = s_tok[buf][(r < NMT * 16) ? r : 0];
+    return (uint32_t)((id >= 0) ? id : 0) * (uint32_t)a.E + (uint32_t)e;
+  };
+  auto aff_raw = [&](const Tile& t, int buf, int (&raw)[2]) {
+    const v4i rd = make_rsrc(a.aff ? a.aff : (const void*)a.tp2id, 0xffffffffu);
+#pragma unroll
+    for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
+      const uint32_t off = a.aff ? elem_offset(aff_index(t.e, buf, tid + 256 * j), a.aff_dtype == MOE_DT_BF16) : 0u;
+      ld_b32(raw[j], off, rd, 0);
+    }
+  };
+  auto aff_put = [&](int e, int buf, const int (&raw)[2]) {
+#pragma unroll
+    for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
+      const int r = tid + 256 * j;
+      if (r < NMT * 16) {
+        float v = 0.f;
+        if (a.aff && s_tok[buf][r] >= 0) v = elem_value(raw[j], aff_index(e, buf, r), a.aff_dtype == MOE_DT_BF16);
+        s_aff[buf][r] = v;
+      }
+    }
+  };
+  // gate/up: bias value (gu*4 + q)*32 + pl belongs to partition p0 + pl; down: value j to column h0 + j.
+  const int hcol = (STAGE == 1) ? (c >> 3) : 0, cl = (STAGE == 1) ? (c & 7) : c;
+  auto bias_index = [&](const Tile& t) {
+    if (STAGE == 1) {
+      const uint32_t p = (uint32_t)(tile_p0(t) + (tid & 31));
+      return ((((uint32_t)t.e * (uint32_t)a.pI + p) * 2u + (uint32_t)(tid >> 7)) * (uint32_t)a.nI + (uint32_t)tile_tI(t)) * 4u +
+             (uint32_t)((tid >> 5) & 3);
+    }
+    return (uint32_t)t.e * (uint32_t)a.H + (uint32_t)tile_h0(t) + (uint32_t)tid;
+  };
+  auto bias_raw = [&](const Tile& t, int& raw) {
+    const v4i rd = make_rsrc(a.bias ? a.bias : (const void*)a.tp2id, 0xffffffffu);
+    ld_b32(raw, a.bias ? elem_offset(bias_index(t), a.bias_dtype == MOE_DT_BF16) : 0u, rd, 0);
+  };
+  auto bias_put = [&](const Tile& t, int buf, int raw) {
+    s_bias[buf][tid] = a.bias ? elem_value(raw, bias_index(t), a.bias_dtype == MOE_DT_BF16) : 0.f;
+  };
+  // what has been requested with the *_raw functions above may be used once this has passed
+  auto all_loads_landed = [&](int (&x)[2], int (&y)[2], int& z) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(y[0]), "+v"(y[1]), "+v"(z));
+  };
 
   // A staging: thread covers rows (tid>>3) + 32 j; its load goes straight to LDS slot tid&7 of that
   // row and fetches the 16-byte chunk (tid&7) ^ (row&7) that belongs there
@@ -307,30 +405,14 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // slots, rows past the end of the chunk) read some valid row instead of being zeroed: rows are
   // independent in a GEMM and the results of such rows are never written out, so what they hold
   // does not matter -- and the loads stay free of branches.
-  uint32_t a_voff[NAJ];
-#pragma unroll
-  for (int j = 0; j < NAJ; ++j) {
-    const int row = arow0 + 32 * j;
-    uint32_t r;
-    if (STAGE == 1) {
-      const int tok = s_tok[row];
-      r = (tok >= 0) ? (uint32_t)tok : 0u;
-    } else {
-      r = (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1)));
-    }
-    a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)((ach ^ (arow0 & 7)) * 16);
-  }
+  // (down stage: the rows are consecutive slots, so one per-lane offset serves all row groups and the group goes
+  // into the scalar offset; rows past the chunk's end may then lie past the end of the buffer, where the range
+  // check of the descriptor returns zeros)
+  constexpr int NAV = (STAGE == 1) ? NAJ : 1;
+  uint32_t a_voff[NAV];
   // A scales: thread covers row tid (and, in a chunk of more than 256 rows, row 256 + tid % 64: every
   // wave issues that load so that all waves count the same loads, the first wave's is used)
-  auto scale_row_off = [&](int row) {
-    if (STAGE == 1) {
-      const int tok = s_tok[row];
-      return ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
-    }
-    return (uint32_t)(slot0 + ((row < nrows) ? row : (nrows - 1))) * (uint32_t)a.a_scale_stride;
-  };
-  const uint32_t as_voff = scale_row_off(tid);
-  const uint32_t as_voff2 = BIG ? scale_row_off(256 + (tid & 63)) : 0u;
+  uint32_t as_voff = 0, as_voff2 = 0;
   // where the scales of row 256 + tid go: the other waves' copies land in a row tile that does not
   // exist (no branch inside the K loop: values that cross one stop being known as uniform)
   const int row_hi = (tid < 64) ? 256 + tid : 31 * 16 + (tid & 15);
@@ -350,16 +432,11 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   // ---- B operand addressing ---------------------------------------------------------------------------
   // byte address inside the expert's weights = uniform part (gate/up, K tile, partition
   // 32*pb + {r | 16 + r}, first column of the wave) + per-lane part (partition 4g, lane's columns).
-  int64_t w_pstride, w_tstride;  // element strides (4-byte weights; scales use the same counts in bytes)
-  v4i rw_, rs_;
-  uint32_t w_voff, s_voff;
-  int64_t colu;
   // A lane loads 16 bytes = 4 adjacent columns of one K row: column 4*cl + t belongs to column tile
   // t.  In the gate/up stage the wave's 32 gate columns take lanes c = 0..7 of each group and its 32
   // up columns lanes c = 8..15, so every column tile is half gate, half up, and one load instruction
   // fetches 128 contiguous bytes of gate and of up for 4 K rows.  (8-byte loads, one tile pair per
   // load, cost the memory pipeline as much per instruction as 16-byte ones.)
-  const int hcol = (STAGE == 1) ? (c >> 3) : 0, cl = (STAGE == 1) ? (c & 7) : c;
   // 4-bit weights (x4: four K values in a 2-byte element): lane group g needs K 32g .. 32g+31 of the
   // slice = partitions 8g .. 8g+7, one 8-byte load (4 columns) per partition; 8-bit weights (4-byte
   // elements): partitions 4g .. 4g+3 and 16+4g .. 16+4g+3, one 16-byte load each.
@@ -367,24 +444,14 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   constexpr int ES = FP4 ? 2 : 4;      // bytes of a weight element
   constexpr int GROWS = FP4 ? 8 : 4;   // partition rows between the lane groups' first rows
   const uint8_t* Wb = (const uint8_t*)a.W;
-  if (STAGE == 1) {
-    w_pstride = 2 * nH * a.I;
-    w_tstride = a.I;
-    colu = (int64_t)tI * 512 + (int64_t)q * Pt + p0;
-    rw_ = make_rsrc(Wb + (int64_t)e * 128 * w_pstride * ES, (uint32_t)(128 * w_pstride * ES));
-    rs_ = make_rsrc(a.W_scale + (int64_t)e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
-    w_voff = (uint32_t)((GROWS * g * w_pstride + hcol * nH * a.I + 4 * cl) * ES);
-    s_voff = (uint32_t)(g * w_pstride + hcol * nH * a.I + 4 * cl);
-  } else {
-    w_pstride = (int64_t)a.nI * a.H;
-    w_tstride = a.H;
-    colu = h0 + 64 * q;
-    const int64_t sp = (a.pI + 7) / 8;
-    rw_ = make_rsrc(Wb + (int64_t)e * a.pI * w_pstride * ES, (uint32_t)(a.pI * w_pstride * ES));
-    rs_ = make_rsrc(a.W_scale + (int64_t)e * sp * w_pstride, (uint32_t)(sp * w_pstride));
-    w_voff = (uint32_t)((GROWS * g * w_pstride + 4 * c) * ES);
-    s_voff = (uint32_t)(g * w_pstride + 4 * c);
-  }
+  // element strides (4-byte weights; scales use the same counts in bytes)
+  const int64_t w_pstride = (STAGE == 1) ? 2 * nH * a.I : (int64_t)a.nI * a.H;
+  const int64_t w_tstride = (STAGE == 1) ? a.I : a.H;
+  const uint32_t w_voff = (STAGE == 1) ? (uint32_t)((GROWS * g * w_pstride + hcol * nH * a.I + 4 * cl) * ES)
+                                       : (uint32_t)((GROWS * g * w_pstride + 4 * c) * ES);
+  const uint32_t s_voff = (STAGE == 1) ? (uint32_t)(g * w_pstride + hcol * nH * a.I + 4 * cl)
+                                       : (uint32_t)(g * w_pstride + 4 * c);
+  v4i rw_, rs_;  // the expert's weights and scales
 
   // A K slice's loads, numbered in issue order:
   //   0 .. NAJ-1            activation rows (16 bytes per lane each, straight into the LDS ring)
@@ -404,23 +471,67 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     RawLoad d[NBL];
     int sc;
   };
-  const v4i ra_ = make_rsrc(a.A, 0xffffffffu), ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_rows * a.a_scale_stride));
+  v4i ra_ = make_rsrc(a.A, (STAGE == 1) ? 0xffffffffu : (uint32_t)(a.a_rows * a.a_stride)),
+      ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_rows * a.a_scale_stride));
+  const int ra_rec = ra_[2], ras_rec = ras_[2];
+  int rw_rec = 0, rs_rec = 0;
+  const int a_group_bytes = uni((int)(32 * a.a_stride));  // down stage: bytes between row groups of 32 slots
   // Scalar byte offset of a weight load = (offset of its row and column within the slice, fixed per
   // load and kept in scalar registers) + (offset of the slice, computed once per slice): one scalar
   // add per load.  Address arithmetic done per load costs more issue cycles than the MFMAs between
   // two loads take.
   int w_soff[NBL];
+  int s_soff = 0;
+  // Point the loads at a tile: rows (token ids of the tile sit in s_tok[buf]), expert, columns.
+  auto aim_loads_at = [&](const Tile& t, int buf) {
 #pragma unroll
-  for (int i = 0; i < NBL; ++i) {
-    const int pr = FP4 ? i : ((i < 4) ? i : (16 + i - 4));
-    w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * ES);
-  }
-  const int s_soff = uni(colu);
+    for (int j = 0; j < NAV; ++j) {
+      const int row = arow0 + 32 * j;
+      uint32_t r;
+      if (STAGE == 1) {
+        const int tok = s_tok[buf][row];
+        r = (tok >= 0) ? (uint32_t)tok : 0u;
+      } else {
+        r = (uint32_t)(t.slot0 + row);
+      }
+      a_voff[j] = r * (uint32_t)a.a_stride + (uint32_t)((ach ^ (arow0 & 7)) * 16);
+    }
+    auto scale_row_off = [&](int row) {
+      if (STAGE == 1) {
+        const int tok = s_tok[buf][row];
+        return ((tok >= 0) ? (uint32_t)tok : 0u) * (uint32_t)a.a_scale_stride;
+      }
+      return (uint32_t)(t.slot0 + ((row < t.nrows) ? row : (t.nrows - 1))) * (uint32_t)a.a_scale_stride;
+    };
+    as_voff = scale_row_off(tid);
+    as_voff2 = BIG ? scale_row_off(256 + (tid & 63)) : 0u;
+    int64_t colu;
+    if (STAGE == 1) {
+      colu = (int64_t)tile_tI(t) * 512 + (int64_t)q * tile_Pt(t) + tile_p0(t);
+      rw_ = make_rsrc(Wb + (int64_t)t.e * 128 * w_pstride * ES, (uint32_t)(128 * w_pstride * ES));
+      rs_ = make_rsrc(a.W_scale + (int64_t)t.e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
+    } else {
+      colu = tile_h0(t) + 64 * q;
+      const int64_t sp = (a.pI + 7) / 8;
+      rw_ = make_rsrc(Wb + (int64_t)t.e * a.pI * w_pstride * ES, (uint32_t)(a.pI * w_pstride * ES));
+      rs_ = make_rsrc(a.W_scale + (int64_t)t.e * sp * w_pstride, (uint32_t)(sp * w_pstride));
+    }
+    rw_rec = rw_[2];
+    rs_rec = rs_[2];
+#pragma unroll
+    for (int i = 0; i < NBL; ++i) {
+      const int pr = FP4 ? i : ((i < 4) ? i : (16 + i - 4));
+      w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * ES);
+    }
+    s_soff = uni(colu);
+  };
   // Everything a slice's loads share: descriptors (of zero records past the end: such a load is out
   // of range, fetches nothing and returns zeros, so the K loop needs no conditions around its loads)
   // and the slice's scalar offsets.
+  // The four descriptors are kept once; what changes from slice to slice is their record count (word 2), which is
+  // set in place for the slice whose loads are about to be issued.
+  int tile_live = -1;  // 0: the loads being issued belong to no tile (behind the last tile of the list)
   struct SliceAddr {
-    v4i ra, ras, rw, rs;
     int a_off, as_off, w_off, s_off;
     uint32_t lds_a;  // LDS address of the ring stage that receives this slice's activations
   };
@@ -428,16 +539,11 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   auto slice_addr = [&](int ks, int st) {
     SliceAddr r;
     r.lds_a = uni((int)(lds_ring + (uint32_t)st * SA));
-    const int live = (ks < nks) ? -1 : 0;
-    auto sel = [&](const v4i& d) {
-      v4i x;
-      x[0] = uni(d[0]);
-      x[1] = uni(d[1]);
-      x[2] = uni(d[2] & live);
-      x[3] = uni(d[3]);
-      return x;
-    };
-    r.ra = sel(ra_); r.ras = sel(ras_); r.rw = sel(rw_); r.rs = sel(rs_);
+    const int live = (ks < nks) ? tile_live : 0;
+    ra_[2] = uni(ra_rec & live);
+    ras_[2] = uni(ras_rec & live);
+    rw_[2] = uni(rw_rec & live);
+    rs_[2] = uni(rs_rec & live);
     const int kt = ks >> 2, pb = ks & 3;
     r.a_off = ks * 128;
     r.as_off = ks * 4;
@@ -449,21 +555,24 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     constexpr int idx = decltype(idx_)::value;
     if constexpr (idx < NAJ) {
       // the wave's 64 lanes fill 8 rows x 128 bytes = 1 KB of the ring stage, in lane order
-      ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[idx], sa.ra, sa.a_off);
+      if constexpr (STAGE == 1)
+        ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[idx], ra_, sa.a_off);
+      else
+        ld_lds_b128(sa.lds_a + (uint32_t)((w * 8 + 32 * idx) * MXROW), a_voff[0], ra_, sa.a_off + idx * a_group_bytes);
     } else if constexpr (idx < NAJ + NSC) {
       // the four scale bytes (K blocks) of a row, for this slice and the D-1 after it: a lane's
       // dwords sit in different cache lines, so this load costs the memory pipeline as many
       // requests as all the activation rows of a slice together -- hence one in D slices
       if constexpr (decltype(with_scales_)::value) {
-        if constexpr (idx == NAJ) ld_dwords(sc0, as_voff, sa.ras, sa.as_off);
-        else ld_dwords(sc1, as_voff2, sa.ras, sa.as_off);
+        if constexpr (idx == NAJ) ld_dwords(sc0, as_voff, ras_, sa.as_off);
+        else ld_dwords(sc1, as_voff2, ras_, sa.as_off);
       }
     } else if constexpr (idx < NAJ + NSC + NBL) {
       constexpr int i = idx - NAJ - NSC;
-      if constexpr (FP4) ld_b64<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
-      else ld_b128<LASTUSE>(b.d[i], w_voff, sa.rw, w_soff[i] + sa.w_off);
+      if constexpr (FP4) ld_b64<LASTUSE>(b.d[i], w_voff, rw_, w_soff[i] + sa.w_off);
+      else ld_b128<LASTUSE>(b.d[i], w_voff, rw_, w_soff[i] + sa.w_off);
     } else {
-      ld_b32(b.sc, s_voff, sa.rs, s_soff + sa.s_off);
+      ld_b32(b.sc, s_voff, rs_, s_soff + sa.s_off);
     }
   };
   // The MFMA wants a lane's scale byte to be that of row 16*mt + c and K block g, one byte per row
@@ -476,13 +585,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     for (int gg = 0; gg < 4; ++gg) sd[(gg * 16 + cc) * SSP + mt] = (uint8_t)((raw >> (8 * gg)) & 0xffu);
   };
 
-  acc_fence();
-  static_for<0, (BIG ? 16 : NMT) * 16>([&](auto i_) { acc_zero<decltype(i_)::value>(); });
   v4f accv[4][4];  // row tiles 16..19
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) accv[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   // ---- K loop ---------------------------------------------------------------------------------------
   // Loads run D slices ahead of the MFMAs (what the memory system delivers is the amount in flight
@@ -600,12 +703,50 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
     __syncthreads();
   };
 
-  // prologue: the first D slices are requested at once; slice 0 needs its activations
-  static_for<0, D>([&](auto u_) {
-    constexpr int u = decltype(u_)::value;
-    const SliceAddr sa = slice_addr(u, u);
-    static_for<0, N0>([&](auto i_) { issue_load(i_, sa, br[u], asr, asr2, std::integral_constant<bool, u == 0>{}); });
-  });
+  // The first D slices of a tile are requested at once (for the first tile before anything else, for every later
+  // one ahead of the epilogue of the tile before it).
+  auto request_first_slices = [&]() {
+    static_for<0, D>([&](auto u_) {
+      constexpr int u = decltype(u_)::value;
+      const SliceAddr sa = slice_addr(u, u);
+      static_for<0, N0>([&](auto i_) { issue_load(i_, sa, br[u], asr, asr2, std::integral_constant<bool, u == 0>{}); });
+    });
+  };
+
+  // ---- first tile: nothing is in flight yet, so plain loads and waits do ----------------------------------
+  Tile cur = tile_at(L);
+  int ids_nn[2] = {0, 0}, aff_n[2] = {0, 0}, bias_n = 0;  // requested ahead of an epilogue, put in place after it
+  ids_raw(cur, ids_nn);
+  bias_raw(cur, bias_n);
+  all_loads_landed(ids_nn, aff_n, bias_n);
+  ids_put(0, cur.nrows, ids_nn);
+  bias_put(cur, 0, bias_n);
+  __syncthreads();
+  if (STAGE == 2) {
+    aff_raw(cur, 0, aff_n);
+    all_loads_landed(ids_nn, aff_n, bias_n);
+    aff_put(cur.e, 0, aff_n);
+  }
+  aim_loads_at(cur, 0);
+  request_first_slices();
+  int Ln = L + Lstep;  // the item after the current one
+  bool have_next = Ln < endL;
+  {
+    // (the wait in here also waits for the first slices: once per workgroup and class)
+    const Tile nx = tile_at(have_next ? Ln : L);
+    ids_raw(nx, ids_nn);
+    all_loads_landed(ids_nn, aff_n, bias_n);
+    if (have_next) ids_put(1, nx.nrows, ids_nn);  // published by the barrier below
+  }
+  int buf = 0;  // which of the two row tables (s_tok, s_aff, s_bias) belongs to the current tile
+
+  for (;;) {
+  acc_fence();
+  static_for<0, (BIG ? 16 : NMT) * 16>([&](auto i_) { acc_zero<decltype(i_)::value>(); });
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) accv[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NLB + (D - 1) * N1) : "memory");
   asm volatile("" : "+v"(asr));
   if constexpr (BIG) asm volatile("" : "+v"(asr2));
@@ -638,45 +779,71 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
   }
   asm volatile("" : : "v"(asr), "v"(asr2));
 
+  // ---- the next tile's first loads, and what the tile after it needs, go out ahead of the epilogue ---------
+  // The loads of the next tile's first D slices are in flight from here until the wait that follows the epilogue
+  // (into the ring stages 0 .. D-1 and into the raw register sets: the epilogue keeps to the last ring stage and
+  // leaves those registers alone), and so are the loads of the next tile's affinities and bias and of the token
+  // ids of the tile after it.
+  // No branch surrounds any of these loads (see above): after the last tile of the list they are issued all the
+  // same, the slices through descriptors of zero records (no traffic), the rest from the addresses of the last
+  // tile.
+  const bool have_nn = Ln + Lstep < endL;
+  const Tile nxt = tile_at(have_next ? Ln : L);
+  const Tile nn = tile_at(have_nn ? Ln + Lstep : L);
+  const int nbuf = have_next ? buf ^ 1 : buf;  // (behind the last tile: its own row table, which holds valid ids)
+  tile_live = have_next ? -1 : 0;
+  aim_loads_at(nxt, nbuf);
+  request_first_slices();
+  tile_live = -1;
+  if (STAGE == 2) aff_raw(nxt, nbuf, aff_n);
+  bias_raw(nxt, bias_n);
+  ids_raw(nn, ids_nn);
+
   // ---- epilogue ---------------------------------------------------------------------------------------------
+  // What the epilogue derives from the thread index it derives again here, from a copy the compiler cannot see
+  // through: otherwise those values are kept in registers across the K loop, where every register counts.
+  int tid_e = threadIdx.x;
+  asm volatile("" : "+v"(tid_e));
+  const int c_e = tid_e & 15, g_e = (tid_e & 63) >> 4;
+  const int hcol_e = (STAGE == 1) ? (c_e >> 3) : 0, cl_e = (STAGE == 1) ? (c_e & 7) : c_e;
   if (STAGE == 1) {
     // act(gate + bias) * (up + bias) in registers, then through LDS, 64 rows at a time, as
     // [row][q][32 partitions] fp32; then one thread per MX block (8 partitions x 4 q) quantises and
     // writes 32 K-contiguous bytes plus the scale byte.
-    float* E = (float*)smem;
+    // (the exchange buffer is the last ring stage, and for the 256-row variants the first 2 KB of the scale stages
+    // behind it: the stages before it are receiving the next tile's first slices)
+    float* E = (float*)(smem + (RING - 1) * SA);
+    static_assert((RING - 1) * SA + MX_LDS_EPI <= Cfg::LDS, "the exchange buffer must fit behind the stages in flight");
     // the lane's four partitions within the workgroup's 32: 4*cl + t
-    float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
-    if (a.bias) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int64_t p = p0 + 4 * cl + t;
-        const int64_t ig = ((((int64_t)e * a.pI + p) * 2 + 0) * a.nI + tI) * 4 + q;
-        const int64_t iu = ((((int64_t)e * a.pI + p) * 2 + 1) * a.nI + tI) * 4 + q;
-        if (a.bias_dtype == MOE_DT_BF16) {
-          bg[t] = bf16_bits_to_f32(((const uint16_t*)a.bias)[ig]);
-          bu[t] = bf16_bits_to_f32(((const uint16_t*)a.bias)[iu]);
-        } else {
-          bg[t] = ((const float*)a.bias)[ig];
-          bu[t] = ((const float*)a.bias)[iu];
-        }
-      }
+    float bg[4], bu[4];
+    {
+      const float4 vg = *(const float4*)(s_bias[buf] + q * 32 + 4 * cl_e), vu = *(const float4*)(s_bias[buf] + 128 + q * 32 + 4 * cl_e);
+      bg[0] = vg.x; bg[1] = vg.y; bg[2] = vg.z; bg[3] = vg.w;
+      bu[0] = vu.x; bu[1] = vu.y; bu[2] = vu.z; bu[3] = vu.w;
     }
-    const int pl0 = 4 * cl;
+    const int pl0 = 4 * cl_e;
     constexpr int NPS = NMT / 4;
     // Clamps as unconditional min/max against +-inf, and the activation kind as a compile-time
     // constant of the pass: a lane evaluates 128 elements here, and per-element decisions made this
     // code longer (and slower) than the K loop.
+    // (derived here, behind a statement the compiler cannot look through, and kept in scalar registers: computed
+    // once ahead of the tile loop they would sit in vector registers across the K loop)
+    int cmask = a.clamp_mask;
+    asm volatile("" : "+s"(cmask));
     const float inf = __builtin_inff();
-    const float g_lo = (a.clamp_mask & MOE_CLAMP_GATE_LO) ? a.clamp[1] : -inf;
-    const float g_hi = (a.clamp_mask & MOE_CLAMP_GATE_HI) ? a.clamp[0] : inf;
-    const float u_lo = (a.clamp_mask & MOE_CLAMP_UP_LO) ? a.clamp[3] : -inf;
-    const float u_hi = (a.clamp_mask & MOE_CLAMP_UP_HI) ? a.clamp[2] : inf;
+    auto limit = [&](int bit, float v, float none) {
+      return __builtin_bit_cast(float, uni(__builtin_bit_cast(int, (cmask & bit) ? v : none)));
+    };
+    const float g_lo = limit(MOE_CLAMP_GATE_LO, a.clamp[1], -inf);
+    const float g_hi = limit(MOE_CLAMP_GATE_HI, a.clamp[0], inf);
+    const float u_lo = limit(MOE_CLAMP_UP_LO, a.clamp[3], -inf);
+    const float u_hi = limit(MOE_CLAMP_UP_HI, a.clamp[2], inf);
     auto passes = [&](auto act_) {
     constexpr int ACT = decltype(act_)::value;
     static_for<0, NPS>([&](auto ps_) {
       constexpr int ps = decltype(ps_)::value;
-      if (ps * 64 < nrows) {
-        __syncthreads();
+      if (ps * 64 < cur.nrows) {
+        lds_barrier();
         static_for<0, 4>([&](auto m_) {
           constexpr int ml = decltype(m_)::value;
           constexpr int mt = ps * 4 + ml;
@@ -695,11 +862,11 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
               const float lo = av[t][k], hi = av[t][2 + k];
-              const float mine = hcol ? hi : lo;
-              const float send = hcol ? lo : hi;
+              const float mine = hcol_e ? hi : lo;
+              const float send = hcol_e ? lo : hi;
               const float recv = __builtin_bit_cast(
                   float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
-              const float gv = hcol ? recv : mine, uv = hcol ? mine : recv;
+              const float gv = hcol_e ? recv : mine, uv = hcol_e ? mine : recv;
               const float gg = fminf(fmaxf(gv + bg[t], g_lo), g_hi);
               const float uu = fminf(fmaxf(uv + bu[t], u_lo), u_hi);
               y[k][t] = act_apply(gg, ACT) * uu;
@@ -707,15 +874,15 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
           }
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
-            const int rl = ml * 16 + 4 * g + 2 * hcol + k;
+            const int rl = ml * 16 + 4 * g_e + 2 * hcol_e + k;
             *(float4*)(E + rl * MX_EP + q * 32 + pl0) = make_float4(y[k][0], y[k][1], y[k][2], y[k][3]);
           }
         });
-        __syncthreads();
+        lds_barrier();
         // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 32 (x 4 q)
-        const int rl = tid >> 2, j = tid & 3;
+        const int rl = tid_e >> 2, j = tid_e & 3;
         const int row = ps * 64 + rl;
-        if (row < nrows) {
+        if (row < cur.nrows) {
           const float* src = E + rl * MX_EP + 8 * j;
           float yv[4][8];
           float am = 0.f;
@@ -733,12 +900,12 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
           for (int k = 0; k < 8; ++k)
             d[k] = pack4_e4m3(clip448(yv[0][k] * is), clip448(yv[1][k] * is), clip448(yv[2][k] * is), clip448(yv[3][k] * is));
-          const int64_t slot = slot0 + row;
-          const int pw = p0 + 8 * j;  // first partition of the block within the intermediate tile
-          uint4* o = (uint4*)(a.Yq + slot * a.y_stride + tI * 512 + pw * 4);
+          const int64_t slot = cur.slot0 + row;
+          const int pw = tile_p0(cur) + 8 * j;  // first partition of the block within the intermediate tile
+          uint4* o = (uint4*)(a.Yq + slot * a.y_stride + tile_tI(cur) * 512 + pw * 4);
           o[0] = make_uint4(d[0], d[1], d[2], d[3]);
           o[1] = make_uint4(d[4], d[5], d[6], d[7]);
-          a.Ys[slot * a.ys_stride + tI * 16 + (pw >> 3)] = (uint8_t)sb;
+          a.Ys[slot * a.ys_stride + tile_tI(cur) * 16 + (pw >> 3)] = (uint8_t)sb;
         }
       }
     });
@@ -749,35 +916,33 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       case MOE_ACT_GELU_TANH: passes(std::integral_constant<int, MOE_ACT_GELU_TANH>{}); break;
       default: passes(std::integral_constant<int, MOE_ACT_SWISH>{}); break;
     }
+    // the scale stages that the exchange buffer reaches into are written at the top of the next tile
+    lds_barrier();
   } else {
-    const int64_t col0 = h0 + 64 * q + 4 * c;
-    float bd[4] = {0.f, 0.f, 0.f, 0.f};
-    if (a.bias) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int64_t ib = (int64_t)e * a.H + col0 + t;
-        bd[t] = (a.bias_dtype == MOE_DT_BF16) ? bf16_bits_to_f32(((const uint16_t*)a.bias)[ib]) : ((const float*)a.bias)[ib];
-      }
+    const int64_t col0 = tile_h0(cur) + 64 * q + 4 * c_e;
+    float bd[4];
+    {
+      const float4 vb = *(const float4*)(s_bias[buf] + 64 * q + 4 * c_e);
+      bd[0] = vb.x; bd[1] = vb.y; bd[2] = vb.z; bd[3] = vb.w;
     }
     const bool post = a.scaling_mode == MOE_SCALE_POST;
     // Rows go out through a descriptor that ends after the chunk's last row, so rows past the end
     // are dropped by the range check and the stores need no branches.  (Rows of padding slots
     // inside the chunk are written too: nothing reads the contributions of such slots.)
-    const v4i rd = make_rsrc(a.D + slot0 * a.H, (uint32_t)((int64_t)nrows * a.H * 2));
-    const uint32_t d_voff = (uint32_t)((4 * g * a.H + col0) * 2);
+    const v4i rd = make_rsrc(a.D + (int64_t)cur.slot0 * a.H, (uint32_t)((int64_t)cur.nrows * a.H * 2));
+    const uint32_t d_voff = (uint32_t)((4 * g_e * a.H + col0) * 2);
     const int rowb = uni(a.H * 2);
     typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
     typedef float v2f __attribute__((ext_vector_type(2)));
-    // the affinities of the lane's rows (4 consecutive rows per row tile), all requested before the
-    // first is used: a read per store, waited for on the spot, made the LDS latency the epilogue's pace
-    v4f aff4[NMT];
-#pragma unroll
-    for (int mt = 0; mt < NMT; ++mt) {
-      aff4[mt] = *(const v4f*)(s_aff + mt * 16 + 4 * g);
-      if (!post) aff4[mt] = (v4f){1.f, 1.f, 1.f, 1.f};
-    }
+    // the affinities of the lane's rows (4 consecutive rows per row tile) are read two row tiles ahead of their
+    // use: a read per store, waited for on the spot, made the LDS latency the epilogue's pace
+    v4f aff_q[3];
+    aff_q[0] = *(const v4f*)(s_aff[buf] + 0 * 16 + 4 * g_e);
+    aff_q[1] = *(const v4f*)(s_aff[buf] + 1 * 16 + 4 * g_e);
     static_for<0, NMT>([&](auto mt_) {
       constexpr int mt = decltype(mt_)::value;
+      if constexpr (mt + 2 < NMT) aff_q[(mt + 2) % 3] = *(const v4f*)(s_aff[buf] + (mt + 2) * 16 + 4 * g_e);
+      const v4f aff4 = post ? aff_q[mt % 3] : (v4f){1.f, 1.f, 1.f, 1.f};
       float av[4][4];  // [column tile][row]
       static_for<0, 16>([&](auto i_) {
         constexpr int i = decltype(i_)::value;
@@ -786,7 +951,7 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       });
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float af = aff4[mt][r];
+        const float af = aff4[r];
         v2i o;
 #pragma unroll
         for (int t = 0; t < 4; t += 2) {
@@ -797,7 +962,25 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
       }
     });
   }
+
+  // ---- hand over to the next tile ------------------------------------------------------------------------
+  // Everything in flight lands here: the next tile's first slices, this tile's stores (stores and loads share
+  // the counter but complete in no fixed order between them, so the K loop's counting waits must not start
+  // while stores are out), and the small loads issued ahead of the epilogue, which may be used from here on.
+  all_loads_landed(ids_nn, aff_n, bias_n);
+  if (!have_next) break;
+  if (STAGE == 2) aff_put(nxt.e, buf ^ 1, aff_n);
+  bias_put(nxt, buf ^ 1, bias_n);
+  if (have_nn) ids_put(buf, nn.nrows, ids_nn);  // the table of the tile that has just ended
+  cur = nxt;
+  L = Ln;
+  Ln += Lstep;
+  have_next = have_nn;
+  buf ^= 1;
+  }
+  return Ln;
 }
+
 
 // One translation unit per (stage, weight format): the build compiles this file once for each with
 // MX_INST_STAGE / MX_INST_WFMT defined, and once without them for the dispatcher below.
@@ -805,36 +988,38 @@ __device__ __forceinline__ void mx_gemm_body(const MxArgs& a, uint8_t* smem, int
 template <int STAGE, int WFMT>
 __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) void mx_gemm_kernel(const MxArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ int s_tok[MX_ROWS_MAX];
-  __shared__ __attribute__((aligned(16))) float s_aff[MX_ROWS_MAX];
-  // Workgroups are handed to the 8 XCDs round-robin by linear index, and each XCD has its own L2.
-  // XCD x therefore takes the x-th contiguous eighth of the chunk list (chunks are ordered by
-  // expert), and walks it chunk by chunk with the column tiles innermost: the workgroups that share
-  // an activation tile, and the chunks that share an expert's weights, then run at the same time
-  // behind the same L2, so each operand crosses the fabric about once.
-  const int n_chunks = __builtin_amdgcn_readfirstlane(*a.n_chunks);
-  const int per_xcd = (n_chunks + 7) >> 3;
-  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-  const int local = j / a.col_tiles, xt = j - local * a.col_tiles;
-  const int chunk = xcd * per_xcd + local;
-  if (local >= per_xcd || chunk >= n_chunks) return;
-  // values read from memory at a uniform address are uniform; say so, so that everything derived
-  // from them (buffer descriptors, scalar offsets) stays in scalar registers
-  const int nrows = __builtin_amdgcn_readfirstlane(a.chunk_rows[chunk]);
-  const int e = __builtin_amdgcn_readfirstlane(a.chunk_expert[chunk]);
-  const int64_t slot0 = __builtin_amdgcn_readfirstlane(a.chunk_slot[chunk]);
-  const bool last = (chunk + 1 >= n_chunks) || (__builtin_amdgcn_readfirstlane(a.chunk_expert[chunk + 1]) != e);
-  if (last) {
-    if (nrows <= 64) mx_gemm_body<STAGE, 4, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 128) mx_gemm_body<STAGE, 8, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 256) mx_gemm_body<STAGE, 16, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else mx_gemm_body<STAGE, 20, true, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-  } else {
-    if (nrows <= 64) mx_gemm_body<STAGE, 4, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 128) mx_gemm_body<STAGE, 8, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else if (nrows <= 256) mx_gemm_body<STAGE, 16, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
-    else mx_gemm_body<STAGE, 20, false, WFMT>(a, smem, s_tok, s_aff, nrows, e, slot0, xt);
+  __shared__ int s_tok[2][MX_ROWS_MAX];
+  __shared__ __attribute__((aligned(16))) float s_aff[2][MX_ROWS_MAX];
+  __shared__ __attribute__((aligned(16))) float s_bias[2][MXT];
+  // One workgroup per CU, for the whole launch.  Workgroups are handed to the 8 XCDs round-robin by linear
+  // index, and each XCD has its own L2.  XCD x therefore takes the x-th contiguous eighth of the chunk list
+  // (chunks are ordered by expert), as a queue of items (chunk, column tile) with the column tiles innermost
+  // and the chunks grouped by class; its workgroups take the items w, w + W, w + 2W, ... (W workgroups on the
+  // XCD).  The workgroups that share an activation tile, and the chunks that share an expert's weights, then run
+  // at the same time behind the same L2, so each operand crosses the fabric about once; and a workgroup's
+  // consecutive items are of one class, i.e. one instance of the code below, which carries its loads from tile
+  // to tile.
+  const int xcd = blockIdx.x & 7, w = blockIdx.x >> 3, W = gridDim.x >> 3;
+  const int32_t* qo = a.q_off + xcd * (CHUNK_CLASSES + 1);
+  const int qbase = __builtin_amdgcn_readfirstlane(qo[0]);
+  int L = w;
+  // classes in queue order (chunk_class): row-tile variants 20, 16, 8, 4, each first "not the last chunk of
+  // its expert", then "last"
+#define MX_RUN_CLASS(CLS_, NMT_, LAST_)                                                                        \
+  {                                                                                                            \
+    const int endL = (__builtin_amdgcn_readfirstlane(qo[CLS_ + 1]) - qbase) * a.col_tiles;                     \
+    if (L < endL) L = mx_gemm_tiles<STAGE, NMT_, LAST_, WFMT>(a, smem, s_tok, s_aff, s_bias, L, endL, W, qbase);       \
+    __syncthreads();                                                                                           \
   }
+  MX_RUN_CLASS(0, 20, false)
+  MX_RUN_CLASS(1, 20, true)
+  MX_RUN_CLASS(2, 16, false)
+  MX_RUN_CLASS(3, 16, true)
+  MX_RUN_CLASS(4, 8, false)
+  MX_RUN_CLASS(5, 8, true)
+  MX_RUN_CLASS(6, 4, false)
+  MX_RUN_CLASS(7, 4, true)
+#undef MX_RUN_CLASS
 }
 
 #define MX_CAT_(a, b, c, d) a##b##c##d
@@ -861,7 +1046,16 @@ int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStr
   if (gx == 0 || gy == 0) return MOE_OK;
   MxArgs m = m0;
   m.col_tiles = (int32_t)gx;
-  const unsigned grid = 8u * ((gy + 7u) / 8u) * gx;  // gy = upper bound on the number of chunks
+  // one workgroup per CU (a workgroup fills a CU's registers and most of its LDS, and walks its share of the
+  // tiles itself); fewer when there cannot be that many tiles (gy = upper bound on the number of chunks)
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
+    return MOE_E_LAUNCH;
+  const uint64_t tiles = (uint64_t)gx * gy;
+  unsigned per_xcd = (unsigned)cus / 8u;
+  if ((tiles + 7u) / 8u < per_xcd) per_xcd = (unsigned)((tiles + 7u) / 8u);
+  const unsigned grid = 8u * per_xcd;
   switch (m.wfmt) {
     case MX_WFMT_E4M3: return stage == 1 ? launch_mx_gemm_s1_f0(m, grid, s) : launch_mx_gemm_s2_f0(m, grid, s);
     case MX_WFMT_E5M2: return stage == 1 ? launch_mx_gemm_s1_f1(m, grid, s) : launch_mx_gemm_s2_f1(m, grid, s);

@@ -325,6 +325,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     m.chunk_slot = bk.chunk_slot;
     m.chunk_rows = bk.chunk_rows;
     m.chunk_expert = bk.chunk_expert;
+    m.q_chunk = bk.q_chunk;
+    m.q_off = bk.q_off;
     m.Yq = ws + p.yq;
     m.Ys = ws + p.ys;
     m.y_stride = p.Iw;
@@ -353,7 +355,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
       m1.a_rows = n_real;
       m1.W = (const uint32_t*)a->gate_up_proj_weight; m1.W_scale = (const uint8_t*)a->gate_up_proj_scale;
       m1.bias = a->gate_and_up_proj_bias;
-      rc = launch_mx_gemm(1, m1, (unsigned)(p.nI * 4), gyc, s);
+      // column tiles of 32 partitions x 4 q, gate and up: 4 per full intermediate tile + those of a short last one
+      rc = launch_mx_gemm(1, m1, (unsigned)((a->I / 512) * 4 + (a->I % 512) / 128), gyc, s);
     } else {
       rc = launch_gemm_stage(a->kind, 1, g1, gx1, gy, s);
     }

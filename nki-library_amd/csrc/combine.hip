@@ -62,6 +62,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
                                              const int32_t* __restrict__ valid_rows, int64_t N, int64_t B, int64_t E,
                                              int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
                                              int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
+                                             int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off,
                                              int64_t max_chunks, int* s_ws) {
   const int64_t na = *n_active;
   int carry = 0;
@@ -94,7 +95,40 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     }
     carry += total;
   }
-  if (threadIdx.x == 0) *n_chunks = (int32_t)((carry < max_chunks) ? carry : max_chunks);
+  const int n = (int)((carry < max_chunks) ? carry : max_chunks);
+  if (threadIdx.x == 0) *n_chunks = (int32_t)n;
+  // Work queues: a counting sort of the chunks by (XCD that owns them, class).  The chunk arrays were written by
+  // this workgroup: make them visible to all of its threads first.
+  __shared__ int s_cnt[8 * CHUNK_CLASSES + 1];
+  __threadfence_block();
+  __syncthreads();
+  const int per = (n + 7) >> 3;
+  for (int i = threadIdx.x; i <= 8 * CHUNK_CLASSES; i += blockDim.x) s_cnt[i] = 0;
+  __syncthreads();
+  auto key_of = [&](int i) {
+    const bool last = (i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]);
+    return (i / per) * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
+  };
+  for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&s_cnt[key_of(i)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int k = 0; k < 8 * CHUNK_CLASSES; ++k) {
+      const int c = s_cnt[k];
+      s_cnt[k] = run;
+      q_off[(k / CHUNK_CLASSES) * (CHUNK_CLASSES + 1) + k % CHUNK_CLASSES] = run;
+      run += c;
+      if (k % CHUNK_CLASSES == CHUNK_CLASSES - 1) q_off[(k / CHUNK_CLASSES) * (CHUNK_CLASSES + 1) + CHUNK_CLASSES] = run;
+    }
+  }
+  __syncthreads();
+  // (the order inside one class is whatever order the atomics are served in: it decides which chunks run at the
+  // same time, never a result)
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int pos = atomicAdd(&s_cnt[key_of(i)], 1);
+    q_chunk[2 * pos] = chunk_slot[i];
+    q_chunk[2 * pos + 1] = chunk_rows[i] | (chunk_expert[i] << 16);  // at most 320 rows, fewer than 32768 experts
+  }
 }
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(int32_t* __restrict__ p, int64_t n) {
@@ -132,11 +166,13 @@ __device__ __forceinline__ void inv_scan(const int32_t* __restrict__ cnt, int32_
 __global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
     const int32_t* __restrict__ b2e, const int32_t* __restrict__ n_active, const int32_t* __restrict__ valid_rows,
     int64_t N, int64_t B, int64_t E, int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
-    int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int64_t max_chunks,
-    const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n_real) {
+    int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int32_t* __restrict__ q_chunk,
+    int32_t* __restrict__ q_off, int64_t max_chunks, const int32_t* __restrict__ cnt, int32_t* __restrict__ off,
+    int64_t n_real) {
   __shared__ int s_ws[16];
   if (blockIdx.x == 0)
-    build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, max_chunks, s_ws);
+    build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, q_chunk, q_off,
+                 max_chunks, s_ws);
   else
     inv_scan(cnt, off, n_real, s_ws);
 }
@@ -220,11 +256,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
 // ---- host-side orchestration used by moe_blockwise() -------------------------------------
 
 size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B) {
-  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B] | n_chunks[4] | 3 x chunk[max_chunks],
-  // each region 256-byte aligned
+  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B] | n_chunks[4] | 5 x chunk[max_chunks] |
+  // q_off[8][CHUNK_CLASSES + 1], each region 256-byte aligned
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
   return al(16) + al((size_t)N * 4) + 2 * al((size_t)T1 * 4) + al((size_t)(T1 + 1) * 4) + al((size_t)N * B * 4) +
-         al(16) + 3 * al((size_t)max_chunks_for(N, B) * 4);
+         al(16) + 5 * al((size_t)max_chunks_for(N, B) * 4) + al((size_t)8 * (CHUNK_CLASSES + 1) * 4);
 }
 
 Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
@@ -241,7 +277,9 @@ Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
   k.n_chunks = (int32_t*)p; p += al(16);
   k.chunk_slot = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
   k.chunk_rows = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
-  k.chunk_expert = (int32_t*)p;
+  k.chunk_expert = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
+  k.q_chunk = (int32_t*)p; p += 2 * al((size_t)k.max_chunks * 4);
+  k.q_off = (int32_t*)p;
   return k;
 }
 
@@ -257,8 +295,8 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
                      a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows, k.cnt);
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(chunks_and_offsets_kernel, dim3(2), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows,
-                     a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.max_chunks, k.cnt,
-                     k.off, n_real);
+                     a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.q_chunk, k.q_off,
+                     k.max_chunks, k.cnt, k.off, n_real);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
   const unsigned gs = (unsigned)((slots + 255) / 256);

@@ -20,8 +20,22 @@ struct Bookkeeping {
   int32_t* chunk_slot;    // [max_chunks]
   int32_t* chunk_rows;    // [max_chunks]
   int32_t* chunk_expert;  // [max_chunks]
+  // Work queues of the large-tile MX kernels.  XCD x owns the x-th contiguous eighth of the chunk list; q_chunk holds
+  // that eighth's chunks grouped by class (row-tile variant x last chunk of its expert, CHUNK_CLASSES of them), two
+  // words per chunk: its first slot, and rows | expert << 16; q_off[x][c] .. q_off[x][c+1] are the positions of
+  // class c of XCD x in q_chunk.
+  int32_t* q_chunk;       // [max_chunks][2]
+  int32_t* q_off;         // [8][CHUNK_CLASSES + 1]
   int64_t max_chunks;
 };
+
+constexpr int CHUNK_CLASSES = 8;
+// class of a chunk: its row-tile variant (0: up to 64 rows, 1: 128, 2: 256, 3: 320), largest first, then whether
+// it is the last chunk of its expert
+__host__ __device__ inline int chunk_class(int rows, bool last) {
+  const int v = rows <= 64 ? 0 : rows <= 128 ? 1 : rows <= 256 ? 2 : 3;
+  return (3 - v) * 2 + (last ? 1 : 0);
+}
 
 constexpr int CHUNK_ROWS = 256;      // rows of every chunk of a run but the last
 constexpr int CHUNK_ROWS_MAX = 320;  // the last chunk of a run takes up to this many

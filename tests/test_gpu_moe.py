@@ -9,7 +9,9 @@ instead of the reference's 5e-2 for the quantised variants
 import numpy as np
 import pytest
 
-from helpers import bf16_tensor, dense_case, f32_tensor, from_bf16_tensor, i32_tensor, mx_case, u8_tensor
+from helpers import (affinities, bf16_tensor, dense_case, f32_tensor, from_bf16_tensor, i32_tensor, mx_case,
+                     mx_weights_random_codes, routing, u8_tensor)
+from oracle.numerics import to_bf16
 from oracle import moe as omoe
 from oracle import rmsnorm as orn
 from oracle.compare import max_abs_rel, max_all_close
@@ -531,6 +533,75 @@ def test_mx_activation_and_clamp_options(I, act, clamps):
     if clamps and len(clamps) == 1:
         # the limit must matter: without it the result is measurably different
         assert max_abs_rel(_golden_mx_options(c, act, None)[:T], g[:T]) > 2 * RTOL
+
+
+@pytest.mark.parametrize(
+    "H,T,I,E,B,k,fmt,dynamic,uint,via_moe_cte",
+    [
+        # the small-token rows of moe_bwmm_mx_shard_I_unit_perms (test_moe_bwmm_mx_cte.py:92-108): Swish, bias, clamps,
+        # skip_token, top-4 / top-8 over 8 experts with B = 256
+        (3072, 1024, 2048, 8, 256, 4, "e2m1", False, False, False),
+        (3072, 1024, 2048, 8, 256, 4, "e2m1", True, False, True),
+        (7168, 1024, 1024, 8, 256, 8, "e4m3", False, False, True),
+        (7168, 1024, 1024, 8, 256, 8, "e4m3", True, False, False),
+        (3072, 1024, 2048, 8, 256, 8, "e5m2", True, True, False),
+    ],
+)
+def test_mx_shard_on_i_entry_points(H, T, I, E, B, k, fmt, dynamic, uint, via_moe_cte):
+    """blockwise_mm_shard_intermediate_mx / _hybrid (bwmm_shard_on_I_mx.py:95-117, :400-426): the shard-on-block MX
+    golden, result in the shape of hidden_states, conditions with one entry per block plus one."""
+    import torch
+    from nkilib.core.moe.moe_cte import MoECTEImplementation, MoECTESpec, QuantizationConfig, SkipMode, moe_cte
+    from nkilib.core.moe.moe_cte.bwmm_shard_on_I_mx import (blockwise_mm_shard_intermediate_mx,
+                                                            blockwise_mm_shard_intermediate_mx_hybrid)
+    from nkilib.core.utils.common_types import ActFnType, ExpertAffinityScaleMode
+
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(41)
+    N, mask, tp2id, b2e, cond = routing(T, k, E, B, skip_token=True)  # not block parallel: conditions has N + 1 entries
+    assert cond.size == N + 1
+    hs = to_bf16(rng.standard_normal((T, H)).astype(np.float32))
+    gu_q, gu_s, d_q, d_s = mx_weights_random_codes(rng, E, H, I, fmt)
+    nI = I // 512
+    gub = to_bf16(rng.uniform(-2.0625, 0.52, size=(E, 128, 2, nI, 4)).astype(np.float32))
+    db = to_bf16(rng.uniform(-1.632, 1.4375, size=(E, H)).astype(np.float32))
+    aff = affinities(rng, T, E, mask, True)
+    if fmt == "e2m1":
+        from oracle.numerics import pack_e2m1_x4
+        gu = torch.from_numpy(pack_e2m1_x4(gu_q).view(np.int16)).to(dev)
+        dw = torch.from_numpy(pack_e2m1_x4(d_q).view(np.int16)).to(dev)
+        wd = None
+    elif uint:
+        gu = torch.from_numpy(gu_q.view(np.uint32).reshape(gu_q.shape[:-1])).to(dev)
+        dw = torch.from_numpy(d_q.view(np.uint32).reshape(d_q.shape[:-1])).to(dev)
+        wd = "float8_e5m2_x4" if fmt == "e5m2" else "float8_e4m3fn_x4"
+    else:
+        tdt = torch.float8_e5m2 if fmt == "e5m2" else torch.float8_e4m3fn
+        gu, dw, wd = u8_tensor(gu_q, dev).view(tdt), u8_tensor(d_q, dev).view(tdt), None
+    common = dict(gate_and_up_proj_bias=bf16_tensor(gub, dev), down_proj_bias=bf16_tensor(db, dev),
+                  activation_function=ActFnType.Swish, skip_dma=SkipMode(True, False),
+                  expert_affinities_scaling_mode=ExpertAffinityScaleMode.POST_SCALE, **REF_MX_CLAMPS)
+    args = (bf16_tensor(hs, dev), bf16_tensor(aff.reshape(-1, 1), dev), gu, dw, i32_tensor(tp2id, dev),
+            i32_tensor(b2e, dev))
+    scales = (u8_tensor(gu_s, dev), u8_tensor(d_s, dev))
+    if via_moe_cte:
+        assert wd is None
+        impl = MoECTEImplementation.shard_on_i_mx_hybrid if dynamic else MoECTEImplementation.shard_on_i_mx
+        out = moe_cte[2](*args, B, MoECTESpec(implementation=impl), conditions=i32_tensor(cond, dev) if dynamic else None,
+                         quantization_config=QuantizationConfig(*scales), **common)
+    elif dynamic:
+        out = blockwise_mm_shard_intermediate_mx_hybrid[2](i32_tensor(cond, dev), *args, gate_up_proj_scale=scales[0],
+                                                           down_proj_scale=scales[1], block_size=B, weight_dtype=wd,
+                                                           **common)
+    else:
+        out = blockwise_mm_shard_intermediate_mx[2](*args, gate_up_proj_scale=scales[0], down_proj_scale=scales[1],
+                                                    block_size=B, weight_dtype=wd, **common)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (T, H)
+    g = omoe.moe_blockwise_mx_ref(hs, aff, gu_q, d_q, gu_s, d_s, tp2id, b2e, B, conditions=cond if dynamic else None,
+                                  gate_up_proj_bias=gub, down_proj_bias=db, activation_function=3, skip_token=True,
+                                  weight_format=fmt, **REF_MX_CLAMPS)
+    _check(from_bf16_tensor(out), g, f"mx shard-on-I H={H} I={I} {fmt}")
 
 
 def test_mx_prequantised_equals_online():

@@ -96,12 +96,24 @@ def test_no_cpu_fallback():
                 MoECTESpec(MoECTEImplementation.shard_on_block))
 
 
-def test_unimplemented_enum_members_raise():
+def test_mx_shard_on_i_entry_points_validate_like_the_reference():
+    """blockwise_mm_shard_intermediate_mx[_hybrid] exist under the reference's import path, refuse PRE_SCALE with the
+    reference's message (bwmm_shard_on_I_mx.py:914-915) and are what the shard_on_i_mx enum members dispatch to."""
     from nkilib.core.moe.moe_cte import MoECTEImplementation, MoECTESpec, moe_cte
+    from nkilib.core.moe.moe_cte.bwmm_shard_on_I_mx import (blockwise_mm_shard_intermediate_mx,
+                                                            blockwise_mm_shard_intermediate_mx_hybrid)
+    from nkilib.core.utils.common_types import ExpertAffinityScaleMode
 
     z = torch.zeros(1)
-    with pytest.raises(AssertionError, match="no dispatch branch"):
-        moe_cte(z, z, z, z, z, z, 128, MoECTESpec(MoECTEImplementation.shard_on_i_mx))
+    with pytest.raises(AssertionError, match="PRE_SCALE mode not implemented"):
+        blockwise_mm_shard_intermediate_mx[2](z, z, z, z, z, z, block_size=256)  # the default mode is PRE_SCALE
+    with pytest.raises(AssertionError, match="conditions is required"):
+        blockwise_mm_shard_intermediate_mx_hybrid(None, z, z, z, z, z, z, block_size=256)
+    with pytest.raises(AssertionError, match="PRE_SCALE mode not implemented"):
+        moe_cte(z, z, z, z, z, z, 256, MoECTESpec(MoECTEImplementation.shard_on_i_mx),
+                expert_affinities_scaling_mode=ExpertAffinityScaleMode.PRE_SCALE)
+    with pytest.raises(AssertionError, match="gate_up_proj_scale and down_proj_scale are required"):
+        moe_cte(z, z, z, z, z, z, 256, MoECTESpec(MoECTEImplementation.shard_on_i_mx_hybrid), conditions=z)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
