@@ -254,6 +254,11 @@ typedef struct moe_bwmm_args {
    * in the workspace.  Ignored by the MXFP8 kind, whose x4 layouts are K-major already. */
   const void* gate_up_proj_weight_kmajor;
   const void* down_proj_weight_kmajor;
+  /* Nullable.  The reference's two-shard kernels return [T1, 2, H] or [2, T1, H] with the sum in shard 0 and
+   * zeros in shard 1 (output_shape, moe_cte.py:333-346).  When set, row t of that second plane lies at
+   * output_shard1 + t*out_row_stride elements and the combine pass writes it as zeros along with row t of
+   * `output`, so the caller needs no separate clear. */
+  void* output_shard1;
 } moe_bwmm_args;
 
 /* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /

@@ -24,7 +24,7 @@ extern "C" const char* moe_error_string(int code) {
   }
 }
 
-extern "C" int moe_abi_version(void) { return 4; }
+extern "C" int moe_abi_version(void) { return 5; }
 
 extern "C" int moe_check_device(void) {
   int dev = 0;
@@ -111,6 +111,10 @@ int validate(const moe_bwmm_args* a) {
     const int64_t pI = a->I > 512 ? 128 : a->I / 4, nI = (a->I + 511) / 512;
     if (a->T1 * a->H >= lim32 || slots * Iw >= lim32) return MOE_E_BAD_SHAPE;
     if (128 * 2 * (a->H / 512) * a->I * es >= lim31 || pI * nI * a->H * es >= lim31) return MOE_E_BAD_SHAPE;
+    // the row tables (token ids, affinities, bias) are fetched through 32-bit byte offsets as well
+    if (slots * 4 >= lim32 || a->T1 * a->E * 4 >= lim32 || a->E * pI * 2 * nI * 4 * 4 >= lim32 ||
+        a->E * a->H * 4 >= lim32)
+      return MOE_E_BAD_SHAPE;
   } else if (a->kind != MOE_KIND_MXFP8) {
     // general tiled kernel, dense kinds: row offsets are kept in units of 4 bytes in 32 bits (the value ~0 is
     // reserved for "no such row"), i.e. each A operand must stay below 2^34 - 4 bytes = 16 GiB

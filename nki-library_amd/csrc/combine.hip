@@ -195,7 +195,8 @@ __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict
 // One workgroup per output row.  D: bf16 [N*B, H] contributions.
 __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict__ D, const int32_t* __restrict__ off,
                                                       const int32_t* __restrict__ list, uint16_t* __restrict__ out,
-                                                      int64_t out_row_stride, int64_t H, int64_t n_real) {
+                                                      uint16_t* __restrict__ out_shard1, int64_t out_row_stride,
+                                                      int64_t H, int64_t n_real) {
   __shared__ int s_sorted[COMBINE_MAX_K];
   const int64_t t = blockIdx.x;
   int cnt = 0, base = 0;
@@ -213,7 +214,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
   }
   __syncthreads();
   uint16_t* orow = out + t * out_row_stride;
-  const bool vec = (H % 8 == 0) && ((out_row_stride % 8) == 0) && (((uintptr_t)out & 15) == 0);
+  uint16_t* zrow = out_shard1 ? out_shard1 + t * out_row_stride : nullptr;  // the other shard's row: zeros
+  const bool vec = (H % 8 == 0) && ((out_row_stride % 8) == 0) && (((uintptr_t)out & 15) == 0) &&
+                   (((uintptr_t)out_shard1 & 15) == 0);
   if (vec) {
     for (int64_t c = (int64_t)threadIdx.x * 8; c < H; c += (int64_t)blockDim.x * 8) {
       float acc[8];
@@ -243,12 +246,14 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
       for (int k = 0; k < 4; ++k)
         o[k] = (uint32_t)f32_to_bf16_bits(acc[2 * k]) | ((uint32_t)f32_to_bf16_bits(acc[2 * k + 1]) << 16);
       *(uint4*)(orow + c) = make_uint4(o[0], o[1], o[2], o[3]);
+      if (zrow) *(uint4*)(zrow + c) = make_uint4(0, 0, 0, 0);
     }
   } else {
     for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
       float acc = 0.f;
       for (int j = 0; j < cnt; ++j) acc = round_to_bf16(acc + bf16_bits_to_f32(D[(int64_t)s_sorted[j] * H + c]));
       orow[c] = f32_to_bf16_bits(acc);
+      if (zrow) zrow[c] = 0;
     }
   }
 }
@@ -308,7 +313,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
 
 int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, int64_t n_real, hipStream_t s) {
   hipLaunchKernelGGL(combine_kernel, dim3((unsigned)a->T1), dim3(256), 0, s, (const uint16_t*)D, k.off, k.list,
-                     (uint16_t*)a->output, a->out_row_stride, a->H, n_real);
+                     (uint16_t*)a->output, (uint16_t*)a->output_shard1, a->out_row_stride, a->H, n_real);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
 }

@@ -315,6 +315,121 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
   }
 }
 
+// The common case of the MXFP8 front end on its own: bf16 input and gamma, RMSNorm on, token-major output and no
+// copy of the normalised values.  Same results as rmsnorm_quant_mx_kernel, with the arithmetic per element cut to
+// what this case needs, because at ~20 vector instructions per element the general kernel is bound by the vector
+// ALUs and not by memory:
+//  - the block's amax is taken on the packed bf16 bit patterns (sign masked off, 16-bit unsigned max: magnitudes of
+//    finite bf16 values order like their bit patterns),
+//  - quantisation is v_cvt_scalef32_pk_fp8_bf16: two bf16 values divided by the power of two in the scale operand's
+//    exponent field and rounded to e4m3 (nearest even), one instruction per pair.  It differs from "multiply, clip
+//    to +-448, convert" in one respect only: a quotient that rounds above 448 gives NaN (0x7f / 0xff) instead of
+//    +-448; nan_to_max() turns those bytes into 0x7e / 0xfe.  (Checked over every finite bf16 value against every
+//    scale byte whose block can hold it.)
+//  - gamma is fetched with the row, ahead of the reduction, so the barrier hides its latency.
+__device__ __forceinline__ uint32_t nan_to_max(uint32_t d) {
+  // a byte is 0x7f / 0xff exactly when its low seven bits are all set: adding 1 to them carries into bit 7
+  const uint32_t m = ((d & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u;
+  return d - (m >> 7);
+}
+
+template <int MAXB>
+__global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? 6 : 3, 8))) void
+rmsnorm_quant_mx_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
+                             uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, int64_t rows, int64_t H,
+                             float eps, float hidden_actual, int tpr) {
+  typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
+  typedef short v2s16 __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf16 __attribute__((ext_vector_type(2)));
+  __shared__ double redd[16];
+  const int tpr_lg = (tpr == 64) ? 6 : ((tpr == 128) ? 7 : 8);
+  const int lt = threadIdx.x & (tpr - 1);
+  const int nblk_row = (int)(H / 32);
+  const int64_t Hq = H / 4;
+  const int64_t row_raw = ((int64_t)blockIdx.x << (8 - tpr_lg)) + (threadIdx.x >> tpr_lg);
+  const int64_t row = row_raw < rows ? row_raw : rows - 1;
+  const int nblk = row_raw < rows ? nblk_row : 0;  // threads of a row past the end own no block
+  const uint16_t* xr = x + row * H;
+
+  uint4 raw[MAXB][4], graw[MAXB][4];
+#pragma unroll
+  for (int j = 0; j < MAXB; ++j) {
+    const int blk = j * tpr + lt;
+    if (blk < nblk) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) raw[j][q] = *(const uint4*)(xr + q * Hq + blk * 8);  // tile*128 + p8*8 == blk*8
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < MAXB; ++j) {
+    const int blk = j * tpr + lt;
+    if (blk < nblk) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) graw[j][q] = *(const uint4*)(gamma + q * Hq + blk * 8);
+    }
+  }
+  {
+    double ss = 0.0;
+#pragma unroll
+    for (int j = 0; j < MAXB; ++j) {
+      if (j * tpr + lt < nblk) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t w[4] = {raw[j][q].x, raw[j][q].y, raw[j][q].z, raw[j][q].w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const double lo = (double)bf16_lo(w[k]), hi = (double)bf16_hi(w[k]);
+            ss = fma(lo, lo, ss);  // the products are exact in double, so fusing changes nothing
+            ss = fma(hi, hi, ss);
+          }
+        }
+      }
+    }
+    const float inv = 1.0f / sqrtf((float)group_sum_f64(ss, redd, tpr) / hidden_actual + eps);
+#pragma unroll
+    for (int j = 0; j < MAXB; ++j) {
+      const int blk = j * tpr + lt;
+      if (blk < nblk) {
+        uint32_t nv[4][4];  // normalised values, rounded to bf16: [q][pair of r]
+        v2u16 mx = {0, 0};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t w[4] = {raw[j][q].x, raw[j][q].y, raw[j][q].z, raw[j][q].w};
+          const uint32_t g[4] = {graw[j][q].x, graw[j][q].y, graw[j][q].z, graw[j][q].w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const uint32_t u =
+                pack2_bf16((bf16_lo(w[k]) * inv) * bf16_lo(g[k]), (bf16_hi(w[k]) * inv) * bf16_hi(g[k]));
+            nv[q][k] = u;
+            mx = __builtin_elementwise_max(mx, __builtin_bit_cast(v2u16, u & 0x7fff7fffu));
+          }
+        }
+        const uint32_t am = mx.x > mx.y ? mx.x : mx.y;    // bf16 bits of the block's amax
+        const int e8 = (int)(am >> 7) - 8;                // its biased exponent, less 8
+        const uint32_t sb = (uint32_t)(e8 < 0 ? 0 : e8);  // mx_scale_byte()
+        const float scale = __uint_as_float(sb << 23);    // 2^(sb - 127): only the exponent field is read
+        uint32_t d[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v2s16 w01 = {0, 0}, w23 = {0, 0};
+          w01 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(w01, __builtin_bit_cast(v2bf16, nv[0][k]), scale, false);
+          w01 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(w01, __builtin_bit_cast(v2bf16, nv[1][k]), scale, true);
+          w23 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(w23, __builtin_bit_cast(v2bf16, nv[2][k]), scale, false);
+          w23 = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(w23, __builtin_bit_cast(v2bf16, nv[3][k]), scale, true);
+          const uint32_t a = __builtin_bit_cast(uint32_t, w01), b = __builtin_bit_cast(uint32_t, w23);
+          // a = (q0 r, q0 r+1, q1 r, q1 r+1), b the same for q2, q3: regroup by r
+          d[2 * k] = nan_to_max(__builtin_amdgcn_perm(b, a, 0x06040200u));
+          d[2 * k + 1] = nan_to_max(__builtin_amdgcn_perm(b, a, 0x07050301u));
+        }
+        uint4* o = (uint4*)(out_q + row * H + (int64_t)blk * 32);
+        o[0] = make_uint4(d[0], d[1], d[2], d[3]);
+        o[1] = make_uint4(d[4], d[5], d[6], d[7]);
+        out_scale[row * nblk + blk] = (uint8_t)sb;
+      }
+    }
+  }
+}
+
 static bool valid_in_dtype(int d) { return d == MOE_DT_BF16 || d == MOE_DT_FP16 || d == MOE_DT_FP32; }
 
 }  // namespace moe
@@ -372,7 +487,16 @@ extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* g
     hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, x, x_dtype, gamma, gamma_dtype, (uint8_t*)out_q,
                        (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout, tpr);
   };
-  if (H <= 32 * RQ_THREADS) {
+  const bool fast = x_dtype == MOE_DT_BF16 && do_norm && gamma_dtype == MOE_DT_BF16 && !out_norm &&
+                    layout == MOE_MX_LAYOUT_TOKEN_MAJOR;
+  if (fast) {
+    auto launch_fast = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, (const uint16_t*)x, (const uint16_t*)gamma,
+                         (uint8_t*)out_q, (uint8_t*)out_scale, rows, H, eps, ha, tpr);
+    };
+    if (H <= 32 * RQ_THREADS) launch_fast(rmsnorm_quant_mx_bf16_kernel<1>);
+    else launch_fast(rmsnorm_quant_mx_bf16_kernel<MXQ_MAX_BLK>);
+  } else if (H <= 32 * RQ_THREADS) {
     if (x16) launch(rmsnorm_quant_mx_kernel<1, true>);
     else launch(rmsnorm_quant_mx_kernel<1, false>);
   } else {

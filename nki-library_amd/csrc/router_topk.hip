@@ -101,12 +101,15 @@ __device__ __forceinline__ v4i rt_rsrc(const void* p, uint32_t bytes) {
   d[3] = 0x00020000;
   return d;
 }
+// (s_nop 4: a scalar operand that a vector instruction has just written -- the compiler reloads spilled scalars
+// with v_readlane -- must not be read by a memory instruction within the next few cycles, and the compiler does
+// not know that these statements are memory instructions)
 __device__ __forceinline__ void rt_ld_lds(uint32_t lds, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                : : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
 __device__ __forceinline__ void rt_ld(v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
-  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(d) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 template <int NT, int MT, bool PIPE>

@@ -98,6 +98,7 @@ class BwmmArgs(ctypes.Structure):
         ("down_activations", c_void_p),
         ("gate_up_proj_weight_kmajor", c_void_p),
         ("down_proj_weight_kmajor", c_void_p),
+        ("output_shard1", c_void_p),
     ]
 
 

@@ -136,15 +136,16 @@ def run_blockwise(
         bias_dt = nv.DT_BF16 if gub.dtype == torch.bfloat16 else nv.DT_FP32
         kernel_assert(db.numel() == E * H, f"down_proj_bias must be [E, H] but got {tuple(db.shape)}")
 
-    # the combine stage writes every row of the result (zeros where a token has no contribution): only the second
-    # shard slot, which the reference leaves zero after its reduction, is cleared here
+    # the combine stage writes every row of the result (zeros where a token has no contribution) and, through
+    # output_shard1, zeros into the second shard slot, which the reference leaves zero after its reduction
+    shard1_ptr = None
     if out_shape_kind == "T2H":
         out = torch.empty((T1, 2, H), dtype=torch.bfloat16, device=dev)
-        out[:, 1].zero_()
+        shard1_ptr = out[:, 1].data_ptr()
         stride = 2 * H
     elif out_shape_kind == "2TH":
         out = torch.empty((2, T1, H), dtype=torch.bfloat16, device=dev)
-        out[1].zero_()
+        shard1_ptr = out[1].data_ptr()
         stride = H
     else:
         out = torch.empty((T1, H), dtype=torch.bfloat16, device=dev)
@@ -164,6 +165,7 @@ def run_blockwise(
     a.block_to_expert = nv.ptr(b2e)
     a.conditions = nv.ptr(cond)
     a.output = nv.ptr(out)
+    a.output_shard1 = shard1_ptr
     a.T1, a.H, a.I, a.E, a.B, a.N = T1, H, I, E, B, N
     a.I_pad = dims.get("I_pad", I)
     a.n_conditions = cond.numel() if cond is not None else 0

@@ -190,3 +190,13 @@ def f32_tensor(x, dev):
     import torch
 
     return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(dev)
+
+
+def dirty_device_memory(nbytes, device="cuda:0"):
+    """Leave a freed block of at least `nbytes` holding 0xff bytes in torch's caching allocator, so that the next
+    torch.empty of that size comes back dirty: what a kernel is said to write must then really be written."""
+    import torch
+
+    t = torch.full((int(nbytes),), 0xFF, dtype=torch.uint8, device=device)
+    torch.cuda.synchronize()
+    del t

@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported():
     for name in declared:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
     assert set(nv.EXPORTED_SYMBOLS) == set(declared)
-    assert L.moe_abi_version() == 4
+    assert L.moe_abi_version() == 5
     assert b"workspace" in L.moe_error_string(-3)
 
 
@@ -110,6 +110,9 @@ def test_shapes_beyond_the_32_bit_offsets_are_refused():
     # one expert's gate/up weights of 2 GiB: 2 * H * I bytes
     big_w = _valid_args(nv, nv.KIND_MXFP8, 129, 16384, 65536, 2, 128, 2, nv.DT_FP8)
     assert ws(big_w) == 0 and rc(big_w) == BAD_SHAPE
+    # affinity table of 2^32 bytes: (T+1) * E fp32 or bf16 entries at 4-byte granularity
+    big_aff = _valid_args(nv, nv.KIND_MXFP8, 2**21 + 1, 512, 512, 512, 128, 64, nv.DT_FP8)
+    assert ws(big_aff) == 0 and rc(big_aff) == BAD_SHAPE
     # ... which 4-bit weights (half the bytes) still fit
     assert ws(_valid_args(nv, nv.KIND_MXFP8, 129, 16384, 65536, 2, 128, 2, nv.DT_FP4_E2M1)) > 0
     # dense kinds: 16 GiB per A operand

@@ -9,7 +9,7 @@ instead of the reference's 5e-2 for the quantised variants
 import numpy as np
 import pytest
 
-from helpers import (affinities, bf16_tensor, dense_case, f32_tensor, from_bf16_tensor, i32_tensor, mx_case,
+from helpers import (affinities, bf16_tensor, dense_case, dirty_device_memory, f32_tensor, from_bf16_tensor, i32_tensor, mx_case,
                      mx_weights_random_codes, routing, u8_tensor)
 from oracle.numerics import to_bf16
 from oracle import moe as omoe
@@ -80,6 +80,7 @@ def _check(actual, golden, what, rtol=RTOL):
 def test_c1_tiny_bf16():
     """BASELINE config 1: T=256, H=512, I=1024, E=8, top-2, B=128, bf16, no quantisation."""
     c = dense_case(256, 512, 1024, 8, 2, 128, seed=0, hidden_std=1.0)
+    dirty_device_memory(257 * 2 * 512 * 2)  # the result buffer starts as 0xff: its zeros are written, not inherited
     out = _run_dense(c)
     assert tuple(out.shape) == (257, 2, 512)
     o = from_bf16_tensor(out)
@@ -376,6 +377,7 @@ def _golden_mx(c, act=0):
 )
 def test_mx_variants(T, H, I, E, k, B, bias, skip, dynamic, alpha, prequant):
     c = mx_case(T, H, I, E, k, B, seed=7, skip_token=skip, bias=bias, alpha=alpha, dynamic=dynamic)
+    dirty_device_memory(2 * (T + 1) * H * 2)
     out = _run_mx(c, prequant=prequant)
     o = from_bf16_tensor(out)
     assert o.shape[0] == 2 and not o[1].any()
