@@ -443,7 +443,8 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
               if (pre) { gv *= s_aff[row]; uv *= s_aff[row]; }
               gv *= sg; uv *= su;
             } else {
-              const float rs = __uint_as_float(sAs[row]);
+              // PRE_SCALE: the affinity scales the token's row, i.e. its dequantisation scale
+              const float rs = pre ? __uint_as_float(sAs[row]) * s_aff[row] : __uint_as_float(sAs[row]);
               gv = (gv * sg) * rs; uv = (uv * su) * rs;
             }
             gv += bg; uv += bu;

@@ -63,8 +63,7 @@ int validate(const moe_bwmm_args* a) {
   if (a->N * a->B >= ((int64_t)1 << 31) || a->T1 * a->E >= ((int64_t)1 << 31)) return MOE_E_BAD_SHAPE;
   const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
   if (Ipad < a->I) return MOE_E_BAD_SHAPE;
-  if ((a->gate_up_activations_T || a->down_activations) && (a->kind != MOE_KIND_BF16 || a->weight_dtype != MOE_DT_BF16))
-    return MOE_E_UNSUPPORTED;
+  if ((a->gate_up_activations_T || a->down_activations) && a->kind != MOE_KIND_BF16) return MOE_E_UNSUPPORTED;
   switch (a->kind) {
     case MOE_KIND_BF16:
       if (a->H % 8 != 0) return MOE_E_BAD_SHAPE;  // 16-byte row slices of bf16 hidden states
@@ -77,8 +76,6 @@ int validate(const moe_bwmm_args* a) {
       if (a->H % 16 != 0 || a->I % 4 != 0) return MOE_E_BAD_SHAPE;
       if (!a->gate_up_proj_scale || !a->down_proj_scale) return MOE_E_BAD_ARG;
       if (a->scale_experts != 1 && a->scale_experts != a->E) return MOE_E_BAD_SHAPE;
-      if (a->scaling_mode == MOE_SCALE_PRE || a->scaling_mode == MOE_SCALE_PRE_DELAYED) return MOE_E_UNSUPPORTED;
-      if (a->clamp_mask) return MOE_E_UNSUPPORTED;
       break;
     case MOE_KIND_MXFP8: {
       // bwmm_shard_on_block_mx.py:586-633, moe_cte_mx_utils.py:260-264

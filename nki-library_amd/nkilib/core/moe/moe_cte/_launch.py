@@ -97,7 +97,7 @@ def run_blockwise(
     checkpoint_down: bool = False,
 ):
     """dims: T1, H, I, E, I_pad.  out_shape_kind: "T2H" ([T1,2,H], slot 0), "2TH" ([2,T1,H], slot 0) or "TH".
-    With ``checkpoint_gate_up`` / ``checkpoint_down`` (bf16 weights only) the result is a tuple: the output, then
+    With ``checkpoint_gate_up`` / ``checkpoint_down`` (bf16 hidden states; bf16 or fp8 weight-only) the result is a tuple: the output, then
     ``gate_up_activations_T`` ``[N, 2, I, B]`` and / or ``down_activations`` ``[N, B, H]`` (bfloat16)."""
     L = nv.lib()
     skip_dma = skip_dma or SkipMode(False, False)
@@ -191,8 +191,7 @@ def run_blockwise(
     a.clamp_mask = mask
     ck_gu = ck_down = None
     if checkpoint_gate_up or checkpoint_down:
-        kernel_assert(kind == nv.KIND_BF16 and weight_dtype == nv.DT_BF16,
-                      "activation checkpoints need bfloat16 hidden states and weights")
+        kernel_assert(kind == nv.KIND_BF16, "activation checkpoints need bfloat16 hidden states")
     if checkpoint_gate_up:
         ck_gu = torch.empty((N, 2, I, B), dtype=torch.bfloat16, device=dev)
         a.gate_up_activations_T = nv.ptr(ck_gu)

@@ -187,8 +187,16 @@ def moe_blockwise_fp8_row_ref(
     down_proj_bias=None,
     activation_function=ACT_SILU,
     skip_token=False,
+    expert_affinities_scaling_mode=POST_SCALE,
+    gate_clamp_upper_limit=None,
+    gate_clamp_lower_limit=None,
+    up_clamp_upper_limit=None,
+    up_clamp_lower_limit=None,
 ):
     """fp8 activations (per-row scale) x fp8 weights (per-output-channel scale).
+
+    Affinity modes and clamps as in moe_blockwise_ref (test_moe_cte_common.py:383-402): PRE_SCALE scales the
+    token's row, which for a quantised row means its dequantisation scale.
 
     hidden_q uint8 [T+1, H] + hidden_row_scale fp32 [T+1]: the RMSNorm-Quant ROW
     record split as test_mlp_common.py:1061-1069.  Projection rule
@@ -221,12 +229,16 @@ def moe_blockwise_fp8_row_ref(
         a = to_bf16(aff[ids, e]).reshape(-1, 1)
         wgu = e4m3fn_decode(gate_up_w_q[e]).reshape(H, 2 * I)
         s = np.asarray(gate_up_w_scale, dtype=np.float32)[e].reshape(-1)
+        if expert_affinities_scaling_mode in (PRE_SCALE, PRE_SCALE_DELAYED):
+            rs = rs * a
         gu = (np.matmul(x, wgu) * s) * rs
         g = gu[:, :I].copy()
         u = gu[:, I:].copy()
         if gate_up_proj_bias is not None:
             g += np.asarray(gate_up_proj_bias, dtype=np.float32)[e, 0, :]
             u += np.asarray(gate_up_proj_bias, dtype=np.float32)[e, 1, :]
+        g = _clip(g, gate_clamp_lower_limit, gate_clamp_upper_limit)
+        u = _clip(u, up_clamp_lower_limit, up_clamp_upper_limit)
         y = (act_fn(g, activation_function) * u).astype(np.float32)
         yc, ys = fp8_row_requant(y)
         yq = e4m3fn_decode(yc)
@@ -235,7 +247,8 @@ def moe_blockwise_fp8_row_ref(
         d = (np.matmul(yq, wd) * sd) * ys
         if down_proj_bias is not None:
             d = d + np.asarray(down_proj_bias, dtype=np.float32)[e]
-        d = d * a
+        if expert_affinities_scaling_mode == POST_SCALE:
+            d = d * a
         _accumulate(out, ids, d.astype(np.float32))
     return out[:T1] if skip_token else out
 

@@ -122,21 +122,29 @@ def test_dense_variants(T, H, I, E, k, B, impl, act, mode, bias, skip, clamp):
     _check(o, g, f"dense {impl} act={act} mode={mode}")
 
 
-def _run_checkpointed(c, impl, act=0, mode=1, clamps=None, on_I=False, tp2id=None, b2e=None):
+def _run_checkpointed(c, impl, act=0, mode=1, clamps=None, on_I=False, tp2id=None, b2e=None, fp8_weights=False):
     import torch
-    from nkilib.core.moe.moe_cte import MoECTEImplementation, MoECTESpec, ShardOnIConfig, SkipMode, moe_cte
+    from nkilib.core.moe.moe_cte import (MoECTEImplementation, MoECTESpec, QuantizationConfig, ShardOnIConfig, SkipMode,
+                                         moe_cte)
     from nkilib.core.utils.common_types import ActFnType, ExpertAffinityScaleMode
 
     dev = torch.device("cuda:0")
     kw = dict(clamps or {})
+    if fp8_weights:
+        gu = u8_tensor(c["gate_up_q"], dev).view(torch.float8_e4m3fn)
+        dw = u8_tensor(c["down_q"], dev).view(torch.float8_e4m3fn)
+        kw["quantization_config"] = QuantizationConfig(f32_tensor(c["gate_up_scale"], dev),
+                                                       f32_tensor(c["down_scale"], dev))
+    else:
+        gu, dw = bf16_tensor(c["gate_up_w"], dev), bf16_tensor(c["down_w"], dev)
     if "gate_up_bias" in c:
         kw["gate_and_up_proj_bias"] = bf16_tensor(c["gate_up_bias"], dev)
         kw["down_proj_bias"] = bf16_tensor(c["down_bias"], dev)
     spec = MoECTESpec(implementation=getattr(MoECTEImplementation, impl),
                       shard_on_I=ShardOnIConfig(checkpoint_activation=True, expert_affinity_multiply_on_I=on_I))
     outs = moe_cte[2](
-        bf16_tensor(c["hidden"], dev), bf16_tensor(c["aff"].reshape(-1, 1), dev), bf16_tensor(c["gate_up_w"], dev),
-        bf16_tensor(c["down_w"], dev), i32_tensor(c["tp2id"] if tp2id is None else tp2id, dev),
+        bf16_tensor(c["hidden"], dev), bf16_tensor(c["aff"].reshape(-1, 1), dev), gu, dw,
+        i32_tensor(c["tp2id"] if tp2id is None else tp2id, dev),
         i32_tensor((c["b2e"] if b2e is None else b2e).reshape(-1, 1), dev), c["B"], spec,
         activation_function=ActFnType(act), skip_dma=SkipMode(c["skip_token"], False),
         expert_affinities_scaling_mode=ExpertAffinityScaleMode(mode), **kw)
@@ -177,6 +185,23 @@ def test_dense_checkpoint_activation(T, H, I, E, k, B, act, mode, bias, skip, cl
         d = from_bf16_tensor(outs[2])
         assert d.shape == (c["N"], B, H)
         _check(d, g_d, "down_activations")
+
+
+def test_dense_checkpoint_activation_fp8_weights():
+    """The checkpoints with fp8 weight-only quantisation (per-channel dequantisation scales,
+    bwmm_shard_on_I.py:160-176 with gate_up_proj_scale / down_proj_scale): the checkpointed projections carry the
+    scales, as the golden's in-place views do (test_moe_cte_common.py:383-405)."""
+    T, H, I, E, k, B = 300, 512, 384, 4, 2, 128
+    c = dense_case(T, H, I, E, k, B, seed=9, quant=True, bias=True, hidden_std=1.0)
+    outs = _run_checkpointed(c, "shard_on_i", act=0, mode=2, fp8_weights=True)
+    g_out, g_gu, g_d = omoe.moe_blockwise_ref(
+        c["hidden"], c["aff"], c["gate_up_w"], c["down_w"], c["tp2id"], c["b2e"], B,
+        gate_up_proj_bias=c.get("gate_up_bias"), down_proj_bias=c.get("down_bias"),
+        gate_up_proj_scale=c["gate_up_scale"], down_proj_scale=c["down_scale"], activation_function=0,
+        expert_affinities_scaling_mode=2, checkpoint_activation=True)
+    _check(from_bf16_tensor(outs[0])[:T], g_out[:T], "checkpointed output, fp8 weights")
+    _check(from_bf16_tensor(outs[1]), g_gu, "gate_up_activations_T, fp8 weights")
+    _check(from_bf16_tensor(outs[2]), g_d, "down_activations, fp8 weights")
 
 
 @pytest.mark.parametrize("mode,on_I", [(2, False), (1, True)])
@@ -268,10 +293,11 @@ def test_fp8_weight_only():
     _check(from_bf16_tensor(out), _golden_dense(c, fp8_weights=True), "fp8 weight-only")
 
 
-def _run_fp8_row(c, gamma):
+def _run_fp8_row(c, gamma, mode=1, clamps=None, act=0):
     import torch
     from nkilib.core.moe.moe_cte import QuantizationConfig, moe_cte
     from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+    from nkilib.core.utils.common_types import ActFnType, ExpertAffinityScaleMode
 
     dev = torch.device("cuda:0")
     rec = rmsnorm_quant_kernel(bf16_tensor(c["hidden"], dev), bf16_tensor(gamma, dev), RmsNormQuantKernelArgs())
@@ -279,7 +305,9 @@ def _run_fp8_row(c, gamma):
         rec, bf16_tensor(c["aff"].reshape(-1, 1), dev), u8_tensor(c["gate_up_q"], dev).view(torch.float8_e4m3fn),
         u8_tensor(c["down_q"], dev).view(torch.float8_e4m3fn), i32_tensor(c["tp2id"], dev),
         i32_tensor(c["b2e"], dev), c["B"], _spec("shard_on_block"),
-        quantization_config=QuantizationConfig(f32_tensor(c["gate_up_scale"], dev), f32_tensor(c["down_scale"], dev)))
+        quantization_config=QuantizationConfig(f32_tensor(c["gate_up_scale"], dev), f32_tensor(c["down_scale"], dev)),
+        activation_function=ActFnType(act), expert_affinities_scaling_mode=ExpertAffinityScaleMode(mode),
+        **(clamps or {}))
     torch.cuda.synchronize()
     return rec, out
 
@@ -299,6 +327,26 @@ def test_fp8_row_pipeline(T, H, I, E, k, B):
     g = omoe.moe_blockwise_fp8_row_ref(codes, scale, c["aff"], c["gate_up_q"], c["down_q"], c["gate_up_scale"],
                                        c["down_scale"], c["tp2id"], c["b2e"], c["B"])
     _check(from_bf16_tensor(out)[:, 0], g, "fp8 row")
+
+
+@pytest.mark.parametrize("mode,clamp,act", [(2, False, 0), (1, True, 3), (2, True, 1), (0, False, 0)])
+def test_fp8_row_scale_modes_and_clamps(mode, clamp, act):
+    """PRE_SCALE (the affinity scales the token's row, i.e. its dequantisation scale), NO_SCALE and the four clamps on
+    the fp8-row kind.  The reference has no kernel with fp8 activations on this path: the rule is the dense
+    golden's (test_moe_cte_common.py:383-402) applied to the row-quantised operands."""
+    import torch
+
+    T, H, I, E, k, B = 384, 1024, 896, 8, 2, 128
+    c = dense_case(T, H, I, E, k, B, seed=16, quant=True, hidden_std=1.0)
+    clamps = dict(gate_clamp_upper_limit=0.6, gate_clamp_lower_limit=-0.5, up_clamp_upper_limit=0.7,
+                  up_clamp_lower_limit=-0.4) if clamp else {}
+    rec, out = _run_fp8_row(c, np.ones((1, H), np.float32), mode=mode, clamps=clamps, act=act)
+    raw = rec.view(torch.uint8).cpu().numpy()
+    codes, scale = raw[:, :H], raw[:, H:].copy().view(np.float32).reshape(-1)
+    g = omoe.moe_blockwise_fp8_row_ref(codes, scale, c["aff"], c["gate_up_q"], c["down_q"], c["gate_up_scale"],
+                                       c["down_scale"], c["tp2id"], c["b2e"], c["B"], activation_function=act,
+                                       expert_affinities_scaling_mode=mode, **clamps)
+    _check(from_bf16_tensor(out)[:, 0], g, f"fp8 row mode={mode} clamp={clamp} act={act}")
 
 
 def _run_mx(c, prequant=False, act=0, weight_dtype=None):
