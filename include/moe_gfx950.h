@@ -230,8 +230,7 @@ typedef struct moe_bwmm_args {
   /* -- options ------------------------------------------------------------------------- */
   int32_t kind;           /* MOE_KIND_*                                                           */
   int32_t weight_dtype;   /* BF16 kind: MOE_DT_BF16 or MOE_DT_FP8_E4M3; MXFP8 kind: MOE_DT_FP8_E4M3 (also
-                           * taken for MOE_DT_BF16, the zero value), MOE_DT_FP8_E5M2 or MOE_DT_FP4_E2M1 (the
-                           * last two on large-tile shapes only: H % 512 == 0 and I % 128 == 0):
+                           * taken for MOE_DT_BF16, the zero value), MOE_DT_FP8_E5M2 or MOE_DT_FP4_E2M1:
                            * nl.float8_e4m3fn_x4 / float8_e5m2_x4 / float4_e2m1fn_x4 in the reference; 4-bit
                            * weights have the same shapes with 2-byte elements                              */
   int32_t affinity_dtype; /* MOE_DT_BF16 or MOE_DT_FP32                                           */

@@ -21,6 +21,8 @@
 //   test/integration/nkilib/core/moe/moe_cte/test_utils.py:474-735 with
 //   test/integration/nkilib/core/mlp/test_mlp_common.py:550-682 (MXFP8),
 //   test/integration/nkilib/core/mlp/test_mlp_common.py:978-1022,1114-1116 (fp8 row scales).
+#include <type_traits>
+
 #include "bwmm.hpp"
 
 namespace moe {
@@ -151,6 +153,7 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
     for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   // ---- K loop ---------------------------------------------------------------------------
+  const bool fp4 = KIND == MOE_KIND_MXFP8 && a.weight_dtype == MOE_DT_FP4_E2M1;  // 4-bit weights
   int nks;
   if (KIND == MOE_KIND_MXFP8) nks = (STAGE == 1) ? (int)(a.H / 128) : a.nI * 4;
   else if (KIND == MOE_KIND_BF16) nks = (int)((a.K + 63) / 64);
@@ -301,6 +304,7 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
     // ---- stage B, transposed into K-contiguous rows ---------------------------------------
     if (KIND == MOE_KIND_MXFP8) {
       const uint32_t* W4 = (const uint32_t*)a.W;
+      const uint16_t* W2 = (const uint16_t*)a.W;
       if (STAGE == 1) {
         // column = tid: (gu, q, pl); rows rho = partitions 32*pb + rho of H tile kt
         const int gu = tid >> 7, q = (tid >> 5) & 3, pl = tid & 31;
@@ -309,10 +313,15 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
         const int64_t nH = a.H / 512;
         const int64_t pstride = 2 * nH * a.I;
         const int64_t base = ((((int64_t)e * 128 + pb * 32) * 2 + gu) * nH + kt) * a.I + i;
+        if (fp4) {  // 2-byte x4 elements: a row's 128 K values are 64 bytes
 #pragma unroll 8
-        for (int rho = 0; rho < 32; ++rho) {
-          const uint32_t v = cv ? W4[base + rho * pstride] : 0u;
-          *(uint32_t*)(sB + tid * LROW + rho * 4) = v;
+          for (int rho = 0; rho < 32; ++rho) *(uint16_t*)(sB + tid * LROW + rho * 2) = cv ? W2[base + rho * pstride] : (uint16_t)0;
+        } else {
+#pragma unroll 8
+          for (int rho = 0; rho < 32; ++rho) {
+            const uint32_t v = cv ? W4[base + rho * pstride] : 0u;
+            *(uint32_t*)(sB + tid * LROW + rho * 4) = v;
+          }
         }
         uint32_t sv = 0;
         if (cv) {
@@ -330,8 +339,9 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
 #pragma unroll 8
         for (int j = 0; j < 16; ++j) {
           const int rho = 2 * j + half;
-          const uint32_t v = (cv && pb * 32 + rho < Ptk) ? W4[base + rho * pstride] : 0u;
-          *(uint32_t*)(sB + col * LROW + rho * 4) = v;
+          const bool ok = cv && pb * 32 + rho < Ptk;
+          if (fp4) *(uint16_t*)(sB + col * LROW + rho * 2) = ok ? W2[base + rho * pstride] : (uint16_t)0;
+          else *(uint32_t*)(sB + col * LROW + rho * 4) = ok ? W4[base + rho * pstride] : 0u;
         }
         if (half == 0) {
           uint32_t sv = 0;
@@ -355,15 +365,29 @@ __global__ __launch_bounds__(GT) __attribute__((amdgpu_waves_per_eu(KIND == MOE_
         af[mt] = lds_read_frag(sA + row * LROW, g);
         sa[mt] = (int)((sAs[row] >> (8 * g)) & 0xffu);
       }
+      // the element format of the weights is an immediate of the instruction (blgp: 0 e4m3, 1 e5m2, 4 e2m1); a
+      // 4-bit operand is four registers, lane group g holding K 32g .. 32g+31 = bytes [16g, 16g+16) of the row
+      auto columns = [&](auto blgp_) {
+        constexpr int BLGP = decltype(blgp_)::value;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const int col = nt * 16 + c;
-        const v8i bf = lds_read_frag(sB + col * LROW, g);
-        const int sb = (int)((sBs[col] >> (8 * g)) & 0xffu);
+        for (int nt = 0; nt < NT; ++nt) {
+          const int col = nt * 16 + c;
+          v8i bf;
+          if constexpr (BLGP == 4) {
+            const v4i lo = *(const v4i*)(sB + col * LROW + 16 * g);
+            bf = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+          } else {
+            bf = lds_read_frag(sB + col * LROW, g);
+          }
+          const int sb = (int)((sBs[col] >> (8 * g)) & 0xffu);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, 0, 0, sa[mt], 0, sb);
-      }
+          for (int mt = 0; mt < 2; ++mt)
+            acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt], bf, acc[nt][mt], 0, BLGP, 0, sa[mt], 0, sb);
+        }
+      };
+      if (a.weight_dtype == MOE_DT_FP8_E5M2) columns(std::integral_constant<int, 1>{});
+      else if (fp4) columns(std::integral_constant<int, 4>{});
+      else columns(std::integral_constant<int, 0>{});
     }
     __syncthreads();
   }

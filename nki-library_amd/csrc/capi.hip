@@ -85,12 +85,10 @@ int validate(const moe_bwmm_args* a) {
       if (!a->gate_up_proj_scale || !a->down_proj_scale) return MOE_E_BAD_ARG;
       // POST_SCALE only (test_moe_bwmm_mx_cte.py:163-167)
       if (a->scaling_mode == MOE_SCALE_PRE || a->scaling_mode == MOE_SCALE_PRE_DELAYED) return MOE_E_UNSUPPORTED;
-      // weight element formats: e4m3 everywhere, e5m2 on the large-tile path
-      if (a->weight_dtype == MOE_DT_FP8_E5M2 || a->weight_dtype == MOE_DT_FP4_E2M1) {
-        if (!mx_fast_path_ok(a->H, a->I)) return MOE_E_UNSUPPORTED;
-      } else if (a->weight_dtype != MOE_DT_FP8_E4M3 && a->weight_dtype != MOE_DT_BF16) {
+      // weight element formats: e4m3 (also for the zero value, MOE_DT_BF16), e5m2, e2m1
+      if (a->weight_dtype != MOE_DT_FP8_E4M3 && a->weight_dtype != MOE_DT_BF16 && a->weight_dtype != MOE_DT_FP8_E5M2 &&
+          a->weight_dtype != MOE_DT_FP4_E2M1)
         return MOE_E_BAD_ARG;
-      }
       break;
     }
   }

@@ -106,8 +106,6 @@ def _bwmm_shard_on_block_mx(
                   f"but holds {guw.numel()} bytes")
     kernel_assert(dw.numel() == E * pI * nI * H * wbytes,
                   f"down_proj_weight must be x4 [E={E}, {pI}, {nI}, {H}] of {wbytes}-byte elements but holds {dw.numel()} bytes")
-    kernel_assert(wdt == nv.DT_FP8 or (H % 512 == 0 and I % 128 == 0),
-                  f"e5m2 / MXFP4 weights need I % 128 == 0 on gfx950, found I={I}")
     kernel_assert(tuple(ds.shape) == (E, (pI + 7) // 8, nI, H),
                   f"down_proj_scale must be [{E}, {(pI + 7) // 8}, {nI}, {H}] but got {tuple(ds.shape)}")
     if gate_and_up_proj_bias is not None:

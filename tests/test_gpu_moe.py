@@ -558,6 +558,20 @@ def test_mx_reference_table(H, T, I, E, B, k, act, fmt, skip, dynamic, uint):
     _check(o[0, :rows], g[:rows], f"mx table H={H} I={I} E={E} B={B} {fmt}")
 
 
+@pytest.mark.parametrize("fmt", ["e5m2", "e2m1"])
+@pytest.mark.parametrize("I,B,uint", [(96, 128, False), (544, 256, True), (160, 128, True), (1056, 128, False)])
+def test_mx_weight_formats_outside_the_large_tile_shapes(fmt, I, B, uint):
+    """e5m2 and MXFP4 weights where I is not a multiple of 128 (the reference takes any I % 16 == 0 whose tail past a
+    multiple of 512 is a multiple of 32, bwmm_shard_on_block_mx.py:620-633): the general tiled kernel, with the
+    reference table's options (Swish, bias, clamps)."""
+    T, H, E, k = 256, 1024, 8, 2
+    c = mx_case(T, H, I, E, k, B, seed=41, bias=True, weight_format=fmt, random_codes=True)
+    out = _run_mx_options(c, 3, REF_MX_CLAMPS, uint)
+    o = from_bf16_tensor(out)
+    assert o.shape[0] == 2 and not o[1].any() and not o[0, T].any()
+    _check(o[0, :T], _golden_mx_options(c, 3, REF_MX_CLAMPS)[:T], f"mx general kernel I={I} B={B} {fmt}")
+
+
 @pytest.mark.parametrize("I", [512, 96, 544])  # large-tile kernels; general tiled kernel (I % 128 != 0), with a tail tile
 @pytest.mark.parametrize(
     "act,clamps",
