@@ -9,7 +9,7 @@ GEMM with fused affinity scaling, and the per-token combine into bf16 rows.
 Default workload: BASELINE config 4, DeepSeek-V3-shaped routed experts (T=8192, H=7168, I=2048,
 E=256, top-8, block 128, MXFP8 weights ~11 GB).  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c5-<T>|c2] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c5-<T>|c2|bf16] [--no-cpu-baseline]
 
 `--workload c2` times BASELINE config 2 instead (fp8 activations with a per-row scale from RMSNorm-Quant, fp8
 weights with per-channel scales, Mixtral-8x7B shape) through the same entry points.
@@ -29,10 +29,35 @@ for _p in (ROOT, os.path.join(ROOT, "nki-library_amd")):
 
 METRIC = "MoE layer TFLOP/s and tokens/s (fp8/MXFP8), % of MFMA peak, 1x MI355X"
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 / MXFP8 MFMA peak
+PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the gate/up kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, scaled by
-# the copy-kernel calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); see profiles/ for the runs they come from.
-MEASURED_TRAFFIC = {("c4", "router"): 8530000000}
+# the copy-kernel calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  The figure is read from the profile summary
+# that holds the runs it comes from, and only while the kernel sources still hash to what that summary was taken
+# from: a kernel changed since then has no measured traffic until it is profiled again.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "mx_gemm_c4_moe_layer.md")
+TRAFFIC_SOURCES = ("nki-library_amd/csrc/bwmm_mx.hip", "nki-library_amd/csrc/bwmm.hpp")
+
+
+def profiled_traffic(workload, routing):
+    import hashlib
+    import re
+
+    if (workload, routing) != ("c4", "router") or not os.path.exists(TRAFFIC_PROFILE):
+        return None
+    text = open(TRAFFIC_PROFILE).read()
+    sha = re.search(r"sha256 of [^:]*: `([0-9a-f]{64})`", text)
+    val = re.search(r"traffic_bytes_per_launch: (\d+)", text)
+    if not sha or not val:
+        return None
+    h = hashlib.sha256()
+    for f in TRAFFIC_SOURCES:
+        h.update(open(os.path.join(ROOT, f), "rb").read())
+    if h.hexdigest() != sha.group(1):
+        return None
+    # the clock the part held during the profiled gate/up launches (GRBM_GUI_ACTIVE over the launch time)
+    ghz = re.search(r"`mx_gemm_kernel<1, 0>` \|[^\n]*\| ([0-9.]+) GHz \|", text)
+    return int(val.group(1)), (float(ghz.group(1)) if ghz else None)
 
 
 def parse_args():
@@ -134,7 +159,9 @@ def cpu_baseline(cfg, t, tp2id, b2e, n_blocks):
 
 
 def bench_fp8_row(args):
-    """BASELINE config 2: RMSNorm-Quant (fp8 rows + fp32 row scale) -> block build -> fp8-row blockwise layer."""
+    """BASELINE config 2: RMSNorm-Quant (fp8 rows + fp32 row scale) -> block build -> fp8-row blockwise layer.
+    `--workload bf16` runs the same stages on the bf16 kind (bf16 hidden states and weights, no front end, no row
+    re-quantisation) at T=4096 H=2048 I=4096 E=8 top-2: a diagnostic for the general tiled kernel."""
     import numpy as np
     import torch
     from nkilib import _native as nv
@@ -146,17 +173,29 @@ def bench_fp8_row(args):
 
     dev = torch.device("cuda:0")
     nv.check(nv.lib().moe_check_device(), "device check")
-    cfg = dict(syn.CONFIGS["c2"])
+    bf16 = args.workload == "bf16"
+    cfg = dict(T=4096, H=2048, I=4096, E=8, k=2, B=128) if bf16 else dict(syn.CONFIGS["c2"])
     T, H, I, E, k, B = (cfg[x] for x in ("T", "H", "I", "E", "k", "B"))
-    gu_q, gu_s, d_q, d_s = syn.fp8_channel_weights(E, H, I, 0.02, dev, seed=0)
+    if bf16:
+        g = torch.Generator(device=dev)
+        g.manual_seed(0)
+        gu_w = (torch.randn((E, H, 2, I), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        d_w = (torch.randn((E, I, H), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        gu_q = gu_s = d_q = d_s = None
+    else:
+        gu_q, gu_s, d_q, d_s = syn.fp8_channel_weights(E, H, I, 0.02, dev, seed=0)
     ids, aff = syn.route(T, E, k, dev, seed=0, mode="softmax")
     x = syn.hidden_states(T, H, dev, seed=0)
     gamma = torch.ones((1, H), dtype=torch.bfloat16, device=dev)
     N = get_n_blocks(T, k, E, B)
     spec = MoECTESpec(implementation=MoECTEImplementation.shard_on_block)
-    qcfg = QuantizationConfig(gu_s, d_s)
-    gu8, d8 = gu_q.view(torch.float8_e4m3fn), d_q.view(torch.float8_e4m3fn)
-    names = ["norm_quant", "build_blocks", "prep", "gate_up", "requant", "down", "combine"]
+    if bf16:
+        kw, gu8, d8 = {}, gu_w, d_w
+        names = ["norm_quant", "build_blocks", "prep", "gate_up", "down", "combine"]
+    else:
+        kw = {"quantization_config": QuantizationConfig(gu_s, d_s)}
+        gu8, d8 = gu_q.view(torch.float8_e4m3fn), d_q.view(torch.float8_e4m3fn)
+        names = ["norm_quant", "build_blocks", "prep", "gate_up", "requant", "down", "combine"]
     events = []
 
     def rec():
@@ -168,14 +207,14 @@ def bench_fp8_row(args):
         if timed:
             events.append([])
             rec()
-        recs = rmsnorm_quant_kernel(x, gamma, RmsNormQuantKernelArgs())
+        recs = x if bf16 else rmsnorm_quant_kernel(x, gamma, RmsNormQuantKernelArgs())
         if timed:
             rec()
         tp2id, b2e, cond = build_token_blocks(ids, E, B, N)
         if timed:
             rec()
         _launch.stage_callback = (lambda name: rec()) if timed else None
-        out = moe_cte[2](recs, aff.reshape(-1, 1), gu8, d8, tp2id, b2e, B, spec, quantization_config=qcfg)
+        out = moe_cte[2](recs, aff.reshape(-1, 1), gu8, d8, tp2id, b2e, B, spec, **kw)
         _launch.stage_callback = None
         return out, recs, tp2id, b2e
 
@@ -198,28 +237,36 @@ def bench_fp8_row(args):
     gu_tflops = flops_gu / (stage_ms["gate_up"] * 1e-3) / 1e12
     # gate/up GEMM: the K-contiguous fp8 weights once (they are made on the first call and kept), the routed fp8
     # rows with their scale, the fp32 intermediate written
-    gu_bytes = E * 2 * H * I + routed * (H + 4) + routed * I * 4
-    roofline = {"bound": "mfma", "achieved": round(gu_tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(gu_tflops / PEAK_FP8_TFLOPS, 4), "traffic": None,
-                "kernel": "moe::bwmm_kernel<1, 1> (gate/up blockwise GEMM of the fp8-row kind with fused act*up, on the "
-                          "K-contiguous weight copies kept from the first call)",
+    # (bf16 kind: bf16 weights and rows, bf16 intermediate)
+    gu_bytes = (E * 2 * H * I * 2 + routed * H * 2 + routed * I * 2) if bf16 else (
+        E * 2 * H * I + routed * (H + 4) + routed * I * 4)
+    peak = PEAK_BF16_TFLOPS if bf16 else PEAK_FP8_TFLOPS
+    roofline = {"bound": "mfma", "achieved": round(gu_tflops, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(gu_tflops / peak, 4), "traffic": None,
+                "kernel": ("moe::bwmm_kernel<0, 1> (gate/up blockwise GEMM of the bf16 kind" if bf16 else
+                           "moe::bwmm_kernel<1, 1> (gate/up blockwise GEMM of the fp8-row kind") +
+                          " with fused act*up, on the K-contiguous weight copies kept from the first call)",
                 "algorithmic_bytes": int(gu_bytes), "algorithmic_flops": int(flops_gu),
                 "avg_launch_ms": round(stage_ms["gate_up"], 4)}
     res = {
         "metric": METRIC, "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "fp8_e4m3 (per-row activation scale, per-channel weight scale, fp32 accumulate)",
+        "vs_baseline": None,
+        "dtype": "bf16 (fp32 accumulate)" if bf16 else
+                 "fp8_e4m3 (per-row activation scale, per-channel weight scale, fp32 accumulate)",
         "data": "synthetic",
-        "config": {"workload": f"c2: fp8-row blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} (N={N} blocks, "
-                               f"{routed} routed rows), RMSNorm-Quant front end + block build + gate/up + row re-quantise "
-                               f"+ down + combine",
+        "config": {"workload": (f"bf16: bf16 blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} (N={N} blocks, "
+                                f"{routed} routed rows), block build + gate/up + down + combine" if bf16 else
+                                f"c2: fp8-row blockwise MoE layer T={T} H={H} I={I} E={E} top-{k} B={B} (N={N} blocks, "
+                                f"{routed} routed rows), RMSNorm-Quant front end + block build + gate/up + row "
+                                f"re-quantise + down + combine"),
                    "T": T, "H": H, "I": I, "E": E, "top_k": k, "block_size": B},
         "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
-        "pct_of_fp8_mfma_peak": round(100.0 * tflops / PEAK_FP8_TFLOPS, 2),
+        "pct_of_mfma_peak": round(100.0 * tflops / peak, 2),
         "stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
         "roofline": roofline,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not bf16:
         from oracle import moe as omoe
 
         tpb = tp2id.cpu().numpy().reshape(-1, B)
@@ -251,7 +298,7 @@ def main():
         print(f"bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
-    if args.workload == "c2":
+    if args.workload in ("c2", "bf16"):
         return bench_fp8_row(args)
     import torch
 
@@ -346,7 +393,8 @@ def main():
     gu_s = stage_ms["gate_up"] * 1e-3
     floor_mfma = flops_gate_up / (PEAK_FP8_TFLOPS * 1e12)
     floor_hbm = gu_bytes / (PEAK_HBM_GBS * 1e9)
-    measured = None if fp4 else MEASURED_TRAFFIC.get((args.workload, args.routing))
+    prof = None if fp4 else profiled_traffic(args.workload, args.routing)
+    measured, sclk_ghz = prof if prof else (None, None)
     if floor_hbm >= floor_mfma:
         roofline = {"bound": "hbm", "achieved": round(gu_bytes / gu_s / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(gu_bytes / gu_s / 1e9 / PEAK_HBM_GBS, 4)}
@@ -362,6 +410,10 @@ def main():
         "frac_of_mfma_peak": round(gate_up_tflops / PEAK_FP8_TFLOPS, 4),
         "frac_of_hbm_peak": round(gu_bytes / gu_s / 1e9 / PEAK_HBM_GBS, 4),
     })
+    if sclk_ghz:
+        # 256 CUs x 4 SIMDs, one 16x16x128 MFMA (65536 flop) per 32 cycles and SIMD
+        roofline["sclk_ghz_profiled"] = sclk_ghz
+        roofline["mfma_peak_at_that_clock_TFLOPs"] = round(1024 * 2048 * sclk_ghz / 1e3, 1)
 
     res = {
         "metric": METRIC,
