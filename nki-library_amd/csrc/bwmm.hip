@@ -691,6 +691,67 @@ int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C,
   return MOE_OK;
 }
 
+// One thread per x4 element (four K values of one output column).
+__global__ __launch_bounds__(256) void relayout_gu_x4_kernel(const uint8_t* __restrict__ W, uint32_t* __restrict__ X,
+                                                             int64_t H, int64_t I, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t nH = H / 512;
+  const int64_t i = idx % I, t = (idx / I) % nH, gu = (idx / (I * nH)) % 2, p = (idx / (I * nH * 2)) % 128,
+                e = idx / (I * nH * 2 * 128);
+  const int64_t h = t * 512 + p * 4;
+  uint32_t v = 0;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) v |= (uint32_t)W[((e * H + h + q) * 2 + gu) * I + i] << (8 * q);
+  X[idx] = v;
+}
+__global__ __launch_bounds__(256) void relayout_down_x4_kernel(const uint8_t* __restrict__ W, uint32_t* __restrict__ X,
+                                                               int64_t H, int64_t I, int64_t I_pad, int64_t pI,
+                                                               int64_t nI, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t h = idx % H, t = (idx / H) % nI, p = (idx / (H * nI)) % pI, e = idx / (H * nI * pI);
+  const int64_t i0 = t * 512 + p * 4;
+  uint32_t v = 0;
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    if (i0 + q < I) v |= (uint32_t)W[(e * I_pad + i0 + q) * H + h] << (8 * q);
+  X[idx] = v;
+}
+__global__ __launch_bounds__(256) void fill_bytes_kernel(uint32_t* __restrict__ p, int64_t words, uint32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < words) p[i] = v;
+}
+
+int launch_fill_bytes(void* p, size_t bytes, uint8_t value, hipStream_t s) {
+  if (bytes == 0) return MOE_OK;
+  if ((bytes & 3) != 0 || ((uintptr_t)p & 3) != 0) return MOE_E_BAD_ARG;
+  const int64_t words = (int64_t)(bytes / 4);
+  hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, (uint32_t*)p, words,
+                     0x01010101u * value);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
+int launch_relayout_x4(const uint8_t* gate_up, const uint8_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
+                       int64_t I, int64_t I_pad, hipStream_t s) {
+  if ((((uintptr_t)dst) & 3) != 0) return MOE_E_BAD_ARG;
+  if (which == 0) {
+    const int64_t total = E * 128 * 2 * (H / 512) * I;
+    if ((total + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
+    hipLaunchKernelGGL(relayout_gu_x4_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gate_up,
+                       (uint32_t*)dst, H, I, total);
+  } else {
+    const int64_t nI = (I + 511) / 512, pI = I > 512 ? 128 : I / 4;
+    const int64_t total = E * pI * nI * H;
+    if ((total + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
+    hipLaunchKernelGGL(relayout_down_x4_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, down,
+                       (uint32_t*)dst, H, I, I_pad, pI, nI, total);
+  }
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
+
 template <int KIND, int STAGE>
 static int launch_gemm(const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s) {
   if (gx == 0 || gy == 0) return MOE_OK;

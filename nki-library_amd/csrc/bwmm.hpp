@@ -69,9 +69,21 @@ struct MxArgs {
   float clamp[4];
   int32_t col_tiles;       // column tiles per chunk (set by the launcher)
   int32_t wfmt;            // element format of the weights, MX_WFMT_*
+  int32_t chunk_interleave;  // chunks whose column tiles alternate in a class's item order, see chunk_interleave_for
+  // MX_WFMT_ROW8 (the fp8-row kind on these kernels): e4m3 operands whose E8M0 tables are constants of 127, a
+  // per-row fp32 scale of the activations and a per-output-channel fp32 scale of the weights in the epilogue
+  const float* w_cscale;   // [cscale_experts][2*I] (gate/up: gate then up) or [cscale_experts][H] (down)
+  int32_t cscale_experts;  // E or 1
+  int32_t w_scale_shared;  // 1: W_scale holds one expert's worth of block scales that serves every expert
+  const float* a_rscale;   // stage 2: row scale of the re-quantised intermediate, [N*B]; stage 1: null, a row's scale
+                           // is the fp32 behind its H codes (the RMSNorm-Quant ROW record)
+  int64_t a_scale_bytes;   // size of the A_scale table when it is not a_rows * a_scale_stride (stride 0: one row
+                           // of constants for every row)
+  float* Y32;              // stage 1 output of this format: fp32 [N*B, y32_stride], columns in natural order
+  int64_t y32_stride;
 };
 
-constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1, MX_WFMT_E2M1 = 2;
+constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1, MX_WFMT_E2M1 = 2, MX_WFMT_ROW8 = 3;
 
 // True when the large-tile kernels cover the shape: every intermediate tile holds a multiple
 // of 32 partitions (I % 128 == 0); other shapes run the general kernel.
@@ -85,6 +97,12 @@ int launch_transpose_w16(const void* src, int w8, uint16_t* dst, int64_t R, int6
                          int64_t nb0, int nb1, int64_t src_bs0, int64_t src_bs1, hipStream_t s);
 int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C, int64_t src_row_stride, int64_t Kp,
                          int64_t nb0, int nb1, int64_t src_bs0, int64_t src_bs1, hipStream_t s);
+// The fp8-row kind's weights in the x4 order the large-tile kernels read, K in natural order: gate/up
+// [E, H, 2, I] -> [E, 128 (p), 2, H/512 (t), I, 4 (q)] with h = t*512 + p*4 + q; down [E, I_pad, H] ->
+// [E, pI, nI, H, 4] with i = t*512 + p*4 + q (zeros past I).
+int launch_relayout_x4(const uint8_t* gate_up, const uint8_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
+                       int64_t I, int64_t I_pad, hipStream_t s);
+int launch_fill_bytes(void* p, size_t bytes, uint8_t value, hipStream_t s);
 int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,
                        int64_t Iw, hipStream_t s);
 

@@ -272,9 +272,16 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // requested before an epilogue, put in place after it.
 template <int STAGE, int NMT, bool LASTUSE, int WFMT>
 __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int (*s_tok)[MX_ROWS_MAX],
-                                             float (*s_aff)[MX_ROWS_MAX], float (*s_bias)[MXT], int L, const int endL,
-                                             const int Lstep, const int qbase) {
+                                             float (*s_aff)[MX_ROWS_MAX], float (*s_bias)[MXT],
+                                             float (*s_rs)[MX_ROWS_MAX], float (*s_wsc)[MXT], int L, const int startL,
+                                             const int endL, const int Lstep, const int qbase) {
   using Cfg = MxCfg<NMT>;
+  // ROW8: the fp8-row kind.  Same K loop on e4m3 operands with block scales of 2^0; what differs is the epilogue
+  // (per-channel weight scale x per-row activation scale ahead of the bias, bias and scales indexed by natural
+  // column, gate/up results written as fp32 rows for the per-row re-quantisation pass) and two more row / column
+  // tables (s_rs, s_wsc: null for the MX formats).
+  constexpr bool ROW8 = WFMT == MX_WFMT_ROW8;
+  constexpr int MFMT = ROW8 ? MX_WFMT_E4M3 : WFMT;  // element format of the MFMA's B operand
   constexpr int D = Cfg::D, RING = Cfg::RING, SA = Cfg::SA, SS = Cfg::SS, SSP = Cfg::SSP;
   constexpr bool BIG = NMT > 16;  // row tiles 16.. accumulate in ordinary registers
   uint8_t* sA = smem;
@@ -298,13 +305,31 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     int nrows, e, slot0, xt;
   };
   typedef int v2i_t __attribute__((ext_vector_type(2)));
+  // Item l of the class -> (chunk position, column tile).  G = a.chunk_interleave chunks at a time: within a
+  // group of G queue positions the chunk varies fastest, so that workgroups with neighbouring items work on the
+  // same column tile of different chunks (of one expert: they share the weight tile); G = 1 is column tiles
+  // innermost.  The last group of a class may hold fewer than G chunks.
+  // (items are numbered through the XCD's whole queue; the class's own run from startL to endL)
+  const int pos0 = startL / a.col_tiles, npos = (endL - startL) / a.col_tiles;
   auto tile_at = [&](int l) {
-    const int pos = l / a.col_tiles;
+    int pos, xt;
+    if (a.chunk_interleave == 1) {
+      pos = l / a.col_tiles;
+      xt = l - pos * a.col_tiles;
+    } else {
+      const int per_group = a.chunk_interleave * a.col_tiles;
+      const int lr = l - startL;
+      const int grp = lr / per_group, j = lr - grp * per_group;
+      const int base = grp * a.chunk_interleave;
+      const int G = (npos - base < a.chunk_interleave) ? npos - base : a.chunk_interleave;
+      xt = j / G;
+      pos = pos0 + base + (j - xt * G);
+    }
     v2i_t raw;
     asm volatile(MX_SGPR_WAIT "s_load_dwordx2 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
                  : "=s"(raw) : "s"(a.q_chunk), "s"((qbase + pos) * 8) : "memory");
     Tile t;
-    t.xt = l - pos * a.col_tiles;
+    t.xt = xt;
     t.slot0 = raw[0];
     t.nrows = raw[1] & 0xffff;
     t.e = raw[1] >> 16;
@@ -375,7 +400,17 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   };
   // gate/up: bias value (gu*4 + q)*32 + pl belongs to partition p0 + pl; down: value j to column h0 + j.
   const int hcol = (STAGE == 1) ? (c >> 3) : 0, cl = (STAGE == 1) ? (c & 7) : c;
+  // the natural column of the thread's table entry: gate/up (gu = tid/128, q = tid/32 % 4, pl = tid % 32) ->
+  // gu * I + tile*512 + q*Pt + p0 + pl; down -> h0 + tid
+  auto natural_col = [&](const Tile& t) {
+    if (STAGE == 1)
+      return (uint32_t)(tid >> 7) * (uint32_t)a.I + (uint32_t)tile_tI(t) * 512u +
+             (uint32_t)((tid >> 5) & 3) * (uint32_t)tile_Pt(t) + (uint32_t)(tile_p0(t) + (tid & 31));
+    return (uint32_t)tile_h0(t) + (uint32_t)tid;
+  };
+  const uint32_t ncols = (STAGE == 1) ? 2u * (uint32_t)a.I : (uint32_t)a.H;  // table entries per expert
   auto bias_index = [&](const Tile& t) {
+    if (ROW8) return (uint32_t)t.e * ncols + natural_col(t);
     if (STAGE == 1) {
       const uint32_t p = (uint32_t)(tile_p0(t) + (tid & 31));
       return ((((uint32_t)t.e * (uint32_t)a.pI + p) * 2u + (uint32_t)(tid >> 7)) * (uint32_t)a.nI + (uint32_t)tile_tI(t)) * 4u +
@@ -390,10 +425,58 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   auto bias_put = [&](const Tile& t, int buf, int raw) {
     s_bias[buf][tid] = a.bias ? elem_value(raw, bias_index(t), a.bias_dtype == MOE_DT_BF16) : 0.f;
   };
+  // ROW8: the weights' per-channel scale of the thread's column (fp32), and the activation rows' scales: gate/up,
+  // the fp32 behind the H codes of the token's record, times the affinity under PRE_SCALE (the affinity scales
+  // the token's row, i.e. its dequantisation scale); down, the scale of the re-quantised intermediate row.
+  auto wsc_raw = [&](const Tile& t, int& raw) {
+    if constexpr (ROW8) {
+      const v4i rd = make_rsrc(a.w_cscale, 0xffffffffu);
+      ld_b32(raw, ((a.cscale_experts > 1 ? (uint32_t)t.e * ncols : 0u) + natural_col(t)) << 2, rd, 0);
+    }
+  };
+  auto wsc_put = [&](int buf, int raw) {
+    if constexpr (ROW8) s_wsc[buf][tid] = __builtin_bit_cast(float, raw);
+  };
+  auto rs_raw = [&](const Tile& t, int buf, int (&raw)[2]) {
+    if constexpr (ROW8) {
+      const v4i rd = make_rsrc((STAGE == 1) ? (const void*)a.A : (const void*)a.a_rscale, 0xffffffffu);
+#pragma unroll
+      for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
+        const int r = tid + 256 * j;
+        uint32_t off;
+        if (STAGE == 1) {
+          const int id = s_tok[buf][(r < NMT * 16) ? r : 0];
+          off = (uint32_t)((id >= 0) ? id : 0) * (uint32_t)a.a_stride + (uint32_t)a.H;
+        } else {
+          off = (uint32_t)(t.slot0 + ((r < t.nrows) ? r : t.nrows - 1)) << 2;
+        }
+        ld_b32(raw[j], off, rd, 0);
+      }
+    }
+  };
+  // (gate/up under PRE_SCALE: `aff` holds what aff_raw fetched for the same rows)
+  auto rs_put = [&](int e, int buf, const int (&raw)[2], const int (&aff)[2]) {
+    if constexpr (ROW8) {
+      const bool pre = STAGE == 1 && (a.scaling_mode == MOE_SCALE_PRE || a.scaling_mode == MOE_SCALE_PRE_DELAYED);
+#pragma unroll
+      for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
+        const int r = tid + 256 * j;
+        if (r < NMT * 16) {
+          float v = __builtin_bit_cast(float, raw[j]);
+          if (STAGE == 1 && s_tok[buf][r] < 0) v = 0.f;
+          if (pre && a.aff && s_tok[buf][r] >= 0) v *= elem_value(aff[j], aff_index(e, buf, r), a.aff_dtype == MOE_DT_BF16);
+          s_rs[buf][r] = v;
+        }
+      }
+    }
+  };
+  // which stages fetch the affinities: down always; gate/up of the fp8-row kind, for PRE_SCALE
+  constexpr bool AFF_ROWS = STAGE == 2 || ROW8;
   // what has been requested with the *_raw functions above may be used once this has passed
-  auto all_loads_landed = [&](int (&x)[2], int (&y)[2], int& z) {
+  auto all_loads_landed = [&](int (&x)[2], int (&y)[2], int& z, int (&u)[2], int& v) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(y[0]), "+v"(y[1]), "+v"(z));
+    if constexpr (ROW8) asm volatile("" : "+v"(u[0]), "+v"(u[1]), "+v"(v));
   };
 
   // A staging: thread covers rows (tid>>3) + 32 j; its load goes straight to LDS slot tid&7 of that
@@ -440,7 +523,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // 4-bit weights (x4: four K values in a 2-byte element): lane group g needs K 32g .. 32g+31 of the
   // slice = partitions 8g .. 8g+7, one 8-byte load (4 columns) per partition; 8-bit weights (4-byte
   // elements): partitions 4g .. 4g+3 and 16+4g .. 16+4g+3, one 16-byte load each.
-  constexpr bool FP4 = WFMT == 2;
+  constexpr bool FP4 = WFMT == MX_WFMT_E2M1;
   constexpr int ES = FP4 ? 2 : 4;      // bytes of a weight element
   constexpr int GROWS = FP4 ? 8 : 4;   // partition rows between the lane groups' first rows
   const uint8_t* Wb = (const uint8_t*)a.W;
@@ -472,7 +555,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     int sc;
   };
   v4i ra_ = make_rsrc(a.A, (STAGE == 1) ? 0xffffffffu : (uint32_t)(a.a_rows * a.a_stride)),
-      ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_rows * a.a_scale_stride));
+      ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_scale_bytes ? a.a_scale_bytes : a.a_rows * a.a_scale_stride));
   const int ra_rec = ra_[2], ras_rec = ras_[2];
   int rw_rec = 0, rs_rec = 0;
   const int a_group_bytes = uni((int)(32 * a.a_stride));  // down stage: bytes between row groups of 32 slots
@@ -509,12 +592,12 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     if (STAGE == 1) {
       colu = (int64_t)tile_tI(t) * 512 + (int64_t)q * tile_Pt(t) + tile_p0(t);
       rw_ = make_rsrc(Wb + (int64_t)t.e * 128 * w_pstride * ES, (uint32_t)(128 * w_pstride * ES));
-      rs_ = make_rsrc(a.W_scale + (int64_t)t.e * 16 * w_pstride, (uint32_t)(16 * w_pstride));
+      rs_ = make_rsrc(a.W_scale + (int64_t)(a.w_scale_shared ? 0 : t.e) * 16 * w_pstride, (uint32_t)(16 * w_pstride));
     } else {
       colu = tile_h0(t) + 64 * q;
       const int64_t sp = (a.pI + 7) / 8;
       rw_ = make_rsrc(Wb + (int64_t)t.e * a.pI * w_pstride * ES, (uint32_t)(a.pI * w_pstride * ES));
-      rs_ = make_rsrc(a.W_scale + (int64_t)t.e * sp * w_pstride, (uint32_t)(sp * w_pstride));
+      rs_ = make_rsrc(a.W_scale + (int64_t)(a.w_scale_shared ? 0 : t.e) * sp * w_pstride, (uint32_t)(sp * w_pstride));
     }
     rw_rec = rw_[2];
     rs_rec = rs_[2];
@@ -678,9 +761,9 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
         constexpr int mt = 2 * gi + j / 4, nt = j % 4;
         constexpr int m = gi * 8 + j;  // MFMA number within the slice
         if constexpr (mt < 16)
-          mfma_asm<16 * mt + 4 * nt, mt % 4, nt, WFMT>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
+          mfma_asm<16 * mt + 4 * nt, mt % 4, nt, MFMT>(af[cur][j / 4], b.f[nt], asc[mt / 4], b.sc);
         else
-          mfma_asm_v<mt % 4, nt, WFMT>(accv[mt - 16][nt], af[cur][j / 4], b.f[nt], asc_hi, b.sc);
+          mfma_asm_v<mt % 4, nt, MFMT>(accv[mt - 16][nt], af[cur][j / 4], b.f[nt], asc_hi, b.sc);
         if constexpr (m == 0) {
           // the scalar arithmetic for the addresses of slice ks+D starts here, behind the first
           // MFMA, instead of ahead of it
@@ -716,16 +799,21 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // ---- first tile: nothing is in flight yet, so plain loads and waits do ----------------------------------
   Tile cur = tile_at(L);
   int ids_nn[2] = {0, 0}, aff_n[2] = {0, 0}, bias_n = 0;  // requested ahead of an epilogue, put in place after it
+  int rs_n[2] = {0, 0}, wsc_n = 0;                          // (fp8-row kind only)
   ids_raw(cur, ids_nn);
   bias_raw(cur, bias_n);
-  all_loads_landed(ids_nn, aff_n, bias_n);
+  wsc_raw(cur, wsc_n);
+  all_loads_landed(ids_nn, aff_n, bias_n, rs_n, wsc_n);
   ids_put(0, cur.nrows, ids_nn);
   bias_put(cur, 0, bias_n);
+  wsc_put(0, wsc_n);
   __syncthreads();
-  if (STAGE == 2) {
+  if (AFF_ROWS) {
     aff_raw(cur, 0, aff_n);
-    all_loads_landed(ids_nn, aff_n, bias_n);
-    aff_put(cur.e, 0, aff_n);
+    rs_raw(cur, 0, rs_n);
+    all_loads_landed(ids_nn, aff_n, bias_n, rs_n, wsc_n);
+    if (STAGE == 2) aff_put(cur.e, 0, aff_n);
+    rs_put(cur.e, 0, rs_n, aff_n);
   }
   aim_loads_at(cur, 0);
   request_first_slices();
@@ -735,7 +823,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     // (the wait in here also waits for the first slices: once per workgroup and class)
     const Tile nx = tile_at(have_next ? Ln : L);
     ids_raw(nx, ids_nn);
-    all_loads_landed(ids_nn, aff_n, bias_n);
+    all_loads_landed(ids_nn, aff_n, bias_n, rs_n, wsc_n);
     if (have_next) ids_put(1, nx.nrows, ids_nn);  // published by the barrier below
   }
   int buf = 0;  // which of the two row tables (s_tok, s_aff, s_bias) belongs to the current tile
@@ -795,8 +883,10 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   aim_loads_at(nxt, nbuf);
   request_first_slices();
   tile_live = -1;
-  if (STAGE == 2) aff_raw(nxt, nbuf, aff_n);
+  if (AFF_ROWS) aff_raw(nxt, nbuf, aff_n);
+  rs_raw(nxt, nbuf, rs_n);
   bias_raw(nxt, bias_n);
+  wsc_raw(nxt, wsc_n);
   ids_raw(nn, ids_nn);
 
   // ---- epilogue ---------------------------------------------------------------------------------------------
@@ -820,6 +910,12 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       const float4 vg = *(const float4*)(s_bias[buf] + q * 32 + 4 * cl_e), vu = *(const float4*)(s_bias[buf] + 128 + q * 32 + 4 * cl_e);
       bg[0] = vg.x; bg[1] = vg.y; bg[2] = vg.z; bg[3] = vg.w;
       bu[0] = vu.x; bu[1] = vu.y; bu[2] = vu.z; bu[3] = vu.w;
+    }
+    float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};  // fp8-row kind: the columns' weight scales
+    if constexpr (ROW8) {
+      const float4 vg = *(const float4*)(s_wsc[buf] + q * 32 + 4 * cl_e), vu = *(const float4*)(s_wsc[buf] + 128 + q * 32 + 4 * cl_e);
+      sg[0] = vg.x; sg[1] = vg.y; sg[2] = vg.z; sg[3] = vg.w;
+      su[0] = vu.x; su[1] = vu.y; su[2] = vu.z; su[3] = vu.w;
     }
     const int pl0 = 4 * cl_e;
     constexpr int NPS = NMT / 4;
@@ -857,6 +953,11 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
             else av[i / 4][i % 4] = accv[mt - 16][i / 4][i % 4];
           });
           float y[2][4];
+          float rsk[2] = {1.f, 1.f};  // fp8-row kind: the scales of the lane's two rows
+          if constexpr (ROW8) {
+            const float2 rr = *(const float2*)(s_rs[buf] + ps * 64 + ml * 16 + 4 * g_e + 2 * hcol_e);
+            rsk[0] = rr.x; rsk[1] = rr.y;
+          }
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -866,7 +967,11 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
               const float send = hcol_e ? lo : hi;
               const float recv = __builtin_bit_cast(
                   float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
-              const float gv = hcol_e ? recv : mine, uv = hcol_e ? mine : recv;
+              float gv = hcol_e ? recv : mine, uv = hcol_e ? mine : recv;
+              if constexpr (ROW8) {
+                gv = (gv * sg[t]) * rsk[k];
+                uv = (uv * su[t]) * rsk[k];
+              }
               const float gg = fminf(fmaxf(gv + bg[t], g_lo), g_hi);
               const float uu = fminf(fmaxf(uv + bu[t], u_lo), u_hi);
               y[k][t] = act_apply(gg, ACT) * uu;
@@ -882,7 +987,19 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
         // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 32 (x 4 q)
         const int rl = tid_e >> 2, j = tid_e & 3;
         const int row = ps * 64 + rl;
-        if (row < cur.nrows) {
+        if (ROW8 && row < cur.nrows) {
+          // fp32 rows in natural column order: the thread's 4 x 8 values are four runs of 8 columns
+          const float* src = E + rl * MX_EP + 8 * j;
+          float* dst = a.Y32 + (int64_t)(cur.slot0 + row) * a.y32_stride + tile_tI(cur) * 512 + tile_p0(cur) + 8 * j;
+          const int Pt = tile_Pt(cur);
+#pragma unroll
+          for (int qq = 0; qq < 4; ++qq) {
+            const float4 lo = *(const float4*)(src + qq * 32), hi = *(const float4*)(src + qq * 32 + 4);
+            *(float4*)(dst + qq * Pt) = lo;
+            *(float4*)(dst + qq * Pt + 4) = hi;
+          }
+        }
+        if (!ROW8 && row < cur.nrows) {
           const float* src = E + rl * MX_EP + 8 * j;
           float yv[4][8];
           float am = 0.f;
@@ -925,6 +1042,11 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       const float4 vb = *(const float4*)(s_bias[buf] + 64 * q + 4 * c_e);
       bd[0] = vb.x; bd[1] = vb.y; bd[2] = vb.z; bd[3] = vb.w;
     }
+    float sd[4] = {1.f, 1.f, 1.f, 1.f};  // fp8-row kind: the columns' weight scales
+    if constexpr (ROW8) {
+      const float4 vs = *(const float4*)(s_wsc[buf] + 64 * q + 4 * c_e);
+      sd[0] = vs.x; sd[1] = vs.y; sd[2] = vs.z; sd[3] = vs.w;
+    }
     const bool post = a.scaling_mode == MOE_SCALE_POST;
     // Rows go out through a descriptor that ends after the chunk's last row, so rows past the end
     // are dropped by the range check and the stores need no branches.  (Rows of padding slots
@@ -939,9 +1061,15 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     v4f aff_q[3];
     aff_q[0] = *(const v4f*)(s_aff[buf] + 0 * 16 + 4 * g_e);
     aff_q[1] = *(const v4f*)(s_aff[buf] + 1 * 16 + 4 * g_e);
+    v4f rs_q[3];  // fp8-row kind: the rows' activation scales, read ahead the same way
+    if constexpr (ROW8) {
+      rs_q[0] = *(const v4f*)(s_rs[buf] + 0 * 16 + 4 * g_e);
+      rs_q[1] = *(const v4f*)(s_rs[buf] + 1 * 16 + 4 * g_e);
+    }
     static_for<0, NMT>([&](auto mt_) {
       constexpr int mt = decltype(mt_)::value;
       if constexpr (mt + 2 < NMT) aff_q[(mt + 2) % 3] = *(const v4f*)(s_aff[buf] + (mt + 2) * 16 + 4 * g_e);
+      if constexpr (ROW8 && mt + 2 < NMT) rs_q[(mt + 2) % 3] = *(const v4f*)(s_rs[buf] + (mt + 2) * 16 + 4 * g_e);
       const v4f aff4 = post ? aff_q[mt % 3] : (v4f){1.f, 1.f, 1.f, 1.f};
       float av[4][4];  // [column tile][row]
       static_for<0, 16>([&](auto i_) {
@@ -952,6 +1080,11 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float af = aff4[r];
+        if constexpr (ROW8) {
+          const float rs = rs_q[mt % 3][r];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) av[t][r] = (av[t][r] * sd[t]) * rs;
+        }
         v2i o;
 #pragma unroll
         for (int t = 0; t < 4; t += 2) {
@@ -967,10 +1100,12 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // Everything in flight lands here: the next tile's first slices, this tile's stores (stores and loads share
   // the counter but complete in no fixed order between them, so the K loop's counting waits must not start
   // while stores are out), and the small loads issued ahead of the epilogue, which may be used from here on.
-  all_loads_landed(ids_nn, aff_n, bias_n);
+  all_loads_landed(ids_nn, aff_n, bias_n, rs_n, wsc_n);
   if (!have_next) break;
   if (STAGE == 2) aff_put(nxt.e, buf ^ 1, aff_n);
+  rs_put(nxt.e, buf ^ 1, rs_n, aff_n);
   bias_put(nxt, buf ^ 1, bias_n);
+  wsc_put(buf ^ 1, wsc_n);
   if (have_nn) ids_put(buf, nn.nrows, ids_nn);  // the table of the tile that has just ended
   cur = nxt;
   L = Ln;
@@ -991,6 +1126,9 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   __shared__ int s_tok[2][MX_ROWS_MAX];
   __shared__ __attribute__((aligned(16))) float s_aff[2][MX_ROWS_MAX];
   __shared__ __attribute__((aligned(16))) float s_bias[2][MXT];
+  // the fp8-row kind's row and column scales (a token entry each for the other formats)
+  __shared__ __attribute__((aligned(16))) float s_rs[2][WFMT == MX_WFMT_ROW8 ? MX_ROWS_MAX : 4];
+  __shared__ __attribute__((aligned(16))) float s_wsc[2][WFMT == MX_WFMT_ROW8 ? MXT : 4];
   // One workgroup per CU, for the whole launch.  Workgroups are handed to the 8 XCDs round-robin by linear
   // index, and each XCD has its own L2.  XCD x therefore takes the x-th contiguous eighth of the chunk list
   // (chunks are ordered by expert), as a queue of items (chunk, column tile) with the column tiles innermost
@@ -1007,8 +1145,11 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // its expert", then "last"
 #define MX_RUN_CLASS(CLS_, NMT_, LAST_)                                                                        \
   {                                                                                                            \
+    const int startL = (__builtin_amdgcn_readfirstlane(qo[CLS_]) - qbase) * a.col_tiles;                       \
     const int endL = (__builtin_amdgcn_readfirstlane(qo[CLS_ + 1]) - qbase) * a.col_tiles;                     \
-    if (L < endL) L = mx_gemm_tiles<STAGE, NMT_, LAST_, WFMT>(a, smem, s_tok, s_aff, s_bias, L, endL, W, qbase);       \
+    if (L < endL)                                                                                              \
+      L = mx_gemm_tiles<STAGE, NMT_, LAST_, WFMT>(a, smem, s_tok, s_aff, s_bias, (float(*)[MX_ROWS_MAX])s_rs,  \
+                                                  (float(*)[MXT])s_wsc, L, startL, endL, W, qbase);           \
     __syncthreads();                                                                                           \
   }
   MX_RUN_CLASS(0, 20, false)
@@ -1041,6 +1182,8 @@ int launch_mx_gemm_s1_f1(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f1(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s1_f2(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f2(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s1_f3(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s2_f3(const MxArgs& m, unsigned grid, hipStream_t s);
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {
   if (gx == 0 || gy == 0) return MOE_OK;
@@ -1060,6 +1203,7 @@ int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStr
     case MX_WFMT_E4M3: return stage == 1 ? launch_mx_gemm_s1_f0(m, grid, s) : launch_mx_gemm_s2_f0(m, grid, s);
     case MX_WFMT_E5M2: return stage == 1 ? launch_mx_gemm_s1_f1(m, grid, s) : launch_mx_gemm_s2_f1(m, grid, s);
     case MX_WFMT_E2M1: return stage == 1 ? launch_mx_gemm_s1_f2(m, grid, s) : launch_mx_gemm_s2_f2(m, grid, s);
+    case MX_WFMT_ROW8: return stage == 1 ? launch_mx_gemm_s1_f3(m, grid, s) : launch_mx_gemm_s2_f3(m, grid, s);
     default: return MOE_E_BAD_ARG;
   }
 }

@@ -121,6 +121,38 @@ int validate(const moe_bwmm_args* a) {
   return MOE_OK;
 }
 
+// The fp8-row kind runs on the large-tile kernels (bwmm_mx.hip, MX_WFMT_ROW8) when the shape is one of theirs and
+// every 32-bit offset they form stays in range; otherwise on the general tiled kernel.  The choice depends on the
+// shape only, because it also decides what the kept weight copies look like.
+bool row8_fast(const moe_bwmm_args* a) {
+  if (a->kind != MOE_KIND_FP8_ROW || !mx_fast_path_ok(a->H, a->I)) return false;
+  const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
+  const int64_t slots = a->N * a->B, Iw = (a->I + 127) / 128 * 128;
+  const int64_t pI = a->I > 512 ? 128 : a->I / 4, nI = (a->I + 511) / 512;
+  if (a->T1 * (a->H + 4) >= lim32 || slots * Iw >= lim32) return false;
+  if (2 * a->H * a->I >= lim31 || pI * nI * a->H * 4 >= lim31) return false;
+  if (slots * 4 >= lim32 || a->T1 * a->E * 4 >= lim32 || a->E * 2 * a->I * 4 >= lim32 || a->E * a->H * 4 >= lim32)
+    return false;
+  return true;
+}
+// What a kept copy of the fp8-row weights holds on that path: the weights in x4 order, one expert's worth of E8M0
+// block scales of 127 (2^0) that serves every expert, and one row of activation block scales of 127.
+struct Row8Copy {
+  size_t w_scale, a_scale, a_scale_bytes, total;
+};
+Row8Copy row8_copy(const moe_bwmm_args* a, int which) {
+  auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  const size_t nH = (size_t)a->H / 512, nI = ((size_t)a->I + 511) / 512, pI = a->I > 512 ? 128 : (size_t)a->I / 4;
+  Row8Copy c;
+  const size_t w = which == 0 ? (size_t)a->E * 2 * a->H * a->I : (size_t)a->E * pI * nI * a->H * 4;
+  const size_t ws = which == 0 ? 16 * 2 * nH * (size_t)a->I : ((pI + 7) / 8) * nI * (size_t)a->H;
+  c.w_scale = al(w);
+  c.a_scale = c.w_scale + al(ws);
+  c.a_scale_bytes = al(which == 0 ? (size_t)a->H / 32 : nI * 16);
+  c.total = c.a_scale + c.a_scale_bytes;
+  return c;
+}
+
 Plan make_plan(const moe_bwmm_args* a) {
   Plan p;
   memset(&p, 0, sizeof(p));
@@ -151,8 +183,17 @@ Plan make_plan(const moe_bwmm_args* a) {
     p.ys = off; off += al256(slots * 4);
     // K-contiguous copies of the fp8 weights: [E, 2, I, Hk] and [E, H, Iw]
     p.Hk = (a->H + 127) / 128 * 128;
-    if (!a->gate_up_proj_weight_kmajor) { p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk); }
-    if (!a->down_proj_weight_kmajor) { p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw); }
+    const bool r8 = row8_fast(a);
+    if (r8) {  // the x4 geometry of the down weights, as for the MXFP8 kind
+      p.nI = (a->I + 511) / 512;
+      p.pI = a->I > 512 ? 128 : a->I / 4;
+    }
+    if (!a->gate_up_proj_weight_kmajor) {
+      p.wt1 = off; off += al256(r8 ? row8_copy(a, 0).total : (size_t)a->E * 2 * a->I * p.Hk);
+    }
+    if (!a->down_proj_weight_kmajor) {
+      p.wt2 = off; off += al256(r8 ? row8_copy(a, 1).total : (size_t)a->E * a->H * p.Iw);
+    }
   }
   p.d = off; off += al256(slots * (size_t)a->H * 2);
   p.total = off;
@@ -169,6 +210,13 @@ int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hip
                                   a->H * 2 * a->I, a->I, s);
     return launch_transpose_w16(a->down_proj_weight, w8, (uint16_t*)dst, a->I, a->H, a->H, p.Iw, a->E, 1, Ipad * a->H, 0, s);
   }
+  if (row8_fast(a)) {
+    const Row8Copy c = row8_copy(a, which);
+    int rc = launch_relayout_x4((const uint8_t*)a->gate_up_proj_weight, (const uint8_t*)a->down_proj_weight,
+                                (uint8_t*)dst, which, a->E, a->H, a->I, Ipad, s);
+    if (rc != MOE_OK) return rc;
+    return launch_fill_bytes((uint8_t*)dst + c.w_scale, c.total - c.w_scale, 127, s);
+  }
   if (which == 0)
     return launch_transpose_fp8((const uint8_t*)a->gate_up_proj_weight, (uint8_t*)dst, a->H, a->I, 2 * a->I, p.Hk, a->E, 2,
                                 a->H * 2 * a->I, a->I, s);
@@ -182,6 +230,7 @@ extern "C" size_t moe_kmajor_weights_bytes(const moe_bwmm_args* a, int which) {
   if (validate(a) != MOE_OK || a->kind == MOE_KIND_MXFP8 || which < 0 || which > 1) return 0;
   const Plan p = make_plan(a);
   const size_t es = a->kind == MOE_KIND_BF16 ? 2 : 1;
+  if (row8_fast(a)) return row8_copy(a, which).total;
   return which == 0 ? (size_t)a->E * 2 * a->I * p.Hk * es : (size_t)a->E * a->H * p.Iw * es;
 }
 
@@ -312,7 +361,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     }
   }
 
-  const bool mx_fast = a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I);
+  const bool r8_fast = row8_fast(a);
+  const bool mx_fast = (a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I)) || r8_fast;
   MxArgs m;
   memset(&m, 0, sizeof(m));
   if (mx_fast) {
@@ -332,10 +382,18 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     m.ys_stride = p.Iw / 32;
     m.D = (uint16_t*)(ws + p.d);
     m.H = a->H; m.I = a->I; m.E = a->E; m.n_real = n_real;
+    m.chunk_interleave = chunk_interleave_for(a->N, a->B, a->E);
     m.pI = (int32_t)p.pI; m.nI = (int32_t)p.nI;
     m.act_fn = a->act_fn; m.scaling_mode = a->scaling_mode; m.clamp_mask = a->clamp_mask;
     m.wfmt = (a->weight_dtype == MOE_DT_FP8_E5M2) ? MX_WFMT_E5M2 : (a->weight_dtype == MOE_DT_FP4_E2M1) ? MX_WFMT_E2M1 : MX_WFMT_E4M3;
     for (int i = 0; i < 4; ++i) m.clamp[i] = g.clamp[i];
+    if (r8_fast) {
+      m.wfmt = MX_WFMT_ROW8;
+      m.cscale_experts = a->scale_experts;
+      m.w_scale_shared = 1;
+      m.Y32 = (float*)(ws + p.y);
+      m.y32_stride = a->I;
+    }
   }
   const unsigned gyc = (unsigned)bk.max_chunks;
   // checkpoints of blocks that never run stay zero
@@ -354,6 +412,13 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
       m1.a_rows = n_real;
       m1.W = (const uint32_t*)a->gate_up_proj_weight; m1.W_scale = (const uint8_t*)a->gate_up_proj_scale;
       m1.bias = a->gate_and_up_proj_bias;
+      if (r8_fast) {
+        const Row8Copy c = row8_copy(a, 0);
+        m1.W = (const uint32_t*)g1.W;  // the x4 copy (kept by the caller or made above)
+        m1.W_scale = g1.W + c.w_scale;
+        m1.A_scale = g1.W + c.a_scale; m1.a_scale_stride = 0; m1.a_scale_bytes = (int64_t)c.a_scale_bytes;
+        m1.w_cscale = (const float*)a->gate_up_proj_scale;
+      }
       // column tiles of 32 partitions x 4 q, gate and up: 4 per full intermediate tile + those of a short last one
       rc = launch_mx_gemm(1, m1, (unsigned)((a->I / 512) * 4 + (a->I % 512) / 128), gyc, s);
     } else {
@@ -372,6 +437,14 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
       m2.a_rows = a->N * a->B;
       m2.W = (const uint32_t*)a->down_proj_weight; m2.W_scale = (const uint8_t*)a->down_proj_scale;
       m2.bias = a->down_proj_bias;
+      if (r8_fast) {
+        const Row8Copy c = row8_copy(a, 1);
+        m2.W = (const uint32_t*)g2.W;
+        m2.W_scale = g2.W + c.w_scale;
+        m2.A_scale = g2.W + c.a_scale; m2.a_scale_stride = 0; m2.a_scale_bytes = (int64_t)c.a_scale_bytes;
+        m2.w_cscale = (const float*)a->down_proj_scale;
+        m2.a_rscale = (const float*)(ws + p.ys);
+      }
       rc = launch_mx_gemm(2, m2, (unsigned)(a->H / 256), gyc, s);
     } else {
       rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);

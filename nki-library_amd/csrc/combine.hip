@@ -63,7 +63,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
                                              int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
                                              int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
                                              int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off,
-                                             int64_t max_chunks, int* s_ws) {
+                                             int64_t max_chunks, int interleave, int* s_ws) {
   const int64_t na = *n_active;
   int carry = 0;
   for (int64_t b0 = 0; b0 < na; b0 += 1024) {
@@ -105,8 +105,10 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   const int per = (n + 7) >> 3;
   for (int i = threadIdx.x; i <= 8 * CHUNK_CLASSES; i += blockDim.x) s_cnt[i] = 0;
   __syncthreads();
+  // (interleaved chunks share their weight tiles through the L2: none of them streams the weights past it, so
+  // "last chunk of its expert" is no class of its own then)
   auto key_of = [&](int i) {
-    const bool last = (i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]);
+    const bool last = interleave == 1 && ((i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]));
     return (i / per) * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
   };
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&s_cnt[key_of(i)], 1);
@@ -124,8 +126,18 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   __syncthreads();
   // (the order inside one class is whatever order the atomics are served in: it decides which chunks run at the
   // same time, never a result)
+  // With interleaving neighbours in the queue must be chunks of the same expert, so a chunk's place in its class
+  // is its rank by chunk index (the chunks of this shape family are few).
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    const int pos = atomicAdd(&s_cnt[key_of(i)], 1);
+    const int key = key_of(i);
+    int pos;
+    if (interleave == 1) {
+      pos = atomicAdd(&s_cnt[key], 1);
+    } else {
+      int rank = 0;
+      for (int j = (i / per) * per; j < i; ++j) rank += key_of(j) == key;
+      pos = s_cnt[key] + rank;
+    }
     q_chunk[2 * pos] = chunk_slot[i];
     q_chunk[2 * pos + 1] = chunk_rows[i] | (chunk_expert[i] << 16);  // at most 320 rows, fewer than 32768 experts
   }
@@ -167,12 +179,12 @@ __global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
     const int32_t* __restrict__ b2e, const int32_t* __restrict__ n_active, const int32_t* __restrict__ valid_rows,
     int64_t N, int64_t B, int64_t E, int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
     int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int32_t* __restrict__ q_chunk,
-    int32_t* __restrict__ q_off, int64_t max_chunks, const int32_t* __restrict__ cnt, int32_t* __restrict__ off,
-    int64_t n_real) {
+    int32_t* __restrict__ q_off, int64_t max_chunks, int interleave, const int32_t* __restrict__ cnt,
+    int32_t* __restrict__ off, int64_t n_real) {
   __shared__ int s_ws[16];
   if (blockIdx.x == 0)
     build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, q_chunk, q_off,
-                 max_chunks, s_ws);
+                 max_chunks, interleave, s_ws);
   else
     inv_scan(cnt, off, n_real, s_ws);
 }
@@ -301,7 +313,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(chunks_and_offsets_kernel, dim3(2), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows,
                      a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.q_chunk, k.q_off,
-                     k.max_chunks, k.cnt, k.off, n_real);
+                     k.max_chunks, chunk_interleave_for(a->N, a->B, a->E), k.cnt, k.off, n_real);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
   const unsigned gs = (unsigned)((slots + 255) / 256);

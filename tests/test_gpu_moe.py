@@ -313,7 +313,9 @@ def _run_fp8_row(c, gamma, mode=1, clamps=None, act=0):
 
 
 @pytest.mark.parametrize("T,H,I,E,k,B", [(256, 512, 512, 4, 2, 128), (384, 1024, 896, 8, 2, 128),
-                                         (300, 512, 640, 2, 2, 128), (768, 1024, 896, 2, 2, 128)])  # 256-row chunk tiles
+                                         (300, 512, 640, 2, 2, 128), (768, 1024, 896, 2, 2, 128),  # 256-row chunk tiles
+                                         # shapes outside the large-tile kernels: the general tiled kernel
+                                         (256, 512, 448, 4, 2, 128), (300, 768, 512, 4, 2, 128)])
 def test_fp8_row_pipeline(T, H, I, E, k, B):
     """RMSNorm-Quant ROW -> fp8 x fp8 blockwise MoE with per-row / per-channel scales (BASELINE config 2 shape family)."""
     import torch
