@@ -691,32 +691,41 @@ int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C,
   return MOE_OK;
 }
 
-// One thread per x4 element (four K values of one output column).
-__global__ __launch_bounds__(256) void relayout_gu_x4_kernel(const uint8_t* __restrict__ W, uint32_t* __restrict__ X,
-                                                             int64_t H, int64_t I, int64_t total) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const int64_t nH = H / 512;
-  const int64_t i = idx % I, t = (idx / I) % nH, gu = (idx / (I * nH)) % 2, p = (idx / (I * nH * 2)) % 128,
-                e = idx / (I * nH * 2 * 128);
-  const int64_t h = t * 512 + p * 4;
-  uint32_t v = 0;
+// One thread per four adjacent output columns: four 4-byte reads (the four K rows of the x4 elements), a 4 x 4 byte
+// transpose, one 16-byte write.  I % 4 == 0 and H % 4 == 0 on this path.
+__device__ __forceinline__ uint4 bytes_4x4_transposed(const uint32_t (&r)[4]) {
+  uint32_t o[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) v |= (uint32_t)W[((e * H + h + q) * 2 + gu) * I + i] << (8 * q);
-  X[idx] = v;
+  for (int c = 0; c < 4; ++c)
+    o[c] = ((r[0] >> (8 * c)) & 0xffu) | (((r[1] >> (8 * c)) & 0xffu) << 8) | (((r[2] >> (8 * c)) & 0xffu) << 16) |
+           (((r[3] >> (8 * c)) & 0xffu) << 24);
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+__global__ __launch_bounds__(256) void relayout_gu_x4_kernel(const uint8_t* __restrict__ W, uint32_t* __restrict__ X,
+                                                             int64_t H, int64_t I, int64_t total4) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over [E, 128, 2, nH, I / 4]
+  if (idx >= total4) return;
+  const int64_t nH = H / 512, I4 = I / 4;
+  const int64_t i = (idx % I4) * 4, t = (idx / I4) % nH, gu = (idx / (I4 * nH)) % 2, p = (idx / (I4 * nH * 2)) % 128,
+                e = idx / (I4 * nH * 2 * 128);
+  const int64_t h = t * 512 + p * 4;
+  uint32_t r[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) r[q] = *(const uint32_t*)(W + ((e * H + h + q) * 2 + gu) * I + i);
+  *(uint4*)(X + idx * 4) = bytes_4x4_transposed(r);
 }
 __global__ __launch_bounds__(256) void relayout_down_x4_kernel(const uint8_t* __restrict__ W, uint32_t* __restrict__ X,
                                                                int64_t H, int64_t I, int64_t I_pad, int64_t pI,
-                                                               int64_t nI, int64_t total) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const int64_t h = idx % H, t = (idx / H) % nI, p = (idx / (H * nI)) % pI, e = idx / (H * nI * pI);
+                                                               int64_t nI, int64_t total4) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over [E, pI, nI, H / 4]
+  if (idx >= total4) return;
+  const int64_t H4 = H / 4;
+  const int64_t h = (idx % H4) * 4, t = (idx / H4) % nI, p = (idx / (H4 * nI)) % pI, e = idx / (H4 * nI * pI);
   const int64_t i0 = t * 512 + p * 4;
-  uint32_t v = 0;
+  uint32_t r[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-    if (i0 + q < I) v |= (uint32_t)W[(e * I_pad + i0 + q) * H + h] << (8 * q);
-  X[idx] = v;
+  for (int q = 0; q < 4; ++q) r[q] = (i0 + q < I) ? *(const uint32_t*)(W + (e * I_pad + i0 + q) * H + h) : 0u;
+  *(uint4*)(X + idx * 4) = bytes_4x4_transposed(r);
 }
 __global__ __launch_bounds__(256) void fill_bytes_kernel(uint32_t* __restrict__ p, int64_t words, uint32_t v) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -735,15 +744,16 @@ int launch_fill_bytes(void* p, size_t bytes, uint8_t value, hipStream_t s) {
 
 int launch_relayout_x4(const uint8_t* gate_up, const uint8_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
                        int64_t I, int64_t I_pad, hipStream_t s) {
-  if ((((uintptr_t)dst) & 3) != 0) return MOE_E_BAD_ARG;
+  if ((((uintptr_t)dst) & 15) != 0 || (((uintptr_t)gate_up) & 3) != 0 || (((uintptr_t)down) & 3) != 0)
+    return MOE_E_BAD_ARG;
   if (which == 0) {
-    const int64_t total = E * 128 * 2 * (H / 512) * I;
+    const int64_t total = E * 128 * 2 * (H / 512) * (I / 4);
     if ((total + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
     hipLaunchKernelGGL(relayout_gu_x4_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gate_up,
                        (uint32_t*)dst, H, I, total);
   } else {
     const int64_t nI = (I + 511) / 512, pI = I > 512 ? 128 : I / 4;
-    const int64_t total = E * pI * nI * H;
+    const int64_t total = E * pI * nI * (H / 4);
     if ((total + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
     hipLaunchKernelGGL(relayout_down_x4_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, down,
                        (uint32_t*)dst, H, I, I_pad, pI, nI, total);
