@@ -62,8 +62,9 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
                                              const int32_t* __restrict__ valid_rows, int64_t N, int64_t B, int64_t E,
                                              int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
                                              int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
-                                             int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off,
-                                             int64_t max_chunks, int interleave, int* s_ws) {
+                                             int32_t* __restrict__ chunk_xcd, int32_t* __restrict__ q_chunk,
+                                             int32_t* __restrict__ q_off, int64_t max_chunks, int interleave,
+                                             int* s_ws) {
   const int64_t na = *n_active;
   int carry = 0;
   for (int64_t b0 = 0; b0 < na; b0 += 1024) {
@@ -102,14 +103,38 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   __shared__ int s_cnt[8 * CHUNK_CLASSES + 1];
   __threadfence_block();
   __syncthreads();
-  const int per = (n + 7) >> 3;
   for (int i = threadIdx.x; i <= 8 * CHUNK_CLASSES; i += blockDim.x) s_cnt[i] = 0;
+  // Which XCD takes which chunks: contiguous parts of the list (chunks of one expert, and experts that follow each
+  // other, stay behind one L2) of about equal work.  Work = row tiles of the kernel variant that runs the chunk
+  // (its column tiles are the same for all); a chunk goes where the middle of its span of the running total falls.
+  // (Equal chunk counts left the XCDs up to a tenth apart in work at ragged expert loads, and a launch ends when
+  // its last XCD does.)
+  auto work_of = [&](int i) {
+    const int r = chunk_rows[i];
+    return r <= 64 ? 4 : r <= 128 ? 8 : r <= 256 ? 16 : 20;
+  };
+  int wcarry = 0;
+  for (int i0 = 0; i0 < n; i0 += 1024) {
+    const int i = i0 + threadIdx.x;
+    int total;
+    const int pre = wcarry + block_excl_scan(i < n ? work_of(i) : 0, s_ws, &total);
+    if (i < n) chunk_xcd[i] = pre;
+    wcarry += total;
+  }
+  __threadfence_block();
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int64_t mid2 = 2 * (int64_t)chunk_xcd[i] + work_of(i);  // twice the middle of the chunk's span
+    const int x = (int)(mid2 * 8 / (2 * (int64_t)wcarry));
+    chunk_xcd[i] = x > 7 ? 7 : x;
+  }
+  __threadfence_block();
   __syncthreads();
   // (interleaved chunks share their weight tiles through the L2: none of them streams the weights past it, so
   // "last chunk of its expert" is no class of its own then)
   auto key_of = [&](int i) {
     const bool last = interleave == 1 && ((i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]));
-    return (i / per) * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
+    return chunk_xcd[i] * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
   };
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&s_cnt[key_of(i)], 1);
   __syncthreads();
@@ -135,7 +160,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
       pos = atomicAdd(&s_cnt[key], 1);
     } else {
       int rank = 0;
-      for (int j = (i / per) * per; j < i; ++j) rank += key_of(j) == key;
+      for (int j = 0; j < i; ++j) rank += key_of(j) == key;
       pos = s_cnt[key] + rank;
     }
     q_chunk[2 * pos] = chunk_slot[i];
@@ -178,13 +203,13 @@ __device__ __forceinline__ void inv_scan(const int32_t* __restrict__ cnt, int32_
 __global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
     const int32_t* __restrict__ b2e, const int32_t* __restrict__ n_active, const int32_t* __restrict__ valid_rows,
     int64_t N, int64_t B, int64_t E, int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
-    int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int32_t* __restrict__ q_chunk,
-    int32_t* __restrict__ q_off, int64_t max_chunks, int interleave, const int32_t* __restrict__ cnt,
-    int32_t* __restrict__ off, int64_t n_real) {
+    int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int32_t* __restrict__ chunk_xcd,
+    int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off, int64_t max_chunks, int interleave,
+    const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n_real) {
   __shared__ int s_ws[16];
   if (blockIdx.x == 0)
-    build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, q_chunk, q_off,
-                 max_chunks, interleave, s_ws);
+    build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, chunk_xcd, q_chunk,
+                 q_off, max_chunks, interleave, s_ws);
   else
     inv_scan(cnt, off, n_real, s_ws);
 }
@@ -273,11 +298,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
 // ---- host-side orchestration used by moe_blockwise() -------------------------------------
 
 size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B) {
-  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B] | n_chunks[4] | 5 x chunk[max_chunks] |
+  // n_active[4] | valid_rows[N] | cnt[T1] | cursor[T1] | off[T1+1] | list[N*B] | n_chunks[4] | 6 x chunk[max_chunks] |
   // q_off[8][CHUNK_CLASSES + 1], each region 256-byte aligned
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
   return al(16) + al((size_t)N * 4) + 2 * al((size_t)T1 * 4) + al((size_t)(T1 + 1) * 4) + al((size_t)N * B * 4) +
-         al(16) + 5 * al((size_t)max_chunks_for(N, B) * 4) + al((size_t)8 * (CHUNK_CLASSES + 1) * 4);
+         al(16) + 6 * al((size_t)max_chunks_for(N, B) * 4) + al((size_t)8 * (CHUNK_CLASSES + 1) * 4);
 }
 
 Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
@@ -295,6 +320,7 @@ Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
   k.chunk_slot = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
   k.chunk_rows = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
   k.chunk_expert = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
+  k.chunk_xcd = (int32_t*)p; p += al((size_t)k.max_chunks * 4);
   k.q_chunk = (int32_t*)p; p += 2 * al((size_t)k.max_chunks * 4);
   k.q_off = (int32_t*)p;
   return k;
@@ -312,7 +338,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
                      a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows, k.cnt);
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(chunks_and_offsets_kernel, dim3(2), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows,
-                     a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.q_chunk, k.q_off,
+                     a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.chunk_xcd, k.q_chunk, k.q_off,
                      k.max_chunks, chunk_interleave_for(a->N, a->B, a->E), k.cnt, k.off, n_real);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;

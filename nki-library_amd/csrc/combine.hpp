@@ -20,8 +20,9 @@ struct Bookkeeping {
   int32_t* chunk_slot;    // [max_chunks]
   int32_t* chunk_rows;    // [max_chunks]
   int32_t* chunk_expert;  // [max_chunks]
-  // Work queues of the large-tile MX kernels.  XCD x owns the x-th contiguous eighth of the chunk list; q_chunk holds
-  // that eighth's chunks grouped by class (row-tile variant x last chunk of its expert, CHUNK_CLASSES of them), two
+  int32_t* chunk_xcd;     // [max_chunks] the XCD whose queue holds the chunk
+  // Work queues of the large-tile MX kernels.  The chunk list is cut into eight contiguous parts of about equal
+  // work (row tiles), one per XCD; q_chunk holds a part's chunks grouped by class (row-tile variant x last chunk of its expert, CHUNK_CLASSES of them), two
   // words per chunk: its first slot, and rows | expert << 16; q_off[x][c] .. q_off[x][c+1] are the positions of
   // class c of XCD x in q_chunk.
   int32_t* q_chunk;       // [max_chunks][2]
