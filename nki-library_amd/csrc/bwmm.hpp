@@ -58,7 +58,7 @@ struct MxArgs {
   const int32_t* chunk_rows;
   const int32_t* chunk_expert;
   const int32_t* q_chunk;  // work queues: two words per chunk, per XCD grouped by class, see Bookkeeping
-  const int32_t* q_off;    // [8][CHUNK_CLASSES + 1]
+  const int32_t* q_off;    // [8][CHUNK_CLASSES + 1], then the chunk interleave
   uint8_t* Yq;             // stage 1 output
   uint8_t* Ys;
   int64_t y_stride, ys_stride;
@@ -69,7 +69,6 @@ struct MxArgs {
   float clamp[4];
   int32_t col_tiles;       // column tiles per chunk (set by the launcher)
   int32_t wfmt;            // element format of the weights, MX_WFMT_*
-  int32_t chunk_interleave;  // chunks whose column tiles alternate in a class's item order, see chunk_interleave_for
   // MX_WFMT_ROW8 (the fp8-row kind on these kernels): e4m3 operands whose E8M0 tables are constants of 127, a
   // per-row fp32 scale of the activations and a per-output-channel fp32 scale of the weights in the epilogue
   const float* w_cscale;   // [cscale_experts][2*I] (gate/up: gate then up) or [cscale_experts][H] (down)

@@ -274,7 +274,7 @@ template <int STAGE, int NMT, bool LASTUSE, int WFMT>
 __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int (*s_tok)[MX_ROWS_MAX],
                                              float (*s_aff)[MX_ROWS_MAX], float (*s_bias)[MXT],
                                              float (*s_rs)[MX_ROWS_MAX], float (*s_wsc)[MXT], int L, const int startL,
-                                             const int endL, const int Lstep, const int qbase) {
+                                             const int endL, const int Lstep, const int qbase, const int interleave) {
   using Cfg = MxCfg<NMT>;
   // ROW8: the fp8-row kind.  Same K loop on e4m3 operands with block scales of 2^0; what differs is the epilogue
   // (per-channel weight scale x per-row activation scale ahead of the bias, bias and scales indexed by natural
@@ -305,7 +305,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     int nrows, e, slot0, xt;
   };
   typedef int v2i_t __attribute__((ext_vector_type(2)));
-  // Item l of the class -> (chunk position, column tile).  G = a.chunk_interleave chunks at a time: within a
+  // Item l of the class -> (chunk position, column tile).  G = `interleave` chunks at a time (chosen with the queues): within a
   // group of G queue positions the chunk varies fastest, so that workgroups with neighbouring items work on the
   // same column tile of different chunks (of one expert: they share the weight tile); G = 1 is column tiles
   // innermost.  The last group of a class may hold fewer than G chunks.
@@ -313,15 +313,15 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   const int pos0 = startL / a.col_tiles, npos = (endL - startL) / a.col_tiles;
   auto tile_at = [&](int l) {
     int pos, xt;
-    if (a.chunk_interleave == 1) {
+    if (interleave == 1) {
       pos = l / a.col_tiles;
       xt = l - pos * a.col_tiles;
     } else {
-      const int per_group = a.chunk_interleave * a.col_tiles;
+      const int per_group = interleave * a.col_tiles;
       const int lr = l - startL;
       const int grp = lr / per_group, j = lr - grp * per_group;
-      const int base = grp * a.chunk_interleave;
-      const int G = (npos - base < a.chunk_interleave) ? npos - base : a.chunk_interleave;
+      const int base = grp * interleave;
+      const int G = (npos - base < interleave) ? npos - base : interleave;
       xt = j / G;
       pos = pos0 + base + (j - xt * G);
     }
@@ -1140,6 +1140,7 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int xcd = blockIdx.x & 7, w = blockIdx.x >> 3, W = gridDim.x >> 3;
   const int32_t* qo = a.q_off + xcd * (CHUNK_CLASSES + 1);
   const int qbase = __builtin_amdgcn_readfirstlane(qo[0]);
+  const int interleave = __builtin_amdgcn_readfirstlane(a.q_off[8 * (CHUNK_CLASSES + 1)]);
   int L = w;
   // classes in queue order (chunk_class): row-tile variants 20, 16, 8, 4, each first "not the last chunk of
   // its expert", then "last"
@@ -1149,7 +1150,8 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int endL = (__builtin_amdgcn_readfirstlane(qo[CLS_ + 1]) - qbase) * a.col_tiles;                     \
     if (L < endL)                                                                                              \
       L = mx_gemm_tiles<STAGE, NMT_, LAST_, WFMT>(a, smem, s_tok, s_aff, s_bias, (float(*)[MX_ROWS_MAX])s_rs,  \
-                                                  (float(*)[MXT])s_wsc, L, startL, endL, W, qbase);           \
+                                                  (float(*)[MXT])s_wsc, L, startL, endL, W, qbase,            \
+                                                  interleave);                                                \
     __syncthreads();                                                                                           \
   }
   MX_RUN_CLASS(0, 20, false)

@@ -382,7 +382,6 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     m.ys_stride = p.Iw / 32;
     m.D = (uint16_t*)(ws + p.d);
     m.H = a->H; m.I = a->I; m.E = a->E; m.n_real = n_real;
-    m.chunk_interleave = chunk_interleave_for(a->N, a->B, a->E);
     m.pI = (int32_t)p.pI; m.nI = (int32_t)p.nI;
     m.act_fn = a->act_fn; m.scaling_mode = a->scaling_mode; m.clamp_mask = a->clamp_mask;
     m.wfmt = (a->weight_dtype == MOE_DT_FP8_E5M2) ? MX_WFMT_E5M2 : (a->weight_dtype == MOE_DT_FP4_E2M1) ? MX_WFMT_E2M1 : MX_WFMT_E4M3;

@@ -63,10 +63,10 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
                                              int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
                                              int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
                                              int32_t* __restrict__ chunk_xcd, int32_t* __restrict__ q_chunk,
-                                             int32_t* __restrict__ q_off, int64_t max_chunks, int interleave,
-                                             int* s_ws) {
+                                             int32_t* __restrict__ q_off, int64_t max_chunks, int* s_ws) {
   const int64_t na = *n_active;
   int carry = 0;
+  int runs = 0;  // runs that hold chunks (over this thread's runs)
   for (int64_t b0 = 0; b0 < na; b0 += 1024) {
     const int64_t b = b0 + threadIdx.x;
     int nch = 0;
@@ -84,6 +84,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
         if (len > 0) nch = (len <= CHUNK_ROWS_MAX) ? 1 : (int)((len - CHUNK_ROWS_MAX + CHUNK_ROWS - 1) / CHUNK_ROWS) + 1;
       }
     }
+    runs += nch > 0;
     int total;
     const int base = carry + block_excl_scan(nch, s_ws, &total);
     for (int k = 0; k < nch; ++k) {
@@ -101,8 +102,22 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   // Work queues: a counting sort of the chunks by (XCD that owns them, class).  The chunk arrays were written by
   // this workgroup: make them visible to all of its threads first.
   __shared__ int s_cnt[8 * CHUNK_CLASSES + 1];
+  __shared__ int s_runs;
+  if (threadIdx.x == 0) s_runs = 0;
   __threadfence_block();
   __syncthreads();
+  if (runs > 0) atomicAdd(&s_runs, runs);
+  __syncthreads();
+  // How many chunks of one expert the large-tile GEMMs work on side by side (the kernels read it behind q_off).
+  // While experts hold fewer than three chunks on average: 1, i.e. a round of an XCD's workgroups covers the column
+  // tiles of one chunk after the other and shares that chunk's activation tile.  With three and more (few experts
+  // with many rows each): that average, up to 8, i.e. the item order of a class alternates between G neighbouring
+  // chunks, which are then mostly chunks of one expert: they work on the same weight tile at the same time and
+  // share it through the L2 instead of streaming it from memory once per chunk.  (Applied to a skewed router's
+  // few hot experts among many single-chunk ones it costs more in activation sharing than it saves: measured.)
+  const int avg = s_runs > 0 ? (n + s_runs / 2) / s_runs : 1;
+  const int interleave = avg < 3 ? 1 : (avg > 8 ? 8 : avg);
+  if (threadIdx.x == 0) q_off[8 * (CHUNK_CLASSES + 1)] = interleave;
   for (int i = threadIdx.x; i <= 8 * CHUNK_CLASSES; i += blockDim.x) s_cnt[i] = 0;
   // Which XCD takes which chunks: contiguous parts of the list (chunks of one expert, and experts that follow each
   // other, stay behind one L2) of about equal work.  Work = row tiles of the kernel variant that runs the chunk
@@ -204,12 +219,12 @@ __global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
     const int32_t* __restrict__ b2e, const int32_t* __restrict__ n_active, const int32_t* __restrict__ valid_rows,
     int64_t N, int64_t B, int64_t E, int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
     int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int32_t* __restrict__ chunk_xcd,
-    int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off, int64_t max_chunks, int interleave,
+    int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off, int64_t max_chunks,
     const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n_real) {
   __shared__ int s_ws[16];
   if (blockIdx.x == 0)
     build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, chunk_xcd, q_chunk,
-                 q_off, max_chunks, interleave, s_ws);
+                 q_off, max_chunks, s_ws);
   else
     inv_scan(cnt, off, n_real, s_ws);
 }
@@ -302,7 +317,7 @@ size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B) {
   // q_off[8][CHUNK_CLASSES + 1], each region 256-byte aligned
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
   return al(16) + al((size_t)N * 4) + 2 * al((size_t)T1 * 4) + al((size_t)(T1 + 1) * 4) + al((size_t)N * B * 4) +
-         al(16) + 6 * al((size_t)max_chunks_for(N, B) * 4) + al((size_t)8 * (CHUNK_CLASSES + 1) * 4);
+         al(16) + 6 * al((size_t)max_chunks_for(N, B) * 4) + al((size_t)(8 * (CHUNK_CLASSES + 1) + 1) * 4);
 }
 
 Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
@@ -339,7 +354,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(chunks_and_offsets_kernel, dim3(2), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows,
                      a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.chunk_xcd, k.q_chunk, k.q_off,
-                     k.max_chunks, chunk_interleave_for(a->N, a->B, a->E), k.cnt, k.off, n_real);
+                     k.max_chunks, k.cnt, k.off, n_real);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
   const unsigned gs = (unsigned)((slots + 255) / 256);

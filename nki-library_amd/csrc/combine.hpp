@@ -26,7 +26,7 @@ struct Bookkeeping {
   // words per chunk: its first slot, and rows | expert << 16; q_off[x][c] .. q_off[x][c+1] are the positions of
   // class c of XCD x in q_chunk.
   int32_t* q_chunk;       // [max_chunks][2]
-  int32_t* q_off;         // [8][CHUNK_CLASSES + 1]
+  int32_t* q_off;         // [8][CHUNK_CLASSES + 1], then one word: the chunk interleave (see build_chunks)
   int64_t max_chunks;
 };
 
@@ -36,17 +36,6 @@ constexpr int CHUNK_CLASSES = 8;
 __host__ __device__ inline int chunk_class(int rows, bool last) {
   const int v = rows <= 64 ? 0 : rows <= 128 ? 1 : rows <= 256 ? 2 : 3;
   return (3 - v) * 2 + (last ? 1 : 0);
-}
-
-// How many chunks of one expert the large-tile GEMMs work on side by side (MxArgs::chunk_interleave): with about
-// one chunk per expert (many experts, few rows each) 1, i.e. a workgroup round covers the column tiles of one
-// chunk after the other and shares that chunk's activation tile; with several chunks per expert (few experts,
-// many rows each) up to 8, i.e. a round covers a few column tiles of G chunks of the same expert, which then
-// share each weight tile through the L2 instead of streaming it from memory once per chunk.  From the average
-// number of slots per expert, so that the bookkeeping and the GEMM launches agree without exchanging anything.
-inline int chunk_interleave_for(int64_t N, int64_t B, int64_t E) {
-  const int64_t g = (N * B / E + 128) / 256;
-  return g < 1 ? 1 : (g > 8 ? 8 : (int)g);
 }
 
 constexpr int CHUNK_ROWS = 256;      // rows of every chunk of a run but the last
