@@ -293,7 +293,7 @@ def test_fp8_weight_only():
     _check(from_bf16_tensor(out), _golden_dense(c, fp8_weights=True), "fp8 weight-only")
 
 
-def _run_fp8_row(c, gamma, mode=1, clamps=None, act=0):
+def _run_fp8_row(c, gamma, mode=1, clamps=None, act=0, shared_scales=False):
     import torch
     from nkilib.core.moe.moe_cte import QuantizationConfig, moe_cte
     from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
@@ -301,13 +301,19 @@ def _run_fp8_row(c, gamma, mode=1, clamps=None, act=0):
 
     dev = torch.device("cuda:0")
     rec = rmsnorm_quant_kernel(bf16_tensor(c["hidden"], dev), bf16_tensor(gamma, dev), RmsNormQuantKernelArgs())
+    kw = dict(clamps or {})
+    if "gate_up_bias" in c:
+        kw["gate_and_up_proj_bias"] = bf16_tensor(c["gate_up_bias"], dev)
+        kw["down_proj_bias"] = bf16_tensor(c["down_bias"], dev)
+    gs, ds = c["gate_up_scale"], c["down_scale"]
+    if shared_scales:  # one set of channel scales for every expert: leading dimension 1
+        gs, ds = gs[:1], ds[:1]
     out = moe_cte(
         rec, bf16_tensor(c["aff"].reshape(-1, 1), dev), u8_tensor(c["gate_up_q"], dev).view(torch.float8_e4m3fn),
         u8_tensor(c["down_q"], dev).view(torch.float8_e4m3fn), i32_tensor(c["tp2id"], dev),
         i32_tensor(c["b2e"], dev), c["B"], _spec("shard_on_block"),
-        quantization_config=QuantizationConfig(f32_tensor(c["gate_up_scale"], dev), f32_tensor(c["down_scale"], dev)),
-        activation_function=ActFnType(act), expert_affinities_scaling_mode=ExpertAffinityScaleMode(mode),
-        **(clamps or {}))
+        quantization_config=QuantizationConfig(f32_tensor(gs, dev), f32_tensor(ds, dev)),
+        activation_function=ActFnType(act), expert_affinities_scaling_mode=ExpertAffinityScaleMode(mode), **kw)
     torch.cuda.synchronize()
     return rec, out
 
@@ -331,24 +337,33 @@ def test_fp8_row_pipeline(T, H, I, E, k, B):
     _check(from_bf16_tensor(out)[:, 0], g, "fp8 row")
 
 
-@pytest.mark.parametrize("mode,clamp,act", [(2, False, 0), (1, True, 3), (2, True, 1), (0, False, 0)])
-def test_fp8_row_scale_modes_and_clamps(mode, clamp, act):
+@pytest.mark.parametrize("mode,clamp,act,I,shared", [(2, False, 0, 896, False), (1, True, 3, 896, True),
+                                                     (2, True, 1, 896, False), (0, False, 0, 896, False),
+                                                     (2, True, 3, 448, True)])  # I = 448: the general tiled kernel
+def test_fp8_row_scale_modes_and_clamps(mode, clamp, act, I, shared):
     """PRE_SCALE (the affinity scales the token's row, i.e. its dequantisation scale), NO_SCALE and the four clamps on
     the fp8-row kind.  The reference has no kernel with fp8 activations on this path: the rule is the dense
     golden's (test_moe_cte_common.py:383-402) applied to the row-quantised operands."""
     import torch
 
-    T, H, I, E, k, B = 384, 1024, 896, 8, 2, 128
-    c = dense_case(T, H, I, E, k, B, seed=16, quant=True, hidden_std=1.0)
+    T, H, E, k, B = 384, 1024, 8, 2, 128
+    c = dense_case(T, H, I, E, k, B, seed=16, quant=True, bias=True, hidden_std=1.0)
     clamps = dict(gate_clamp_upper_limit=0.6, gate_clamp_lower_limit=-0.5, up_clamp_upper_limit=0.7,
                   up_clamp_lower_limit=-0.4) if clamp else {}
-    rec, out = _run_fp8_row(c, np.ones((1, H), np.float32), mode=mode, clamps=clamps, act=act)
+    rec, out = _run_fp8_row(c, np.ones((1, H), np.float32), mode=mode, clamps=clamps, act=act, shared_scales=shared)
     raw = rec.view(torch.uint8).cpu().numpy()
     codes, scale = raw[:, :H], raw[:, H:].copy().view(np.float32).reshape(-1)
-    g = omoe.moe_blockwise_fp8_row_ref(codes, scale, c["aff"], c["gate_up_q"], c["down_q"], c["gate_up_scale"],
-                                       c["down_scale"], c["tp2id"], c["b2e"], c["B"], activation_function=act,
+    gs, ds = c["gate_up_scale"], c["down_scale"]
+    if shared:
+        gs, ds = np.repeat(gs[:1], E, axis=0), np.repeat(ds[:1], E, axis=0)
+    g = omoe.moe_blockwise_fp8_row_ref(codes, scale, c["aff"], c["gate_up_q"], c["down_q"], gs, ds, c["tp2id"],
+                                       c["b2e"], c["B"], gate_up_proj_bias=c["gate_up_bias"],
+                                       down_proj_bias=c["down_bias"], activation_function=act,
                                        expert_affinities_scaling_mode=mode, **clamps)
-    _check(from_bf16_tensor(out)[:, 0], g, f"fp8 row mode={mode} clamp={clamp} act={act}")
+    o = from_bf16_tensor(out)[:, 0]
+    # (the golden scatters the down bias to the padding token's row as well; the kernels leave that row zero)
+    assert not o[T].any()
+    _check(o[:T], g[:T], f"fp8 row mode={mode} clamp={clamp} act={act} I={I} shared={shared}")
 
 
 def _run_mx(c, prequant=False, act=0, weight_dtype=None):
