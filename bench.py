@@ -74,6 +74,9 @@ def parse_args():
     ap.add_argument("--weights", default="mxfp8", choices=["mxfp8", "mxfp4"],
                     help="mxfp8: e4m3 expert weights (the reported workload); mxfp4: float4_e2m1fn_x4 weights, same "
                          "layer (diagnostic: half the weight bytes; no CPU baseline)")
+    ap.add_argument("--no-mx-weight-copies", action="store_true",
+                    help="diagnostic: read the MXFP8 expert weights in the reference layout in place instead of the "
+                         "copies in the kernels' read order that moe_cte makes once per weight tensor pair")
     ap.add_argument("--routing", default="router", choices=["router", "balanced"],
                     help="router: top-k of synthetic scores (the reported workload); balanced: every expert gets "
                          "exactly T*k/E rows (diagnostic, shows the cost of ragged expert loads)")
@@ -308,6 +311,7 @@ def main():
     from nkilib.core.moe.moe_cte import (MoECTEImplementation, MoECTESpec, QuantizationConfig, build_token_blocks,
                                          get_n_blocks, moe_cte)
     from nkilib.core.moe.moe_cte import _launch
+    _launch.mx_weight_copies = not args.no_mx_weight_copies
     from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"

@@ -530,10 +530,20 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // element strides (4-byte weights; scales use the same counts in bytes)
   const int64_t w_pstride = (STAGE == 1) ? 2 * nH * a.I : (int64_t)a.nI * a.H;
   const int64_t w_tstride = (STAGE == 1) ? a.I : a.H;
-  const uint32_t w_voff = (STAGE == 1) ? (uint32_t)((GROWS * g * w_pstride + hcol * nH * a.I + 4 * cl) * ES)
-                                       : (uint32_t)((GROWS * g * w_pstride + 4 * c) * ES);
+  // a.w_packed (gate/up only): the weights are a copy in the order these loads read them (see mx_pack_weights_kernel): load i of
+  // wave q in slice ks of column tile xt is 1 KB at ((xt * nks + ks) * 4 + q) * 8 KB + i * 1 KB of the expert's
+  // copy, a lane's 16 bytes at 16 * lane: each workgroup reads its weights as one contiguous 32 KB run per slice.
+  // (the two address forms are blended with the 0 / 1 flag as a factor: a conditional expression here may become
+  // a branch, and values that cross a branch in this function are no longer known to the compiler as uniform)
+  const int pk = a.w_packed ? 1 : 0, npk = 1 - pk;
+  const uint32_t w_voff = (uint32_t)pk * (uint32_t)(lane * 16) +
+                          (uint32_t)npk * ((STAGE == 1) ? (uint32_t)((GROWS * g * w_pstride + hcol * nH * a.I + 4 * cl) * ES)
+                                                        : (uint32_t)((GROWS * g * w_pstride + 4 * c) * ES));
   const uint32_t s_voff = (STAGE == 1) ? (uint32_t)(g * w_pstride + hcol * nH * a.I + 4 * cl)
                                        : (uint32_t)(g * w_pstride + 4 * c);
+  // bytes of one expert's weights: the reference layout's, or col_tiles x nks runs of 32 KB
+  const int64_t w_expert_bytes = pk * ((int64_t)a.col_tiles * nks * 32768) +
+                                 npk * ((STAGE == 1) ? 128 * w_pstride * ES : (int64_t)a.pI * w_pstride * ES);
   v4i rw_, rs_;  // the expert's weights and scales
 
   // A K slice's loads, numbered in issue order:
@@ -591,12 +601,12 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     int64_t colu;
     if (STAGE == 1) {
       colu = (int64_t)tile_tI(t) * 512 + (int64_t)q * tile_Pt(t) + tile_p0(t);
-      rw_ = make_rsrc(Wb + (int64_t)t.e * 128 * w_pstride * ES, (uint32_t)(128 * w_pstride * ES));
+      rw_ = make_rsrc(Wb + (int64_t)t.e * w_expert_bytes, (uint32_t)w_expert_bytes);
       rs_ = make_rsrc(a.W_scale + (int64_t)(a.w_scale_shared ? 0 : t.e) * 16 * w_pstride, (uint32_t)(16 * w_pstride));
     } else {
       colu = tile_h0(t) + 64 * q;
       const int64_t sp = (a.pI + 7) / 8;
-      rw_ = make_rsrc(Wb + (int64_t)t.e * a.pI * w_pstride * ES, (uint32_t)(a.pI * w_pstride * ES));
+      rw_ = make_rsrc(Wb + (int64_t)t.e * w_expert_bytes, (uint32_t)w_expert_bytes);
       rs_ = make_rsrc(a.W_scale + (int64_t)(a.w_scale_shared ? 0 : t.e) * sp * w_pstride, (uint32_t)(sp * w_pstride));
     }
     rw_rec = rw_[2];
@@ -604,7 +614,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
     for (int i = 0; i < NBL; ++i) {
       const int pr = FP4 ? i : ((i < 4) ? i : (16 + i - 4));
-      w_soff[i] = uni(((int64_t)pr * w_pstride + colu) * ES);
+      w_soff[i] = uni(pk * (((t.xt * nks) * 4 + q) * 8192 + i * 1024) + npk * (int)(((int64_t)pr * w_pstride + colu) * ES));
     }
     s_soff = uni(colu);
   };
@@ -630,7 +640,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     const int kt = ks >> 2, pb = ks & 3;
     r.a_off = ks * 128;
     r.as_off = ks * 4;
-    r.w_off = uni(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * ES);
+    r.w_off = uni(pk * (ks * 32768) + npk * (int)(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * ES));
     r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
@@ -1130,10 +1140,11 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   __shared__ __attribute__((aligned(16))) float s_rs[2][WFMT == MX_WFMT_ROW8 ? MX_ROWS_MAX : 4];
   __shared__ __attribute__((aligned(16))) float s_wsc[2][WFMT == MX_WFMT_ROW8 ? MXT : 4];
   // One workgroup per CU, for the whole launch.  Workgroups are handed to the 8 XCDs round-robin by linear
-  // index, and each XCD has its own L2.  XCD x therefore takes the x-th contiguous eighth of the chunk list
-  // (chunks are ordered by expert), as a queue of items (chunk, column tile) with the column tiles innermost
-  // and the chunks grouped by class; its workgroups take the items w, w + W, w + 2W, ... (W workgroups on the
-  // XCD).  The workgroups that share an activation tile, and the chunks that share an expert's weights, then run
+  // index, and each XCD has its own L2.  XCD x therefore takes the x-th of eight contiguous parts of the chunk
+  // list (chunks are ordered by expert; the parts hold about equal work), as a queue of items (chunk, column
+  // tile) with the chunks grouped by class and, inside a class, the column tiles innermost (or alternating between
+  // a few chunks of one expert, see tile_at); its workgroups take the items w, w + W, w + 2W, ... (W workgroups on
+  // the XCD).  The workgroups that share an activation tile, and the chunks that share an expert's weights, then run
   // at the same time behind the same L2, so each operand crosses the fabric about once; and a workgroup's
   // consecutive items are of one class, i.e. one instance of the code below, which carries its loads from tile
   // to tile.
@@ -1177,6 +1188,39 @@ int MX_CAT(launch_mx_gemm_s, MX_INST_STAGE, _f, MX_INST_WFMT)(const MxArgs& m, u
 }
 
 #else  // dispatcher
+
+// The gate/up weights in the kernel's read order (see launch_mx_pack_weights in bwmm.hpp).  One thread per 16-byte
+// piece; the source address is what mx_gemm_tiles<1, ...> computes for that load (w_voff + w_soff[i] + w_off).
+__global__ __launch_bounds__(256) void mx_pack_weights_kernel(const uint8_t* __restrict__ W, uint4* __restrict__ dst,
+                                                              int64_t H, int64_t I, int64_t col_tiles, int64_t nks,
+                                                              int64_t pieces) {
+  const int64_t d = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (d >= pieces) return;
+  const int lane = (int)(d & 63), i = (int)((d >> 6) & 7), q = (int)((d >> 9) & 3);
+  const int64_t ks = (d >> 11) % nks, xt = ((d >> 11) / nks) % col_tiles, e = (d >> 11) / (nks * col_tiles);
+  const int g = lane >> 4, c = lane & 15;
+  const int64_t pr = (i < 4) ? i : (16 + i - 4), kt = ks >> 2, pb = ks & 3;
+  const int64_t nH = H / 512, pstride = 2 * nH * I;
+  const int64_t tI = xt >> 2, p0 = (xt & 3) * 32;
+  const int64_t rows_t = (I - tI * 512 < 512) ? (I - tI * 512) : 512;
+  const int64_t colu = tI * 512 + q * (rows_t / 4) + p0;
+  const int64_t elem = (4 * g + pr + pb * 32) * pstride + (c >> 3) * nH * I + 4 * (c & 7) + colu + kt * I;
+  dst[d] = *(const uint4*)(W + (e * 128 * pstride + elem) * 4);
+}
+
+size_t mx_packed_weights_bytes(int64_t E, int64_t H, int64_t I) {
+  return (size_t)E * ((I / 512) * 4 + (I % 512) / 128) * (H / 128) * 32768;
+}
+int launch_mx_pack_weights(const void* W, void* dst, int64_t E, int64_t H, int64_t I, hipStream_t s) {
+  if (!mx_fast_path_ok(H, I) || (((uintptr_t)W) & 15) != 0 || (((uintptr_t)dst) & 15) != 0) return MOE_E_BAD_ARG;
+  const int64_t ct = (I / 512) * 4 + (I % 512) / 128, nks = H / 128;
+  const int64_t pieces = E * ct * nks * 2048;
+  if ((pieces + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
+  hipLaunchKernelGGL(mx_pack_weights_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s,
+                     (const uint8_t*)W, (uint4*)dst, H, I, ct, nks, pieces);
+  MOE_CHECK_LAUNCH();
+  return MOE_OK;
+}
 
 int launch_mx_gemm_s1_f0(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f0(const MxArgs& m, unsigned grid, hipStream_t s);

@@ -137,6 +137,7 @@ def _bwmm_shard_on_block_mx(
         expert_affinities_scaling_mode=expert_affinities_scaling_mode,
         gate_clamp_upper_limit=gate_clamp_upper_limit, gate_clamp_lower_limit=gate_clamp_lower_limit,
         up_clamp_upper_limit=up_clamp_upper_limit, up_clamp_lower_limit=up_clamp_lower_limit, weight_dtype=wdt,
+        weight_objects=(gate_up_proj_weight, down_proj_weight),
     )
 
 

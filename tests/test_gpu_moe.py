@@ -366,6 +366,29 @@ def test_fp8_row_scale_modes_and_clamps(mode, clamp, act, I, shared):
     _check(o[:T], g[:T], f"fp8 row mode={mode} clamp={clamp} act={act} I={I} shared={shared}")
 
 
+@pytest.mark.parametrize("T,H,I,E,k,B,fmt", [(512, 1024, 640, 8, 2, 128, "e4m3"), (300, 512, 1024, 2, 2, 256, "e5m2"),
+                                             (256, 512, 128, 4, 2, 128, "e4m3")])
+def test_mx_weight_copies_are_bit_equal(T, H, I, E, k, B, fmt):
+    """Copies of the 8-bit MX weights in the kernels' read order (``_launch.mx_weight_copies``): same bits out as from
+    the reference layout, for full and short intermediate tiles, several chunks per expert, both 8-bit formats."""
+    import torch
+    from nkilib.core.moe.moe_cte import _launch
+
+    c = mx_case(T, H, I, E, k, B, seed=51, bias=True, weight_format=fmt, random_codes=True)
+    was = _launch.mx_weight_copies
+    try:
+        _launch.mx_weight_copies = False
+        plain = _run_mx_options(c, 3, REF_MX_CLAMPS, False)
+        _launch.clear_kmajor_weight_cache()
+        _launch.mx_weight_copies = True
+        first = _run_mx_options(c, 3, REF_MX_CLAMPS, False)
+        assert torch.equal(first, plain)
+    finally:
+        _launch.mx_weight_copies = was
+        _launch.clear_kmajor_weight_cache()
+    _check(from_bf16_tensor(plain)[0, :T], _golden_mx_options(c, 3, REF_MX_CLAMPS)[:T], f"mx copies {fmt} I={I}")
+
+
 def _run_mx(c, prequant=False, act=0, weight_dtype=None):
     import torch
     from nkilib.core.moe.moe_cte import QuantizationConfig, SkipMode, moe_cte
