@@ -251,10 +251,11 @@ typedef struct moe_bwmm_args {
   /* Optional K-contiguous copies of the bf16 / fp8 weights of the BF16 and FP8_ROW kinds, made once by
    * moe_prepare_kmajor_weights (they depend on the weights only).  Both NULL: every call makes its own copies
    * in the workspace.  MXFP8 kind: the x4 layouts are K-major already and are read in place when both are NULL;
-   * for 8-bit weights on shapes with H % 512 == 0 and I % 128 == 0 the same two calls make a copy of the gate/up
-   * weights in the order the kernel reads them (each workgroup then reads its weights as contiguous 32 KB runs:
-   * the gate/up GEMM is 5 % faster at H = 7168, I = 2048, for a second copy of those weights in memory); used when
-   * gate_up_proj_weight_kmajor is set.  There is no such copy of the down weights (size 0, pointer ignored). */
+   * on shapes with H % 512 == 0 and I % 128 == 0 the same two calls make a copy of the gate/up weights in the
+   * order the kernel reads them (each workgroup then reads its weights as contiguous 32 KB runs: the gate/up GEMM
+   * is 5 % faster at H = 7168, I = 2048 with 8-bit weights, for a second copy of those weights in memory); used
+   * when gate_up_proj_weight_kmajor is set.  A copy of the down weights exists for 4-bit weights only
+   * (moe_kmajor_weights_bytes(args, 1) is 0 otherwise and the pointer is ignored). */
   const void* gate_up_proj_weight_kmajor;
   const void* down_proj_weight_kmajor;
   /* Nullable.  The reference's two-shard kernels return [T1, 2, H] or [2, T1, H] with the sum in shard 0 and

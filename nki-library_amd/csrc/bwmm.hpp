@@ -69,7 +69,7 @@ struct MxArgs {
   float clamp[4];
   int32_t col_tiles;       // column tiles per chunk (set by the launcher)
   int32_t wfmt;            // element format of the weights, MX_WFMT_*
-  int32_t w_packed;        // 1 (gate/up): W is a copy of the 8-bit weights in the kernel's read order (launch_mx_pack_weights)
+  int32_t w_packed;        // 1: W is a copy of the weights in the kernel's read order (launch_mx_pack_weights)
   // MX_WFMT_ROW8 (the fp8-row kind on these kernels): e4m3 operands whose E8M0 tables are constants of 127, a
   // per-row fp32 scale of the activations and a per-output-channel fp32 scale of the weights in the epilogue
   const float* w_cscale;   // [cscale_experts][2*I] (gate/up: gate then up) or [cscale_experts][H] (down)
@@ -89,11 +89,11 @@ constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1, MX_WFMT_E2M1 = 2, MX_WFMT_ROW8
 // of 32 partitions (I % 128 == 0); other shapes run the general kernel.
 inline bool mx_fast_path_ok(int64_t H, int64_t I) { return H % 512 == 0 && I % 128 == 0; }
 int launch_mx_gemm(int stage, const MxArgs& m, unsigned gx, unsigned gy, hipStream_t s);
-// Copy of the 8-bit x4 gate/up weights in the order the large-tile kernel reads them: for expert e, column tile xt,
-// K slice ks, wave q, load i, lane l the 16 bytes that the lane's i-th load of that slice fetches, at
-// ((((e * col_tiles + xt) * nks + ks) * 4 + q) * 8 + i) * 1024 + 16 * l.  Same size as the reference layout.
-int launch_mx_pack_weights(const void* W, void* dst, int64_t E, int64_t H, int64_t I, hipStream_t s);
-size_t mx_packed_weights_bytes(int64_t E, int64_t H, int64_t I);
+// Copy of the x4 weights of one stage (1 gate/up, 2 down) in the order the large-tile kernel reads them: for expert
+// e, column tile xt, K slice ks, wave q, load i, lane l the 16 bytes (4-bit weights: 8) that the lane's i-th load of
+// that slice fetches, at ((((e * col_tiles + xt) * nks + ks) * 4 + q) * 8 + i) * 64 + l such pieces.
+int launch_mx_pack_weights(int stage, int fp4, const void* W, void* dst, int64_t E, int64_t H, int64_t I, hipStream_t s);
+size_t mx_packed_weights_bytes(int stage, int fp4, int64_t E, int64_t H, int64_t I);
 
 int launch_gemm_stage(int kind, int stage, const GemmArgs& g, unsigned gx, unsigned gy, hipStream_t s);
 // batches [nb0][nb1] of byte matrices [R, C] -> [C, Kp] (K-contiguous, zero tail), see bwmm.hip

@@ -530,19 +530,24 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // element strides (4-byte weights; scales use the same counts in bytes)
   const int64_t w_pstride = (STAGE == 1) ? 2 * nH * a.I : (int64_t)a.nI * a.H;
   const int64_t w_tstride = (STAGE == 1) ? a.I : a.H;
-  // a.w_packed (gate/up only): the weights are a copy in the order these loads read them (see mx_pack_weights_kernel): load i of
-  // wave q in slice ks of column tile xt is 1 KB at ((xt * nks + ks) * 4 + q) * 8 KB + i * 1 KB of the expert's
-  // copy, a lane's 16 bytes at 16 * lane: each workgroup reads its weights as one contiguous 32 KB run per slice.
+  // a.w_packed: the weights are a copy in the order these loads read them (see mx_pack_weights_kernel): load i of
+  // wave q in slice ks of column tile xt is 1 KB (4-bit weights: 512 bytes) at ((xt * nks + ks) * 4 + q) * 8 + i
+  // such units into the expert's copy, a lane's 16 (8) bytes in lane order: each workgroup reads its weights as one
+  // contiguous 32 (16) KB run per slice.
   // (the two address forms are blended with the 0 / 1 flag as a factor: a conditional expression here may become
   // a branch, and values that cross a branch in this function are no longer known to the compiler as uniform)
   const int pk = a.w_packed ? 1 : 0, npk = 1 - pk;
-  const uint32_t w_voff = (uint32_t)pk * (uint32_t)(lane * 16) +
+  constexpr int PK_LANE = FP4 ? 8 : 16;        // bytes a lane loads
+  constexpr int PK_LOAD = 64 * PK_LANE;         // ... a load instruction
+  constexpr int PK_WAVE = 8 * PK_LOAD;          // ... a wave per K slice
+  constexpr int PK_SLICE = 4 * PK_WAVE;         // ... the workgroup per K slice
+  const uint32_t w_voff = (uint32_t)pk * (uint32_t)(lane * PK_LANE) +
                           (uint32_t)npk * ((STAGE == 1) ? (uint32_t)((GROWS * g * w_pstride + hcol * nH * a.I + 4 * cl) * ES)
                                                         : (uint32_t)((GROWS * g * w_pstride + 4 * c) * ES));
   const uint32_t s_voff = (STAGE == 1) ? (uint32_t)(g * w_pstride + hcol * nH * a.I + 4 * cl)
                                        : (uint32_t)(g * w_pstride + 4 * c);
   // bytes of one expert's weights: the reference layout's, or col_tiles x nks runs of 32 KB
-  const int64_t w_expert_bytes = pk * ((int64_t)a.col_tiles * nks * 32768) +
+  const int64_t w_expert_bytes = pk * ((int64_t)a.col_tiles * nks * PK_SLICE) +
                                  npk * ((STAGE == 1) ? 128 * w_pstride * ES : (int64_t)a.pI * w_pstride * ES);
   v4i rw_, rs_;  // the expert's weights and scales
 
@@ -614,7 +619,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
     for (int i = 0; i < NBL; ++i) {
       const int pr = FP4 ? i : ((i < 4) ? i : (16 + i - 4));
-      w_soff[i] = uni(pk * (((t.xt * nks) * 4 + q) * 8192 + i * 1024) + npk * (int)(((int64_t)pr * w_pstride + colu) * ES));
+      w_soff[i] = uni(pk * (((t.xt * nks) * 4 + q) * PK_WAVE + i * PK_LOAD) + npk * (int)(((int64_t)pr * w_pstride + colu) * ES));
     }
     s_soff = uni(colu);
   };
@@ -640,7 +645,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     const int kt = ks >> 2, pb = ks & 3;
     r.a_off = ks * 128;
     r.as_off = ks * 4;
-    r.w_off = uni(pk * (ks * 32768) + npk * (int)(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * ES));
+    r.w_off = uni(pk * (ks * PK_SLICE) + npk * (int)(((int64_t)(pb * 32) * w_pstride + (int64_t)kt * w_tstride) * ES));
     r.s_off = uni((int64_t)(pb * 4) * w_pstride + (int64_t)kt * w_tstride);
     return r;
   };
@@ -1189,35 +1194,63 @@ int MX_CAT(launch_mx_gemm_s, MX_INST_STAGE, _f, MX_INST_WFMT)(const MxArgs& m, u
 
 #else  // dispatcher
 
-// The gate/up weights in the kernel's read order (see launch_mx_pack_weights in bwmm.hpp).  One thread per 16-byte
-// piece; the source address is what mx_gemm_tiles<1, ...> computes for that load (w_voff + w_soff[i] + w_off).
-__global__ __launch_bounds__(256) void mx_pack_weights_kernel(const uint8_t* __restrict__ W, uint4* __restrict__ dst,
-                                                              int64_t H, int64_t I, int64_t col_tiles, int64_t nks,
-                                                              int64_t pieces) {
+// The weights of one stage in the kernel's read order (see launch_mx_pack_weights in bwmm.hpp).  One thread per
+// lane-sized piece (16 bytes, 8 for 4-bit weights); the source address is what mx_gemm_tiles computes for that load
+// (w_voff + w_soff[i] + w_off).
+template <int LB>
+__global__ __launch_bounds__(256) void mx_pack_weights_kernel(int stage, const uint8_t* __restrict__ W,
+                                                              uint8_t* __restrict__ dst, int64_t H, int64_t I,
+                                                              int64_t col_tiles, int64_t nks, int64_t pieces) {
+  constexpr bool FP4 = LB == 8;
+  constexpr int ES = FP4 ? 2 : 4, GROWS = FP4 ? 8 : 4;
   const int64_t d = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (d >= pieces) return;
   const int lane = (int)(d & 63), i = (int)((d >> 6) & 7), q = (int)((d >> 9) & 3);
   const int64_t ks = (d >> 11) % nks, xt = ((d >> 11) / nks) % col_tiles, e = (d >> 11) / (nks * col_tiles);
   const int g = lane >> 4, c = lane & 15;
-  const int64_t pr = (i < 4) ? i : (16 + i - 4), kt = ks >> 2, pb = ks & 3;
-  const int64_t nH = H / 512, pstride = 2 * nH * I;
-  const int64_t tI = xt >> 2, p0 = (xt & 3) * 32;
-  const int64_t rows_t = (I - tI * 512 < 512) ? (I - tI * 512) : 512;
-  const int64_t colu = tI * 512 + q * (rows_t / 4) + p0;
-  const int64_t elem = (4 * g + pr + pb * 32) * pstride + (c >> 3) * nH * I + 4 * (c & 7) + colu + kt * I;
-  dst[d] = *(const uint4*)(W + (e * 128 * pstride + elem) * 4);
+  const int64_t pr = FP4 ? i : ((i < 4) ? i : (16 + i - 4)), kt = ks >> 2, pb = ks & 3;
+  int64_t elem, expert_elems;
+  if (stage == 1) {
+    const int64_t nH = H / 512, pstride = 2 * nH * I;
+    const int64_t tI = xt >> 2, p0 = (xt & 3) * 32;
+    const int64_t rows_t = (I - tI * 512 < 512) ? (I - tI * 512) : 512;
+    const int64_t colu = tI * 512 + q * (rows_t / 4) + p0;
+    elem = (GROWS * g + pr + pb * 32) * pstride + (c >> 3) * nH * I + 4 * (c & 7) + colu + kt * I;
+    expert_elems = 128 * pstride;
+  } else {
+    const int64_t nI = (I + 511) / 512, pI = I > 512 ? 128 : I / 4, pstride = nI * H;
+    elem = (GROWS * g + pr + pb * 32) * pstride + 4 * c + xt * 256 + 64 * q + kt * H;
+    expert_elems = pI * pstride;
+  }
+  const uint8_t* src = W + (e * expert_elems + elem) * ES;
+  if constexpr (FP4) *(uint2*)(dst + d * LB) = *(const uint2*)src;
+  else *(uint4*)(dst + d * LB) = *(const uint4*)src;
 }
 
-size_t mx_packed_weights_bytes(int64_t E, int64_t H, int64_t I) {
-  return (size_t)E * ((I / 512) * 4 + (I % 512) / 128) * (H / 128) * 32768;
+static void mx_pack_geometry(int stage, int64_t H, int64_t I, int64_t* col_tiles, int64_t* nks) {
+  const int64_t over_i = (I / 512) * 4 + (I % 512) / 128;
+  *col_tiles = stage == 1 ? over_i : H / 256;
+  *nks = stage == 1 ? H / 128 : over_i;
 }
-int launch_mx_pack_weights(const void* W, void* dst, int64_t E, int64_t H, int64_t I, hipStream_t s) {
+size_t mx_packed_weights_bytes(int stage, int fp4, int64_t E, int64_t H, int64_t I) {
+  int64_t ct, nks;
+  mx_pack_geometry(stage, H, I, &ct, &nks);
+  return (size_t)E * ct * nks * (fp4 ? 16384 : 32768);
+}
+int launch_mx_pack_weights(int stage, int fp4, const void* W, void* dst, int64_t E, int64_t H, int64_t I,
+                           hipStream_t s) {
   if (!mx_fast_path_ok(H, I) || (((uintptr_t)W) & 15) != 0 || (((uintptr_t)dst) & 15) != 0) return MOE_E_BAD_ARG;
-  const int64_t ct = (I / 512) * 4 + (I % 512) / 128, nks = H / 128;
+  int64_t ct, nks;
+  mx_pack_geometry(stage, H, I, &ct, &nks);
   const int64_t pieces = E * ct * nks * 2048;
   if ((pieces + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
-  hipLaunchKernelGGL(mx_pack_weights_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s,
-                     (const uint8_t*)W, (uint4*)dst, H, I, ct, nks, pieces);
+  const dim3 grid((unsigned)((pieces + 255) / 256));
+  if (fp4)
+    hipLaunchKernelGGL(mx_pack_weights_kernel<8>, grid, dim3(256), 0, s, stage, (const uint8_t*)W, (uint8_t*)dst, H, I,
+                       ct, nks, pieces);
+  else
+    hipLaunchKernelGGL(mx_pack_weights_kernel<16>, grid, dim3(256), 0, s, stage, (const uint8_t*)W, (uint8_t*)dst, H, I,
+                       ct, nks, pieces);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
 }

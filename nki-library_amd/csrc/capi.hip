@@ -226,15 +226,19 @@ int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hip
 
 }  // namespace
 
-// MXFP8 kind: copies exist for 8-bit weights on the large-tile path (the weights in the kernels' read order)
-static bool mx_packable(const moe_bwmm_args* a) {
-  return a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I) && a->weight_dtype != MOE_DT_FP4_E2M1;
+// MXFP8 kind: copies of the weights in the kernels' read order exist on the large-tile path: of the gate/up weights
+// for every format, of the down weights for 4-bit ones (whose pieces in the reference layout are 512 bytes; the
+// 8-bit ones' 1 KB pieces were measured no slower than a copy).
+static bool mx_packable(const moe_bwmm_args* a, int which) {
+  if (a->kind != MOE_KIND_MXFP8 || !mx_fast_path_ok(a->H, a->I)) return false;
+  return which == 0 || a->weight_dtype == MOE_DT_FP4_E2M1;
 }
 
 extern "C" size_t moe_kmajor_weights_bytes(const moe_bwmm_args* a, int which) {
   if (validate(a) != MOE_OK || which < 0 || which > 1) return 0;
-  // (MXFP8: the gate/up weights only -- the down GEMM was measured no faster on such a copy)
-  if (a->kind == MOE_KIND_MXFP8) return (mx_packable(a) && which == 0) ? mx_packed_weights_bytes(a->E, a->H, a->I) : 0;
+  if (a->kind == MOE_KIND_MXFP8)
+    return mx_packable(a, which) ? mx_packed_weights_bytes(which + 1, a->weight_dtype == MOE_DT_FP4_E2M1, a->E, a->H, a->I)
+                                 : 0;
   const Plan p = make_plan(a);
   const size_t es = a->kind == MOE_KIND_BF16 ? 2 : 1;
   if (row8_fast(a)) return row8_copy(a, which).total;
@@ -244,10 +248,14 @@ extern "C" size_t moe_kmajor_weights_bytes(const moe_bwmm_args* a, int which) {
 extern "C" int moe_prepare_kmajor_weights(const moe_bwmm_args* a, void* gate_up_kmajor, void* down_kmajor, void* stream) {
   int rc = validate(a);
   if (rc != MOE_OK) return rc;
-  if (a->kind == MOE_KIND_MXFP8) {  // gate/up only; down_kmajor is not used
-    if (!mx_packable(a)) return MOE_E_UNSUPPORTED;
+  if (a->kind == MOE_KIND_MXFP8) {  // down_kmajor is used where moe_kmajor_weights_bytes(a, 1) is not 0
+    if (!mx_packable(a, 0)) return MOE_E_UNSUPPORTED;
+    const int fp4 = a->weight_dtype == MOE_DT_FP4_E2M1;
     if (!gate_up_kmajor || (((uintptr_t)gate_up_kmajor) & 255) != 0) return MOE_E_BAD_ARG;
-    return launch_mx_pack_weights(a->gate_up_proj_weight, gate_up_kmajor, a->E, a->H, a->I, (hipStream_t)stream);
+    rc = launch_mx_pack_weights(1, fp4, a->gate_up_proj_weight, gate_up_kmajor, a->E, a->H, a->I, (hipStream_t)stream);
+    if (rc != MOE_OK || !mx_packable(a, 1)) return rc;
+    if (!down_kmajor || (((uintptr_t)down_kmajor) & 255) != 0) return MOE_E_BAD_ARG;
+    return launch_mx_pack_weights(2, fp4, a->down_proj_weight, down_kmajor, a->E, a->H, a->I, (hipStream_t)stream);
   }
   if (!gate_up_kmajor || !down_kmajor) return MOE_E_BAD_ARG;
   if ((((uintptr_t)gate_up_kmajor) & 255) != 0 || (((uintptr_t)down_kmajor) & 255) != 0) return MOE_E_BAD_ARG;
@@ -422,7 +430,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
       m1.a_rows = n_real;
       m1.W = (const uint32_t*)a->gate_up_proj_weight; m1.W_scale = (const uint8_t*)a->gate_up_proj_scale;
       m1.bias = a->gate_and_up_proj_bias;
-      if (mx_packable(a) && a->gate_up_proj_weight_kmajor) {
+      if (mx_packable(a, 0) && a->gate_up_proj_weight_kmajor) {
         m1.W = (const uint32_t*)a->gate_up_proj_weight_kmajor;
         m1.w_packed = 1;
       }
@@ -451,6 +459,10 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
       m2.a_rows = a->N * a->B;
       m2.W = (const uint32_t*)a->down_proj_weight; m2.W_scale = (const uint8_t*)a->down_proj_scale;
       m2.bias = a->down_proj_bias;
+      if (mx_packable(a, 1) && a->down_proj_weight_kmajor) {
+        m2.W = (const uint32_t*)a->down_proj_weight_kmajor;
+        m2.w_packed = 1;
+      }
       if (r8_fast) {
         const Row8Copy c = row8_copy(a, 1);
         m2.W = (const uint32_t*)g2.W;

@@ -367,10 +367,12 @@ def test_fp8_row_scale_modes_and_clamps(mode, clamp, act, I, shared):
 
 
 @pytest.mark.parametrize("T,H,I,E,k,B,fmt", [(512, 1024, 640, 8, 2, 128, "e4m3"), (300, 512, 1024, 2, 2, 256, "e5m2"),
-                                             (256, 512, 128, 4, 2, 128, "e4m3")])
+                                             (256, 512, 128, 4, 2, 128, "e4m3"), (512, 1024, 640, 8, 2, 128, "e2m1"),
+                                             (300, 512, 1024, 2, 2, 256, "e2m1")])
 def test_mx_weight_copies_are_bit_equal(T, H, I, E, k, B, fmt):
-    """Copies of the 8-bit MX weights in the kernels' read order (``_launch.mx_weight_copies``): same bits out as from
-    the reference layout, for full and short intermediate tiles, several chunks per expert, both 8-bit formats."""
+    """Copies of the MX weights in the kernels' read order (``_launch.mx_weight_copies``: gate/up for every format, down
+    for 4-bit weights): same bits out as from the reference layout, for full and short intermediate tiles and several
+    chunks per expert."""
     import torch
     from nkilib.core.moe.moe_cte import _launch
 
