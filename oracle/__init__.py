@@ -24,6 +24,11 @@ Parity unpinned (no source, fixture or mathematical fact fixes them):
     returns (the reference's bf16 logits tie often); the oracle selects on
     fp32 logits and breaks ties towards the lower expert index.
 
+  * the fp8-row kind under PRE_SCALE / NO_SCALE and with clamps
+    (``moe.moe_blockwise_fp8_row_ref``): the reference has no kernel with fp8
+    activations on this path; the rule is the dense golden's applied to the
+    row-quantised operands (the affinity scales the row's dequantisation scale).
+
 Modules
   numerics   bf16 / fp8-e4m3fn / E8M0 encode + decode
   mx         OCP-MX (8x4 block) quantise / dequantise / matmul goldens
