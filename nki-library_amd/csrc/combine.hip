@@ -114,7 +114,8 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   // with many rows each): that average, up to 8, i.e. the item order of a class alternates between G neighbouring
   // chunks, which are then mostly chunks of one expert: they work on the same weight tile at the same time and
   // share it through the L2 instead of streaming it from memory once per chunk.  (Applied to a skewed router's
-  // few hot experts among many single-chunk ones it costs more in activation sharing than it saves: measured.)
+  // few hot experts among many single-chunk ones it costs more in activation sharing than it saves, and at two
+  // chunks per expert on average it changes nothing: both measured.)
   const int avg = s_runs > 0 ? (n + s_runs / 2) / s_runs : 1;
   const int interleave = avg < 3 ? 1 : (avg > 8 ? 8 : avg);
   if (threadIdx.x == 0) q_off[8 * (CHUNK_CLASSES + 1)] = interleave;
@@ -151,7 +152,14 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     const bool last = interleave == 1 && ((i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]));
     return chunk_xcd[i] * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
   };
-  for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&s_cnt[key_of(i)], 1);
+  // (the keys of up to 4096 chunks are kept in LDS for the rank loop below)
+  constexpr int KEYS_IN_LDS = 4096;
+  __shared__ uint8_t s_key[KEYS_IN_LDS];
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int key = key_of(i);
+    if (i < KEYS_IN_LDS) s_key[i] = (uint8_t)key;
+    atomicAdd(&s_cnt[key], 1);
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
     int run = 0;
@@ -175,7 +183,11 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
       pos = atomicAdd(&s_cnt[key], 1);
     } else {
       int rank = 0;
-      for (int j = 0; j < i; ++j) rank += key_of(j) == key;
+      if (n <= KEYS_IN_LDS) {
+        for (int j = 0; j < i; ++j) rank += s_key[j] == key;
+      } else {
+        for (int j = 0; j < i; ++j) rank += key_of(j) == key;
+      }
       pos = s_cnt[key] + rank;
     }
     q_chunk[2 * pos] = chunk_slot[i];
