@@ -117,7 +117,9 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   // few hot experts among many single-chunk ones it costs more in activation sharing than it saves, and at two
   // chunks per expert on average it changes nothing: both measured.)
   const int avg = s_runs > 0 ? (n + s_runs / 2) / s_runs : 1;
-  const int interleave = avg < 3 ? 1 : (avg > 8 ? 8 : avg);
+  // (not beyond the number of chunks whose keys fit in LDS for the rank order below)
+  constexpr int KEYS_IN_LDS = 4096;
+  const int interleave = (avg < 3 || n > KEYS_IN_LDS) ? 1 : (avg > 8 ? 8 : avg);
   if (threadIdx.x == 0) q_off[8 * (CHUNK_CLASSES + 1)] = interleave;
   for (int i = threadIdx.x; i <= 8 * CHUNK_CLASSES; i += blockDim.x) s_cnt[i] = 0;
   // Which XCD takes which chunks: contiguous parts of the list (chunks of one expert, and experts that follow each
@@ -152,9 +154,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     const bool last = interleave == 1 && ((i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]));
     return chunk_xcd[i] * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
   };
-  // (the keys of up to 4096 chunks are kept in LDS for the rank loop below)
-  constexpr int KEYS_IN_LDS = 4096;
-  __shared__ uint8_t s_key[KEYS_IN_LDS];
+  __shared__ uint8_t s_key[KEYS_IN_LDS];  // the chunks' keys, for the rank loop below
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     const int key = key_of(i);
     if (i < KEYS_IN_LDS) s_key[i] = (uint8_t)key;
@@ -183,11 +183,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
       pos = atomicAdd(&s_cnt[key], 1);
     } else {
       int rank = 0;
-      if (n <= KEYS_IN_LDS) {
-        for (int j = 0; j < i; ++j) rank += s_key[j] == key;
-      } else {
-        for (int j = 0; j < i; ++j) rank += key_of(j) == key;
-      }
+      for (int j = 0; j < i; ++j) rank += s_key[j] == key;
       pos = s_cnt[key] + rank;
     }
     q_chunk[2 * pos] = chunk_slot[i];
