@@ -91,6 +91,25 @@ def test_row_quant(rows, H, quant_only, kind, lower_bound):
         assert (codes == 0x77).all()  # 240.0
 
 
+@pytest.mark.parametrize("rows,H,lower_bound", [(3, 512, 0.0), (130, 2048, 0.0), (257, 4096, 0.5), (33, 7168, 0.0),
+                                                (9, 8200, 0.0), (17, 16384, 0.5)])
+def test_row_quant_bf16_kernel_equals_the_general_one(rows, H, lower_bound):
+    """bf16 input with bf16 gamma runs a specialised kernel; the same gamma values held as fp32 run the general one.
+    Both do the same arithmetic in the same order: records equal byte for byte (codes and scale)."""
+    import torch
+    from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
+
+    rng = np.random.default_rng(7)
+    x, g = _gen("gauss", rows, H, rng)
+    x[0, 0, :5] = 0.0
+    dev = torch.device("cuda:0")
+    kargs = RmsNormQuantKernelArgs(lower_bound=lower_bound)
+    xt, gt = bf16_tensor(x, dev), bf16_tensor(g, dev)
+    fast = rmsnorm_quant_kernel(xt, gt, kargs).view(torch.uint8)
+    general = rmsnorm_quant_kernel(xt, gt.float(), kargs).view(torch.uint8)
+    assert torch.equal(fast, general)
+
+
 @pytest.mark.parametrize("rows,H,quant_only", [(2, 16384, True), (160, 16384, False), (64, 4096, False)])
 def test_static_quant(rows, H, quant_only):
     import torch
