@@ -65,6 +65,24 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
                                              int32_t* __restrict__ chunk_xcd, int32_t* __restrict__ q_chunk,
                                              int32_t* __restrict__ q_off, int64_t max_chunks, int* s_ws) {
   const int64_t na = *n_active;
+  // The walk along a run below is a chain of dependent reads, one block after the other: from LDS when the active
+  // blocks fit there (a global read per step made the run length the pace of this kernel).
+  constexpr int BLOCKS_IN_LDS = 4096;
+  __shared__ int s_e[BLOCKS_IN_LDS], s_v[BLOCKS_IN_LDS];
+  const bool staged = na <= BLOCKS_IN_LDS;
+  if (staged) {
+    for (int64_t j = threadIdx.x; j < na; j += blockDim.x) {
+      s_e[j] = b2e[j];
+      s_v[j] = valid_rows[j];
+    }
+    __syncthreads();
+  }
+  auto expert_of = [&](int64_t j) { return staged ? s_e[j] : b2e[j]; };
+  auto valid_of = [&](int64_t j) { return staged ? s_v[j] : valid_rows[j]; };
+  // The chunk list as the later steps of this function read it: from LDS as well while it fits (each step would
+  // otherwise begin with a round trip to the L2 for what the step before has just written).
+  constexpr int CHUNKS_IN_LDS = 2048;
+  __shared__ int s_cslot[CHUNKS_IN_LDS], s_cre[CHUNKS_IN_LDS], s_cx[CHUNKS_IN_LDS];
   int carry = 0;
   int runs = 0;  // runs that hold chunks (over this thread's runs)
   for (int64_t b0 = 0; b0 < na; b0 += 1024) {
@@ -73,11 +91,13 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     int64_t last_end = -1;
     int e = -1;
     if (b < na) {
-      e = b2e[b];
-      const bool start = (b == 0) || (b2e[b - 1] != e);
+      e = expert_of(b);
+      const bool start = (b == 0) || (expert_of(b - 1) != e);
       if (start && e >= 0 && e < E) {
-        for (int64_t j = b; j < na && b2e[j] == e; ++j)
-          if (valid_rows[j] > 0) last_end = j * B + valid_rows[j];
+        for (int64_t j = b; j < na && expert_of(j) == e; ++j) {
+          const int v = valid_of(j);
+          if (v > 0) last_end = j * B + v;
+        }
         // chunks of CHUNK_ROWS rows; the last one absorbs a remainder of up to CHUNK_ROWS_MAX - CHUNK_ROWS
         // rows, which saves the pass over the expert's weights that a small chunk of its own would cost
         const int64_t len = last_end - b * B;
@@ -89,10 +109,15 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     const int base = carry + block_excl_scan(nch, s_ws, &total);
     for (int k = 0; k < nch; ++k) {
       const int64_t s0 = b * B + (int64_t)k * CHUNK_ROWS;
+      const int32_t rows = (int32_t)((k + 1 < nch) ? CHUNK_ROWS : (last_end - s0));
       if (base + k < max_chunks) {
         chunk_slot[base + k] = (int32_t)s0;
-        chunk_rows[base + k] = (int32_t)((k + 1 < nch) ? CHUNK_ROWS : (last_end - s0));
+        chunk_rows[base + k] = rows;
         chunk_expert[base + k] = e;
+      }
+      if (base + k < CHUNKS_IN_LDS) {
+        s_cslot[base + k] = (int32_t)s0;
+        s_cre[base + k] = rows | (e << 16);  // at most 320 rows, fewer than 32768 experts
       }
     }
     carry += total;
@@ -127,8 +152,17 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
   // (its column tiles are the same for all); a chunk goes where the middle of its span of the running total falls.
   // (Equal chunk counts left the XCDs up to a tenth apart in work at ragged expert loads, and a launch ends when
   // its last XCD does.)
+  const bool in_lds = n <= CHUNKS_IN_LDS;
+  auto rows_of = [&](int i) { return in_lds ? (s_cre[i] & 0xffff) : chunk_rows[i]; };
+  auto chunk_expert_of = [&](int i) { return in_lds ? (s_cre[i] >> 16) : chunk_expert[i]; };
+  auto slot_of = [&](int i) { return in_lds ? s_cslot[i] : chunk_slot[i]; };
+  auto xcd_of = [&](int i) { return in_lds ? s_cx[i] : chunk_xcd[i]; };
+  auto xcd_put = [&](int i, int v) {
+    if (in_lds) s_cx[i] = v;
+    else chunk_xcd[i] = v;
+  };
   auto work_of = [&](int i) {
-    const int r = chunk_rows[i];
+    const int r = rows_of(i);
     return r <= 64 ? 4 : r <= 128 ? 8 : r <= 256 ? 16 : 20;
   };
   int wcarry = 0;
@@ -136,23 +170,23 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     const int i = i0 + threadIdx.x;
     int total;
     const int pre = wcarry + block_excl_scan(i < n ? work_of(i) : 0, s_ws, &total);
-    if (i < n) chunk_xcd[i] = pre;
+    if (i < n) xcd_put(i, pre);
     wcarry += total;
   }
   __threadfence_block();
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    const int64_t mid2 = 2 * (int64_t)chunk_xcd[i] + work_of(i);  // twice the middle of the chunk's span
+    const int64_t mid2 = 2 * (int64_t)xcd_of(i) + work_of(i);  // twice the middle of the chunk's span
     const int x = (int)(mid2 * 8 / (2 * (int64_t)wcarry));
-    chunk_xcd[i] = x > 7 ? 7 : x;
+    xcd_put(i, x > 7 ? 7 : x);
   }
   __threadfence_block();
   __syncthreads();
   // (interleaved chunks share their weight tiles through the L2: none of them streams the weights past it, so
   // "last chunk of its expert" is no class of its own then)
   auto key_of = [&](int i) {
-    const bool last = interleave == 1 && ((i + 1 >= n) || (chunk_expert[i + 1] != chunk_expert[i]));
-    return chunk_xcd[i] * CHUNK_CLASSES + chunk_class(chunk_rows[i], last);
+    const bool last = interleave == 1 && ((i + 1 >= n) || (chunk_expert_of(i + 1) != chunk_expert_of(i)));
+    return xcd_of(i) * CHUNK_CLASSES + chunk_class(rows_of(i), last);
   };
   __shared__ uint8_t s_key[KEYS_IN_LDS];  // the chunks' keys, for the rank loop below
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -186,8 +220,8 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
       for (int j = 0; j < i; ++j) rank += s_key[j] == key;
       pos = s_cnt[key] + rank;
     }
-    q_chunk[2 * pos] = chunk_slot[i];
-    q_chunk[2 * pos + 1] = chunk_rows[i] | (chunk_expert[i] << 16);  // at most 320 rows, fewer than 32768 experts
+    q_chunk[2 * pos] = slot_of(i);
+    q_chunk[2 * pos + 1] = rows_of(i) | (chunk_expert_of(i) << 16);  // at most 320 rows, fewer than 32768 experts
   }
 }
 
