@@ -246,8 +246,8 @@ def bench_fp8_row(args):
     peak = PEAK_BF16_TFLOPS if bf16 else PEAK_FP8_TFLOPS
     roofline = {"bound": "mfma", "achieved": round(gu_tflops, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(gu_tflops / peak, 4), "traffic": None,
-                "kernel": ("moe::bwmm_kernel<0, 1> (gate/up blockwise GEMM of the bf16 kind with fused act*up, on the "
-                           "K-contiguous weight copies kept from the first call)" if bf16 else
+                "kernel": ("moe::mx_gemm_kernel<1, 4> (gate/up blockwise GEMM of the bf16 kind on the large-tile kernels with "
+                           "fused act*up, on the x4-ordered weight copies kept from the first call)" if bf16 else
                            "moe::mx_gemm_kernel<1, 3> (gate/up blockwise GEMM of the fp8-row kind on the large-tile "
                            "kernels with fused scales and act*up, on the x4-ordered weight copies kept from the first "
                            "call)"),

@@ -250,7 +250,11 @@ typedef struct moe_bwmm_args {
   void* down_activations;
   /* Optional K-contiguous copies of the bf16 / fp8 weights of the BF16 and FP8_ROW kinds, made once by
    * moe_prepare_kmajor_weights (they depend on the weights only).  Both NULL: every call makes its own copies
-   * in the workspace.  MXFP8 kind: the x4 layouts are K-major already and are read in place when both are NULL;
+   * in the workspace.  (What a copy holds depends on the kind, the weight type and the shape only -- for bf16
+   * weights with H % 256 == 0 and I % 128 == 0, and fp8-row weights with H % 512 == 0 and I % 128 == 0, the order
+   * the large-tile kernels read, otherwise K-contiguous rows -- so one pair serves every call with those weights;
+   * a bf16 call on such a shape that asks for activation checkpoints runs the general kernel and makes its own
+   * K-contiguous copies regardless.)  MXFP8 kind: the x4 layouts are K-major already and are read in place when both are NULL;
    * on shapes with H % 512 == 0 and I % 128 == 0 the same two calls make a copy of the gate/up weights in the
    * order the kernel reads them (each workgroup then reads its weights as contiguous 32 KB runs: the gate/up GEMM
    * is 5 % faster at H = 7168, I = 2048 with 8-bit weights, for a second copy of those weights in memory); used

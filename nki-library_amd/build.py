@@ -20,7 +20,7 @@ OUT_DIR = os.path.join(HERE, "nkilib", "_lib")
 OUT = os.path.join(OUT_DIR, "libmoe_gfx950.so")
 SOURCES = ["rmsnorm_quant.hip", "build_blocks.hip", "combine.hip", "bwmm.hip", "bwmm_mx.hip", "router_topk.hip", "index_ops.hip", "capi.hip"]
 # (stage, weight format) instances of the large-tile MX GEMM; formats as MX_WFMT_* in csrc/bwmm.hpp
-MX_INSTANCES = [(1, 0), (2, 0), (1, 1), (2, 1), (1, 2), (2, 2), (1, 3), (2, 3)]
+MX_INSTANCES = [(1, 0), (2, 0), (1, 1), (2, 1), (1, 2), (2, 2), (1, 3), (2, 3), (1, 4), (2, 4)]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

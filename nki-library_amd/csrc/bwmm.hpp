@@ -81,9 +81,14 @@ struct MxArgs {
                            // of constants for every row)
   float* Y32;              // stage 1 output of this format: fp32 [N*B, y32_stride], columns in natural order
   int64_t y32_stride;
+  // MX_WFMT_BF16 (the bf16 kind on these kernels): both operands bf16, read as bytes exactly like the 8-bit formats
+  // (a 128-byte K slice is 64 elements, multiplied by two v_mfma_f32_16x16x32_bf16 where the 8-bit formats issue
+  // one 128-deep MFMA), so H (gate/up) and I (down) are the K extents in BYTES; no scales of any kind (w_cscale
+  // may still carry per-channel scales of weights widened from fp8); gate/up writes bf16 [N*B, y_stride elements]
+  // in natural column order through Yq.
 };
 
-constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1, MX_WFMT_E2M1 = 2, MX_WFMT_ROW8 = 3;
+constexpr int MX_WFMT_E4M3 = 0, MX_WFMT_E5M2 = 1, MX_WFMT_E2M1 = 2, MX_WFMT_ROW8 = 3, MX_WFMT_BF16 = 4;
 
 // True when the large-tile kernels cover the shape: every intermediate tile holds a multiple
 // of 32 partitions (I % 128 == 0); other shapes run the general kernel.
@@ -107,6 +112,10 @@ int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C,
 // [E, pI, nI, H, 4] with i = t*512 + p*4 + q (zeros past I).
 int launch_relayout_x4(const uint8_t* gate_up, const uint8_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
                        int64_t I, int64_t I_pad, hipStream_t s);
+// The same for bf16 weights ([E, H, 2, I] / [E, I_pad, H] bf16): an x4 element holds two consecutive K values of
+// its column, the layout that of 8-bit weights with K extents of 2H / 2I bytes.
+int launch_relayout_x4_bf16(const uint16_t* gate_up, const uint16_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
+                            int64_t I, int64_t I_pad, hipStream_t s);
 int launch_fill_bytes(void* p, size_t bytes, uint8_t value, hipStream_t s);
 int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,
                        int64_t Iw, hipStream_t s);

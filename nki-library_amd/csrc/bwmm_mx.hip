@@ -130,8 +130,19 @@ __device__ __forceinline__ float acc_get() {
     else if constexpr (WFMT == 1) MX_MFMA_ASM(" blgp:1", SEL_, SELHI_); \
     else MX_MFMA_ASM(" blgp:4", SEL_, SELHI_);             \
   }
+// MX_WFMT_BF16: the 128 K bytes are 64 bf16 values; the first four registers of both fragments (K bytes [16g, 16g+16)
+// of the slice = elements 8g .. 8g+7 of its first 32) and the last four (the same of its second 32) are the operands
+// of two 32-deep bf16 MFMAs, which take the time of the one 128-deep 8-bit MFMA.  No scales.
+__device__ __forceinline__ v4i lo4(const v8i& x) { return (v4i){x[0], x[1], x[2], x[3]}; }
+__device__ __forceinline__ v4i hi4(const v8i& x) { return (v4i){x[4], x[5], x[6], x[7]}; }
+__device__ __forceinline__ v4i lo4(const v4i& x) { return x; }  // (4-bit operands: never instantiated for bf16)
+__device__ __forceinline__ v4i hi4(const v4i& x) { return x; }
 template <int ACC, int OA, int OB, int WFMT, class BOp>
 __device__ __forceinline__ void mfma_asm(const v8i& af, const BOp& bf, int sa, int sb) {
+  if constexpr (WFMT == MX_WFMT_BF16) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 a[%0:%1], %2, %3, a[%0:%1]\n\tv_mfma_f32_16x16x32_bf16 a[%0:%1], %4, %5, a[%0:%1]"
+                 : : "n"(ACC), "n"(ACC + 3), "v"(lo4(af)), "v"(lo4(bf)), "v"(hi4(af)), "v"(hi4(bf)));
+  } else {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
   MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
@@ -148,6 +159,7 @@ __device__ __forceinline__ void mfma_asm(const v8i& af, const BOp& bf, int sa, i
   MX_MFMA_CASE(1, 3, "[1,1,0]", "[0,1,0]");
   MX_MFMA_CASE(2, 3, "[0,1,0]", "[1,1,0]");
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
+  }
 }
 #undef MX_MFMA_CASE
 #undef MX_MFMA_ASM
@@ -163,6 +175,10 @@ __device__ __forceinline__ void mfma_asm(const v8i& af, const BOp& bf, int sa, i
   }
 template <int OA, int OB, int WFMT, class BOp>
 __device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const BOp& bf, int sa, int sb) {
+  if constexpr (WFMT == MX_WFMT_BF16) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
+                 : "+v"(c) : "v"(lo4(af)), "v"(lo4(bf)), "v"(hi4(af)), "v"(hi4(bf)));
+  } else {
   MX_MFMA_CASE(0, 0, "[0,0,0]", "[0,0,0]");
   MX_MFMA_CASE(1, 0, "[1,0,0]", "[0,0,0]");
   MX_MFMA_CASE(2, 0, "[0,0,0]", "[1,0,0]");
@@ -179,6 +195,7 @@ __device__ __forceinline__ void mfma_asm_v(v4f& c, const v8i& af, const BOp& bf,
   MX_MFMA_CASE(1, 3, "[1,1,0]", "[0,1,0]");
   MX_MFMA_CASE(2, 3, "[0,1,0]", "[1,1,0]");
   MX_MFMA_CASE(3, 3, "[1,1,0]", "[1,1,0]");
+  }
 }
 #undef MX_MFMA_CASE
 #undef MX_MFMA_ASM
@@ -280,8 +297,12 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // (per-channel weight scale x per-row activation scale ahead of the bias, bias and scales indexed by natural
   // column, gate/up results written as fp32 rows for the per-row re-quantisation pass) and two more row / column
   // tables (s_rs, s_wsc: null for the MX formats).
-  constexpr bool ROW8 = WFMT == MX_WFMT_ROW8;
-  constexpr int MFMT = ROW8 ? MX_WFMT_E4M3 : WFMT;  // element format of the MFMA's B operand
+  // BF16: the bf16 kind.  The same again, on bf16 operands (see mfma_asm) with no scales at all: row "scales" are 1
+  // (0 for a slot without a token), column scales 1 unless per-channel scales of widened fp8 weights are given, and
+  // the gate/up results go out as bf16 rows in natural column order, which the down stage reads as they are.
+  constexpr bool BF16 = WFMT == MX_WFMT_BF16;
+  constexpr bool ROW8 = WFMT == MX_WFMT_ROW8 || BF16;
+  constexpr int MFMT = BF16 ? MX_WFMT_BF16 : ROW8 ? MX_WFMT_E4M3 : WFMT;  // element format of the MFMA's B operand
   constexpr int D = Cfg::D, RING = Cfg::RING, SA = Cfg::SA, SS = Cfg::SS, SSP = Cfg::SSP;
   constexpr bool BIG = NMT > 16;  // row tiles 16.. accumulate in ordinary registers
   uint8_t* sA = smem;
@@ -430,23 +451,25 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   // the token's row, i.e. its dequantisation scale); down, the scale of the re-quantised intermediate row.
   auto wsc_raw = [&](const Tile& t, int& raw) {
     if constexpr (ROW8) {
-      const v4i rd = make_rsrc(a.w_cscale, 0xffffffffu);
-      ld_b32(raw, ((a.cscale_experts > 1 ? (uint32_t)t.e * ncols : 0u) + natural_col(t)) << 2, rd, 0);
+      const v4i rd = make_rsrc(a.w_cscale ? (const void*)a.w_cscale : (const void*)a.tp2id, 0xffffffffu);
+      ld_b32(raw, a.w_cscale ? ((a.cscale_experts > 1 ? (uint32_t)t.e * ncols : 0u) + natural_col(t)) << 2 : 0u, rd, 0);
     }
   };
   auto wsc_put = [&](int buf, int raw) {
-    if constexpr (ROW8) s_wsc[buf][tid] = __builtin_bit_cast(float, raw);
+    if constexpr (ROW8) s_wsc[buf][tid] = a.w_cscale ? __builtin_bit_cast(float, raw) : 1.f;
   };
   auto rs_raw = [&](const Tile& t, int buf, int (&raw)[2]) {
     if constexpr (ROW8) {
-      const v4i rd = make_rsrc((STAGE == 1) ? (const void*)a.A : (const void*)a.a_rscale, 0xffffffffu);
+      // (bf16: nothing to fetch; the load stays, from an address that is valid, so that every format issues the
+      // same loads)
+      const v4i rd = make_rsrc((STAGE == 1 || BF16) ? (const void*)a.A : (const void*)a.a_rscale, 0xffffffffu);
 #pragma unroll
       for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
         const int r = tid + 256 * j;
         uint32_t off;
         if (STAGE == 1) {
           const int id = s_tok[buf][(r < NMT * 16) ? r : 0];
-          off = (uint32_t)((id >= 0) ? id : 0) * (uint32_t)a.a_stride + (uint32_t)a.H;
+          off = (uint32_t)((id >= 0) ? id : 0) * (uint32_t)a.a_stride + (BF16 ? 0u : (uint32_t)a.H);
         } else {
           off = (uint32_t)(t.slot0 + ((r < t.nrows) ? r : t.nrows - 1)) << 2;
         }
@@ -462,7 +485,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
         const int r = tid + 256 * j;
         if (r < NMT * 16) {
-          float v = __builtin_bit_cast(float, raw[j]);
+          float v = BF16 ? 1.f : __builtin_bit_cast(float, raw[j]);
           if (STAGE == 1 && s_tok[buf][r] < 0) v = 0.f;
           if (pre && a.aff && s_tok[buf][r] >= 0) v *= elem_value(aff[j], aff_index(e, buf, r), a.aff_dtype == MOE_DT_BF16);
           s_rs[buf][r] = v;
@@ -1002,7 +1025,24 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
         // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 32 (x 4 q)
         const int rl = tid_e >> 2, j = tid_e & 3;
         const int row = ps * 64 + rl;
-        if (ROW8 && row < cur.nrows) {
+        if (BF16 && row < cur.nrows) {
+          // bf16 rows in natural column order: the thread's 4 x 8 values are four runs of 8 columns
+          typedef __bf16 v2bf_ __attribute__((ext_vector_type(2)));
+          typedef float v2f_ __attribute__((ext_vector_type(2)));
+          const float* src = E + rl * MX_EP + 8 * j;
+          uint16_t* dst = (uint16_t*)a.Yq + (int64_t)(cur.slot0 + row) * a.y_stride + tile_tI(cur) * 512 + tile_p0(cur) + 8 * j;
+          const int Pt = tile_Pt(cur);
+#pragma unroll
+          for (int qq = 0; qq < 4; ++qq) {
+            const float4 lo = *(const float4*)(src + qq * 32), hi = *(const float4*)(src + qq * 32 + 4);
+            const v2f_ p0 = {lo.x, lo.y}, p1 = {lo.z, lo.w}, p2 = {hi.x, hi.y}, p3 = {hi.z, hi.w};
+            *(uint4*)(dst + qq * Pt) = make_uint4(__builtin_bit_cast(uint32_t, __builtin_convertvector(p0, v2bf_)),
+                                                  __builtin_bit_cast(uint32_t, __builtin_convertvector(p1, v2bf_)),
+                                                  __builtin_bit_cast(uint32_t, __builtin_convertvector(p2, v2bf_)),
+                                                  __builtin_bit_cast(uint32_t, __builtin_convertvector(p3, v2bf_)));
+          }
+        }
+        if (ROW8 && !BF16 && row < cur.nrows) {
           // fp32 rows in natural column order: the thread's 4 x 8 values are four runs of 8 columns
           const float* src = E + rl * MX_EP + 8 * j;
           float* dst = a.Y32 + (int64_t)(cur.slot0 + row) * a.y32_stride + tile_tI(cur) * 512 + tile_p0(cur) + 8 * j;
@@ -1142,8 +1182,8 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   __shared__ __attribute__((aligned(16))) float s_aff[2][MX_ROWS_MAX];
   __shared__ __attribute__((aligned(16))) float s_bias[2][MXT];
   // the fp8-row kind's row and column scales (a token entry each for the other formats)
-  __shared__ __attribute__((aligned(16))) float s_rs[2][WFMT == MX_WFMT_ROW8 ? MX_ROWS_MAX : 4];
-  __shared__ __attribute__((aligned(16))) float s_wsc[2][WFMT == MX_WFMT_ROW8 ? MXT : 4];
+  __shared__ __attribute__((aligned(16))) float s_rs[2][(WFMT == MX_WFMT_ROW8 || WFMT == MX_WFMT_BF16) ? MX_ROWS_MAX : 4];
+  __shared__ __attribute__((aligned(16))) float s_wsc[2][(WFMT == MX_WFMT_ROW8 || WFMT == MX_WFMT_BF16) ? MXT : 4];
   // One workgroup per CU, for the whole launch.  Workgroups are handed to the 8 XCDs round-robin by linear
   // index, and each XCD has its own L2.  XCD x therefore takes the x-th of eight contiguous parts of the chunk
   // list (chunks are ordered by expert; the parts hold about equal work), as a queue of items (chunk, column
@@ -1263,6 +1303,8 @@ int launch_mx_gemm_s1_f2(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f2(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s1_f3(const MxArgs& m, unsigned grid, hipStream_t s);
 int launch_mx_gemm_s2_f3(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s1_f4(const MxArgs& m, unsigned grid, hipStream_t s);
+int launch_mx_gemm_s2_f4(const MxArgs& m, unsigned grid, hipStream_t s);
 
 int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStream_t s) {
   if (gx == 0 || gy == 0) return MOE_OK;
@@ -1283,6 +1325,7 @@ int launch_mx_gemm(int stage, const MxArgs& m0, unsigned gx, unsigned gy, hipStr
     case MX_WFMT_E5M2: return stage == 1 ? launch_mx_gemm_s1_f1(m, grid, s) : launch_mx_gemm_s2_f1(m, grid, s);
     case MX_WFMT_E2M1: return stage == 1 ? launch_mx_gemm_s1_f2(m, grid, s) : launch_mx_gemm_s2_f2(m, grid, s);
     case MX_WFMT_ROW8: return stage == 1 ? launch_mx_gemm_s1_f3(m, grid, s) : launch_mx_gemm_s2_f3(m, grid, s);
+    case MX_WFMT_BF16: return stage == 1 ? launch_mx_gemm_s1_f4(m, grid, s) : launch_mx_gemm_s2_f4(m, grid, s);
     default: return MOE_E_BAD_ARG;
   }
 }

@@ -135,20 +135,45 @@ bool row8_fast(const moe_bwmm_args* a) {
     return false;
   return true;
 }
-// What a kept copy of the fp8-row weights holds on that path: the weights in x4 order, one expert's worth of E8M0
-// block scales of 127 (2^0) that serves every expert, and one row of activation block scales of 127.
+// The bf16 kind with bf16 weights runs there too (MX_WFMT_BF16) when the K extents in bytes (2H, 2I) are shapes of
+// those kernels and the offsets fit -- which, as above, also decides what kept weight copies look like -- except for
+// calls that ask for activation checkpoints, which their epilogues do not write: those run the general kernel on
+// copies of their own, made per call (kept copies are in the other order).
+bool bf16_fast_shape(const moe_bwmm_args* a) {
+  if (a->kind != MOE_KIND_BF16 || a->weight_dtype != MOE_DT_BF16) return false;
+  if (a->H % 256 != 0 || a->I % 128 != 0) return false;
+  const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
+  const int64_t slots = a->N * a->B, Ib = 2 * a->I, Hb = 2 * a->H;
+  const int64_t pI = Ib > 512 ? 128 : Ib / 4, nI = (Ib + 511) / 512;
+  if (a->T1 * Hb >= lim32 || slots * Ib >= lim32) return false;
+  if (2 * Hb * a->I >= lim31 || pI * nI * a->H * 4 >= lim31) return false;
+  if (slots * 4 >= lim32 || a->T1 * a->E * 4 >= lim32 || a->E * 2 * a->I * 4 >= lim32 || a->E * a->H * 4 >= lim32)
+    return false;
+  return true;
+}
+bool bf16_fast(const moe_bwmm_args* a) {
+  return bf16_fast_shape(a) && !a->gate_up_activations_T && !a->down_activations;
+}
+// kept copies of the bf16 kind's weights are in the order this call reads
+bool bf16_kept_usable(const moe_bwmm_args* a) { return bf16_fast(a) || !bf16_fast_shape(a); }
+// What a kept copy of the fp8-row (bf16) weights holds on that path: the weights in x4 order, one expert's worth of
+// E8M0 block scales of 127 (2^0) that serves every expert, and one row of activation block scales of 127 (the bf16
+// kernels fetch the tables like the others and ignore what they hold).  K extents in bytes: H, I for fp8, twice
+// that for bf16.
 struct Row8Copy {
   size_t w_scale, a_scale, a_scale_bytes, total;
 };
 Row8Copy row8_copy(const moe_bwmm_args* a, int which) {
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
-  const size_t nH = (size_t)a->H / 512, nI = ((size_t)a->I + 511) / 512, pI = a->I > 512 ? 128 : (size_t)a->I / 4;
+  const size_t es = a->kind == MOE_KIND_BF16 ? 2 : 1;
+  const size_t Hb = (size_t)a->H * es, Ib = (size_t)a->I * es;
+  const size_t nH = Hb / 512, nI = (Ib + 511) / 512, pI = Ib > 512 ? 128 : Ib / 4;
   Row8Copy c;
-  const size_t w = which == 0 ? (size_t)a->E * 2 * a->H * a->I : (size_t)a->E * pI * nI * a->H * 4;
+  const size_t w = which == 0 ? (size_t)a->E * 2 * Hb * a->I : (size_t)a->E * pI * nI * a->H * 4;
   const size_t ws = which == 0 ? 16 * 2 * nH * (size_t)a->I : ((pI + 7) / 8) * nI * (size_t)a->H;
   c.w_scale = al(w);
   c.a_scale = c.w_scale + al(ws);
-  c.a_scale_bytes = al(which == 0 ? (size_t)a->H / 32 : nI * 16);
+  c.a_scale_bytes = al(which == 0 ? Hb / 32 : nI * 16);
   c.total = c.a_scale + c.a_scale_bytes;
   return c;
 }
@@ -174,8 +199,18 @@ Plan make_plan(const moe_bwmm_args* a) {
     p.y = off; off += al256(slots * (size_t)p.Iw * 2);
     // K-contiguous bf16 copies of the weights: [E, 2, I, Hk] and [E, H, Iw]
     p.Hk = (a->H + 63) / 64 * 64;
-    if (!a->gate_up_proj_weight_kmajor) { p.wt1 = off; off += al256((size_t)a->E * 2 * a->I * p.Hk * 2); }
-    if (!a->down_proj_weight_kmajor) { p.wt2 = off; off += al256((size_t)a->E * a->H * p.Iw * 2); }
+    const bool bf = bf16_fast(a);
+    if (bf) {  // the x4 geometry of the down weights over 2I bytes of K
+      p.nI = (2 * a->I + 511) / 512;
+      p.pI = 2 * a->I > 512 ? 128 : a->I / 2;
+    }
+    const bool kept = bf16_kept_usable(a);
+    if (!(a->gate_up_proj_weight_kmajor && kept)) {
+      p.wt1 = off; off += al256(bf ? row8_copy(a, 0).total : (size_t)a->E * 2 * a->I * p.Hk * 2);
+    }
+    if (!(a->down_proj_weight_kmajor && kept)) {
+      p.wt2 = off; off += al256(bf ? row8_copy(a, 1).total : (size_t)a->E * a->H * p.Iw * 2);
+    }
   } else {
     p.Iw = (a->I + 127) / 128 * 128;
     p.y = off; off += al256(slots * (size_t)a->I * 4);
@@ -201,8 +236,16 @@ Plan make_plan(const moe_bwmm_args* a) {
 }
 
 // K-contiguous copy of the gate/up (which == 0) or down (which == 1) weights of the BF16 / FP8_ROW kinds.
-int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hipStream_t s) {
+// (bf16_x4: the bf16 kind's copy in the large-tile kernels' order rather than K-contiguous)
+int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hipStream_t s, bool bf16_x4) {
   const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
+  if (bf16_x4) {
+    const Row8Copy c = row8_copy(a, which);
+    int rc = launch_relayout_x4_bf16((const uint16_t*)a->gate_up_proj_weight, (const uint16_t*)a->down_proj_weight,
+                                     (uint8_t*)dst, which, a->E, a->H, a->I, Ipad, s);
+    if (rc != MOE_OK) return rc;
+    return launch_fill_bytes((uint8_t*)dst + c.w_scale, c.total - c.w_scale, 127, s);
+  }
   if (a->kind == MOE_KIND_BF16) {
     const int w8 = a->weight_dtype == MOE_DT_FP8_E4M3;
     if (which == 0)
@@ -241,7 +284,7 @@ extern "C" size_t moe_kmajor_weights_bytes(const moe_bwmm_args* a, int which) {
                                  : 0;
   const Plan p = make_plan(a);
   const size_t es = a->kind == MOE_KIND_BF16 ? 2 : 1;
-  if (row8_fast(a)) return row8_copy(a, which).total;
+  if (row8_fast(a) || bf16_fast_shape(a)) return row8_copy(a, which).total;
   return which == 0 ? (size_t)a->E * 2 * a->I * p.Hk * es : (size_t)a->E * a->H * p.Iw * es;
 }
 
@@ -260,9 +303,9 @@ extern "C" int moe_prepare_kmajor_weights(const moe_bwmm_args* a, void* gate_up_
   if (!gate_up_kmajor || !down_kmajor) return MOE_E_BAD_ARG;
   if ((((uintptr_t)gate_up_kmajor) & 255) != 0 || (((uintptr_t)down_kmajor) & 255) != 0) return MOE_E_BAD_ARG;
   const Plan p = make_plan(a);
-  rc = kmajor_copy(a, p, 0, gate_up_kmajor, (hipStream_t)stream);
+  rc = kmajor_copy(a, p, 0, gate_up_kmajor, (hipStream_t)stream, bf16_fast_shape(a));
   if (rc != MOE_OK) return rc;
-  return kmajor_copy(a, p, 1, down_kmajor, (hipStream_t)stream);
+  return kmajor_copy(a, p, 1, down_kmajor, (hipStream_t)stream, bf16_fast_shape(a));
 }
 
 extern "C" size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* a) {
@@ -347,16 +390,18 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     g2.A = ws + p.y; g2.a_stride = p.Iw * 2; g2.K = p.Iw;
     gx1 = (unsigned)((a->I + 127) / 128);
     // K-contiguous bf16 copies of the weights (fp8 weights are widened on the way), as for the fp8-row kind below
-    g1.W = a->gate_up_proj_weight_kmajor ? (const uint8_t*)a->gate_up_proj_weight_kmajor : ws + p.wt1;
-    g2.W = a->down_proj_weight_kmajor ? (const uint8_t*)a->down_proj_weight_kmajor : ws + p.wt2;
+    const bool kept = bf16_kept_usable(a);
+    const bool have1 = a->gate_up_proj_weight_kmajor && kept, have2 = a->down_proj_weight_kmajor && kept;
+    g1.W = have1 ? (const uint8_t*)a->gate_up_proj_weight_kmajor : ws + p.wt1;
+    g2.W = have2 ? (const uint8_t*)a->down_proj_weight_kmajor : ws + p.wt2;
     g1.Kp = p.Hk * 2;
     g2.Kp = p.Iw * 2;
-    if ((stages & MOE_STAGE_GATE_UP) && !a->gate_up_proj_weight_kmajor) {
-      rc = kmajor_copy(a, p, 0, ws + p.wt1, s);
+    if ((stages & MOE_STAGE_GATE_UP) && !have1) {
+      rc = kmajor_copy(a, p, 0, ws + p.wt1, s, bf16_fast(a));
       if (rc != MOE_OK) return rc;
     }
-    if ((stages & MOE_STAGE_DOWN) && !a->down_proj_weight_kmajor) {
-      rc = kmajor_copy(a, p, 1, ws + p.wt2, s);
+    if ((stages & MOE_STAGE_DOWN) && !have2) {
+      rc = kmajor_copy(a, p, 1, ws + p.wt2, s, bf16_fast(a));
       if (rc != MOE_OK) return rc;
     }
   } else {
@@ -371,16 +416,17 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     g1.Kp = p.Hk;
     g2.Kp = p.Iw;
     if ((stages & MOE_STAGE_GATE_UP) && !a->gate_up_proj_weight_kmajor) {
-      rc = kmajor_copy(a, p, 0, ws + p.wt1, s);
+      rc = kmajor_copy(a, p, 0, ws + p.wt1, s, false);
       if (rc != MOE_OK) return rc;
     }
     if ((stages & MOE_STAGE_DOWN) && !a->down_proj_weight_kmajor) {
-      rc = kmajor_copy(a, p, 1, ws + p.wt2, s);
+      rc = kmajor_copy(a, p, 1, ws + p.wt2, s, false);
       if (rc != MOE_OK) return rc;
     }
   }
 
-  const bool r8_fast = row8_fast(a);
+  const bool bf_fast = bf16_fast(a);
+  const bool r8_fast = row8_fast(a) || bf_fast;  // (what the two share: x4 copies with unit scale tables)
   const bool mx_fast = (a->kind == MOE_KIND_MXFP8 && mx_fast_path_ok(a->H, a->I)) || r8_fast;
   MxArgs m;
   memset(&m, 0, sizeof(m));
@@ -412,6 +458,12 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
       m.Y32 = (float*)(ws + p.y);
       m.y32_stride = a->I;
     }
+    if (bf_fast) {
+      m.wfmt = MX_WFMT_BF16;
+      m.Y32 = nullptr;
+      m.Yq = ws + p.y;  // bf16 [N*B, Iw]
+      m.y_stride = p.Iw;
+    }
   }
   const unsigned gyc = (unsigned)bk.max_chunks;
   // checkpoints of blocks that never run stay zero
@@ -441,6 +493,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
         m1.A_scale = g1.W + c.a_scale; m1.a_scale_stride = 0; m1.a_scale_bytes = (int64_t)c.a_scale_bytes;
         m1.w_cscale = (const float*)a->gate_up_proj_scale;
       }
+      if (bf_fast) m1.H = 2 * a->H;  // K in bytes
+
       // column tiles of 32 partitions x 4 q, gate and up: 4 per full intermediate tile + those of a short last one
       rc = launch_mx_gemm(1, m1, (unsigned)((a->I / 512) * 4 + (a->I % 512) / 128), gyc, s);
     } else {
@@ -471,6 +525,12 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
         m2.w_cscale = (const float*)a->down_proj_scale;
         m2.a_rscale = (const float*)(ws + p.ys);
       }
+      if (bf_fast) {
+        m2.A = ws + p.y; m2.a_stride = p.Iw * 2;
+        m2.I = 2 * a->I;  // K in bytes
+        m2.a_rscale = nullptr;
+      }
+
       rc = launch_mx_gemm(2, m2, (unsigned)(a->H / 256), gyc, s);
     } else {
       rc = launch_gemm_stage(a->kind, 2, g2, gx2, gy, s);

@@ -103,6 +103,11 @@ def test_c1_tiny_bf16():
         (300, 512, 384, 2, 2, 128, "shard_on_block", 0, 1, True, False, False),
         (640, 576, 520, 2, 2, 128, "shard_on_i", 3, 2, False, False, True),
         (600, 512, 384, 2, 2, 128, "shard_on_block", 1, 1, True, True, False),
+        # shapes of the large-tile kernels (H % 256 == 0, I % 128 == 0) with the options above: PRE_SCALE and clamps;
+        # chunks of 257..320 rows (E = 2: 320 rows per expert); a short last intermediate tile (I = 640)
+        (512, 768, 512, 8, 2, 128, "shard_on_i", 3, 2, False, False, True),
+        (320, 512, 640, 2, 2, 64, "shard_on_block", 0, 1, True, False, True),
+        (1100, 256, 128, 3, 2, 128, "shard_on_i", 2, 1, True, True, False),
     ],
 )
 def test_dense_variants(T, H, I, E, k, B, impl, act, mode, bias, skip, clamp):
