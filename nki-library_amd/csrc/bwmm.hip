@@ -762,13 +762,26 @@ int launch_relayout_x4(const uint8_t* gate_up, const uint8_t* down, uint8_t* dst
   return MOE_OK;
 }
 
-// bf16 weights: one thread per four adjacent output columns, two 8-byte reads (the two K rows of the x4 elements),
-// one 16-byte write.
+// bf16 weights (W8: fp8-e4m3 weights widened to bf16 on the way, exactly): one thread per four adjacent output
+// columns, two 8-byte (4-byte) reads (the two K rows of the x4 elements), one 16-byte write.
+template <bool W8>
+__device__ __forceinline__ uint2 four_as_bf16(const void* W, int64_t elem) {
+  if constexpr (W8) {
+    const uint32_t raw = *(const uint32_t*)((const uint8_t*)W + elem);
+    uint32_t v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] = f32_to_bf16_bits(e4m3_to_f32((raw >> (8 * q)) & 0xffu));
+    return make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
+  } else {
+    return *(const uint2*)((const uint16_t*)W + elem);
+  }
+}
 __device__ __forceinline__ uint4 pairs_of_4(const uint2& r0, const uint2& r1) {
   return make_uint4((r0.x & 0xffffu) | (r1.x << 16), (r0.x >> 16) | (r1.x & 0xffff0000u), (r0.y & 0xffffu) | (r1.y << 16),
                     (r0.y >> 16) | (r1.y & 0xffff0000u));
 }
-__global__ __launch_bounds__(256) void relayout_gu_x4_bf16_kernel(const uint16_t* __restrict__ W, uint32_t* __restrict__ X,
+template <bool W8>
+__global__ __launch_bounds__(256) void relayout_gu_x4_bf16_kernel(const void* __restrict__ W, uint32_t* __restrict__ X,
                                                                   int64_t H, int64_t I, int64_t total4) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over [E, 128, 2, 2H / 512, I / 4]
   if (idx >= total4) return;
@@ -776,11 +789,12 @@ __global__ __launch_bounds__(256) void relayout_gu_x4_bf16_kernel(const uint16_t
   const int64_t i = (idx % I4) * 4, t = (idx / I4) % nH, gu = (idx / (I4 * nH)) % 2, p = (idx / (I4 * nH * 2)) % 128,
                 e = idx / (I4 * nH * 2 * 128);
   const int64_t h = t * 256 + p * 2;
-  const uint2 r0 = *(const uint2*)(W + ((e * H + h) * 2 + gu) * I + i);
-  const uint2 r1 = *(const uint2*)(W + ((e * H + h + 1) * 2 + gu) * I + i);
+  const uint2 r0 = four_as_bf16<W8>(W, ((e * H + h) * 2 + gu) * I + i);
+  const uint2 r1 = four_as_bf16<W8>(W, ((e * H + h + 1) * 2 + gu) * I + i);
   *(uint4*)(X + idx * 4) = pairs_of_4(r0, r1);
 }
-__global__ __launch_bounds__(256) void relayout_down_x4_bf16_kernel(const uint16_t* __restrict__ W,
+template <bool W8>
+__global__ __launch_bounds__(256) void relayout_down_x4_bf16_kernel(const void* __restrict__ W,
                                                                     uint32_t* __restrict__ X, int64_t H, int64_t I,
                                                                     int64_t I_pad, int64_t pI, int64_t nI,
                                                                     int64_t total4) {
@@ -790,26 +804,35 @@ __global__ __launch_bounds__(256) void relayout_down_x4_bf16_kernel(const uint16
   const int64_t h = (idx % H4) * 4, t = (idx / H4) % nI, p = (idx / (H4 * nI)) % pI, e = idx / (H4 * nI * pI);
   const int64_t i0 = t * 256 + p * 2;
   const uint2 zero = make_uint2(0u, 0u);
-  const uint2 r0 = (i0 < I) ? *(const uint2*)(W + (e * I_pad + i0) * H + h) : zero;
-  const uint2 r1 = (i0 + 1 < I) ? *(const uint2*)(W + (e * I_pad + i0 + 1) * H + h) : zero;
+  const uint2 r0 = (i0 < I) ? four_as_bf16<W8>(W, (e * I_pad + i0) * H + h) : zero;
+  const uint2 r1 = (i0 + 1 < I) ? four_as_bf16<W8>(W, (e * I_pad + i0 + 1) * H + h) : zero;
   *(uint4*)(X + idx * 4) = pairs_of_4(r0, r1);
 }
-int launch_relayout_x4_bf16(const uint16_t* gate_up, const uint16_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
+int launch_relayout_x4_bf16(const void* gate_up, const void* down, int w8, uint8_t* dst, int which, int64_t E, int64_t H,
                             int64_t I, int64_t I_pad, hipStream_t s) {
-  if ((((uintptr_t)dst) & 15) != 0 || (((uintptr_t)gate_up) & 7) != 0 || (((uintptr_t)down) & 7) != 0 || H % 256 != 0 ||
-      I % 4 != 0)
+  const uintptr_t src_align = w8 ? 3 : 7;
+  if ((((uintptr_t)dst) & 15) != 0 || (((uintptr_t)gate_up) & src_align) != 0 || (((uintptr_t)down) & src_align) != 0 ||
+      H % 256 != 0 || I % 4 != 0)
     return MOE_E_BAD_ARG;
   if (which == 0) {
     const int64_t total = E * 128 * 2 * (H / 256) * (I / 4);
     if ((total + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
-    hipLaunchKernelGGL(relayout_gu_x4_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gate_up,
-                       (uint32_t*)dst, H, I, total);
+    if (w8)
+      hipLaunchKernelGGL(relayout_gu_x4_bf16_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gate_up,
+                         (uint32_t*)dst, H, I, total);
+    else
+      hipLaunchKernelGGL(relayout_gu_x4_bf16_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, gate_up,
+                         (uint32_t*)dst, H, I, total);
   } else {
     const int64_t Ib = 2 * I, nI = (Ib + 511) / 512, pI = Ib > 512 ? 128 : Ib / 4;
     const int64_t total = E * pI * nI * (H / 4);
     if ((total + 255) / 256 >= (int64_t)1 << 31) return MOE_E_BAD_SHAPE;
-    hipLaunchKernelGGL(relayout_down_x4_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, down,
-                       (uint32_t*)dst, H, I, I_pad, pI, nI, total);
+    if (w8)
+      hipLaunchKernelGGL(relayout_down_x4_bf16_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, down,
+                         (uint32_t*)dst, H, I, I_pad, pI, nI, total);
+    else
+      hipLaunchKernelGGL(relayout_down_x4_bf16_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, down,
+                         (uint32_t*)dst, H, I, I_pad, pI, nI, total);
   }
   MOE_CHECK_LAUNCH();
   return MOE_OK;

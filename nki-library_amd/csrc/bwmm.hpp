@@ -112,9 +112,10 @@ int launch_transpose_fp8(const uint8_t* src, uint8_t* dst, int64_t R, int64_t C,
 // [E, pI, nI, H, 4] with i = t*512 + p*4 + q (zeros past I).
 int launch_relayout_x4(const uint8_t* gate_up, const uint8_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
                        int64_t I, int64_t I_pad, hipStream_t s);
-// The same for bf16 weights ([E, H, 2, I] / [E, I_pad, H] bf16): an x4 element holds two consecutive K values of
-// its column, the layout that of 8-bit weights with K extents of 2H / 2I bytes.
-int launch_relayout_x4_bf16(const uint16_t* gate_up, const uint16_t* down, uint8_t* dst, int which, int64_t E, int64_t H,
+// The same for the bf16 kind's weights ([E, H, 2, I] / [E, I_pad, H] bf16, or fp8-e4m3 when w8, widened to bf16): an
+// x4 element holds two consecutive K values of its column, the layout that of 8-bit weights with K extents of
+// 2H / 2I bytes.
+int launch_relayout_x4_bf16(const void* gate_up, const void* down, int w8, uint8_t* dst, int which, int64_t E, int64_t H,
                             int64_t I, int64_t I_pad, hipStream_t s);
 int launch_fill_bytes(void* p, size_t bytes, uint8_t value, hipStream_t s);
 int launch_row_requant(const float* Y, uint8_t* Yq, float* ys, const Bookkeeping& k, int64_t N, int64_t B, int64_t I,

@@ -135,12 +135,12 @@ bool row8_fast(const moe_bwmm_args* a) {
     return false;
   return true;
 }
-// The bf16 kind with bf16 weights runs there too (MX_WFMT_BF16) when the K extents in bytes (2H, 2I) are shapes of
+// The bf16 kind (bf16 weights, or fp8 weights widened to bf16 in the copy) runs there too (MX_WFMT_BF16) when the K extents in bytes (2H, 2I) are shapes of
 // those kernels and the offsets fit -- which, as above, also decides what kept weight copies look like -- except for
 // calls that ask for activation checkpoints, which their epilogues do not write: those run the general kernel on
 // copies of their own, made per call (kept copies are in the other order).
 bool bf16_fast_shape(const moe_bwmm_args* a) {
-  if (a->kind != MOE_KIND_BF16 || a->weight_dtype != MOE_DT_BF16) return false;
+  if (a->kind != MOE_KIND_BF16 || (a->weight_dtype != MOE_DT_BF16 && a->weight_dtype != MOE_DT_FP8_E4M3)) return false;
   if (a->H % 256 != 0 || a->I % 128 != 0) return false;
   const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
   const int64_t slots = a->N * a->B, Ib = 2 * a->I, Hb = 2 * a->H;
@@ -241,7 +241,7 @@ int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hip
   const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
   if (bf16_x4) {
     const Row8Copy c = row8_copy(a, which);
-    int rc = launch_relayout_x4_bf16((const uint16_t*)a->gate_up_proj_weight, (const uint16_t*)a->down_proj_weight,
+    int rc = launch_relayout_x4_bf16(a->gate_up_proj_weight, a->down_proj_weight, a->weight_dtype == MOE_DT_FP8_E4M3,
                                      (uint8_t*)dst, which, a->E, a->H, a->I, Ipad, s);
     if (rc != MOE_OK) return rc;
     return launch_fill_bytes((uint8_t*)dst + c.w_scale, c.total - c.w_scale, 127, s);
