@@ -276,3 +276,49 @@ def test_c2_fp8_row_subset_equals_golden_and_full_run():
     err = max_abs_rel(o[:T2], g[:T2])
     print(f"c2 subset of {T2} tokens: max-abs-rel {err:.3e} (rtol {RTOL})", flush=True)
     assert max_all_close(o[:T2], g[:T2], rtol=RTOL, atol=ATOL)
+
+
+def test_bf16_layer_subset_equals_golden_and_full_run():
+    """The bf16 kind at the size bench.py's `--workload bf16` times (T=4096 H=2048 I=4096 E=8 top-2: 1024 rows per
+    expert, i.e. four 256-row chunks of one expert side by side on the large-tile kernels): the tokens routed to
+    experts {0, 1} only are checked against the golden, and against their rows in the full 4096-token run."""
+    import torch
+    from nkilib import synthetic as syn
+    from nkilib.core.moe.moe_cte import MoECTEImplementation, MoECTESpec, build_token_blocks, get_n_blocks, moe_cte
+
+    dev = torch.device("cuda:0")
+    T, H, I, E, k, B = 4096, 2048, 4096, 8, 2, 128
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    gu_w = (torch.randn((E, H, 2, I), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    d_w = (torch.randn((E, I, H), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    ids, aff = syn.route(T, E, k, dev, seed=3, mode="softmax")
+    x = syn.hidden_states(T, H, dev, seed=3)
+
+    def layer(ids_, aff_, x_, gu_, d_):
+        T_, E_ = x_.shape[0] - 1, aff_.shape[1]
+        N = get_n_blocks(T_, k, E_, B, n_block_per_iter=2)
+        tp2id, b2e, cond = build_token_blocks(ids_, E_, B, N, n_conditions=N + 2)
+        out_ = moe_cte(x_, aff_.reshape(-1, 1), gu_, d_, tp2id, b2e, B,
+                       MoECTESpec(implementation=MoECTEImplementation.shard_on_block), conditions=cond)
+        torch.cuda.synchronize()
+        return out_, tp2id, b2e, cond
+
+    out, _, _, _ = layer(ids, aff, x, gu_w, d_w)
+    assert not bool(out[T].any())
+
+    experts = torch.tensor([0, 1], device=dev)
+    keep = torch.nonzero((ids < 2).all(dim=1)).reshape(-1)
+    assert keep.numel() >= 32, keep.numel()
+    ids2, aff2, x2 = _subset_problem(ids, aff, x, keep, experts)
+    gu2, d2 = gu_w[:2].contiguous(), d_w[:2].contiguous()
+    out2, tp2id, b2e, cond = layer(ids2, aff2, x2, gu2, d2)
+    T2 = keep.numel()
+    assert torch.equal(out2[:T2], out[keep]), "rows of the full run differ from the subset run"
+
+    g = omoe.moe_blockwise_ref(_bf16_np(x2), _bf16_np(aff2), _bf16_np(gu2), _bf16_np(d2), tp2id.cpu().numpy().reshape(-1),
+                               b2e.cpu().numpy().reshape(-1), B, conditions=cond.cpu().numpy().reshape(-1))
+    o = _bf16_np(out2)[:, 0]
+    err = max_abs_rel(o[:T2], g[:T2])
+    print(f"bf16 subset of {T2} tokens: max-abs-rel {err:.3e} (rtol {RTOL})", flush=True)
+    assert max_all_close(o[:T2], g[:T2], rtol=RTOL, atol=ATOL)
