@@ -183,16 +183,17 @@ __global__ __launch_bounds__(RQ_THREADS) void rmsnorm_quant_fp8_kernel(
   }
 }
 
-// The common case of the ROW front end on its own: bf16 input and gamma, RMSNorm on, 16-byte aligned rows of a
-// multiple of 8 elements.  Same arithmetic in the same order as rmsnorm_quant_fp8_kernel<0> (the two are compared
+// The common case of the ROW (MODE 0) and STATIC (MODE 1) front ends on their own: bf16 input and gamma, RMSNorm on,
+// 16-byte aligned rows of a multiple of 8 elements.  Same arithmetic in the same order as rmsnorm_quant_fp8_kernel (the two are compared
 // bit for bit in the tests), without its per-element dtype and bounds decisions, with the row kept packed as loaded
 // until it is used (MAXC chunks of 8 elements per thread instead of room for the longest row) and gamma fetched
 // with the row, ahead of the first reduction: the general kernel spends its time in the vector ALUs and, at 8
 // chunks of unpacked values per thread, runs four workgroups per CU.
-template <int MAXC>
+template <int MAXC, int MODE>
 __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXC <= 2 ? 6 : MAXC <= 4 ? 4 : 3, 8))) void
 rmsnorm_quant_row_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
-                              uint8_t* __restrict__ out, int64_t H, float eps, float lower_bound) {
+                              const float* __restrict__ static_scale, uint8_t* __restrict__ out, int64_t H, float eps,
+                              float lower_bound) {
   __shared__ float red[16];
   __shared__ double redd[16];
   const int64_t row = blockIdx.x;
@@ -233,23 +234,31 @@ rmsnorm_quant_row_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __
     for (int k = 0; k < 4; ++k) {
       v[j][2 * k] = (bf16_lo(w[k]) * inv) * bf16_lo(g[k]);
       v[j][2 * k + 1] = (bf16_hi(w[k]) * inv) * bf16_hi(g[k]);
-      am = fmaxf(am, fmaxf(fabsf(v[j][2 * k]), fabsf(v[j][2 * k + 1])));
+      if (MODE == 0) am = fmaxf(am, fmaxf(fabsf(v[j][2 * k]), fabsf(v[j][2 * k + 1])));
     }
   }
-  am = block_max(am, red);
-  const bool clip = lower_bound > 0.f;  // uniform
-  if (clip) am = fminf(am, lower_bound);
-  const float dq = fmaxf(am / 240.0f, 1e-6f);  // rmsnorm_quant.py:597-604
-  const float qs = 1.0f / dq;
-  uint8_t* orow = out + row * (H + 4);
-  if (threadIdx.x == 0) *(uint32_t*)(orow + H) = __float_as_uint(dq);  // H % 8 == 0: the record's scale is 4-byte aligned
+  const bool clip = MODE == 0 && lower_bound > 0.f;  // uniform
+  float qs;
+  uint8_t* orow = out + row * (MODE == 0 ? H + 4 : H);
+  if (MODE == 0) {
+    am = block_max(am, red);
+    if (clip) am = fminf(am, lower_bound);
+    const float dq = fmaxf(am / 240.0f, 1e-6f);  // rmsnorm_quant.py:597-604
+    qs = 1.0f / dq;
+    if (threadIdx.x == 0) *(uint32_t*)(orow + H) = __float_as_uint(dq);  // H % 8 == 0: the record's scale is 4-byte aligned
+  } else {
+    qs = 1.0f / static_scale[0];
+  }
 #pragma unroll
   for (int j = 0; j < MAXC; ++j) {
     const int64_t i = ((int64_t)j * RQ_THREADS + threadIdx.x) * 8;
     if (i < H) {
       float q[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) q[k] = (clip ? fminf(fmaxf(v[j][k], -lower_bound), lower_bound) : v[j][k]) * qs;
+      for (int k = 0; k < 8; ++k) {
+        if (MODE == 0) q[k] = (clip ? fminf(fmaxf(v[j][k], -lower_bound), lower_bound) : v[j][k]) * qs;
+        else q[k] = fminf(fmaxf(v[j][k] * qs, -240.0f), 240.0f);
+      }
       *(uint32_t*)(orow + i) = pack4_e4m3(q[0], q[1], q[2], q[3]);
       *(uint32_t*)(orow + i + 4) = pack4_e4m3(q[4], q[5], q[6], q[7]);
     }
@@ -509,6 +518,20 @@ static bool valid_in_dtype(int d) { return d == MOE_DT_BF16 || d == MOE_DT_FP16 
 
 using namespace moe;
 
+template <int MODE>
+static void launch_bf16_front_end(const void* x, const void* gamma, const float* static_scale, void* out, int64_t rows,
+                                  int64_t H, float eps, float lower_bound, hipStream_t stream) {
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(RQ_THREADS), 0, stream, (const uint16_t*)x,
+                       (const uint16_t*)gamma, static_scale, (uint8_t*)out, H, eps, lower_bound);
+  };
+  const int64_t chunks = (H + RQ_THREADS * 8 - 1) / (RQ_THREADS * 8);
+  if (chunks <= 1) launch(rmsnorm_quant_row_bf16_kernel<1, MODE>);
+  else if (chunks <= 2) launch(rmsnorm_quant_row_bf16_kernel<2, MODE>);
+  else if (chunks <= 4) launch(rmsnorm_quant_row_bf16_kernel<4, MODE>);
+  else launch(rmsnorm_quant_row_bf16_kernel<8, MODE>);
+}
+
 extern "C" int moe_rmsnorm_quant_fp8_row(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out,
                                          int64_t rows, int64_t H, float eps, float lower_bound, int do_norm,
                                          void* stream) {
@@ -519,15 +542,7 @@ extern "C" int moe_rmsnorm_quant_fp8_row(const void* x, int x_dtype, const void*
   if (rows == 0) return MOE_OK;
   const int vec_ok = (H % 8 == 0) && (((uintptr_t)x & 15) == 0) && (!do_norm || ((uintptr_t)gamma & 15) == 0);
   if (vec_ok && do_norm && x_dtype == MOE_DT_BF16 && gamma_dtype == MOE_DT_BF16 && (((uintptr_t)out & 3) == 0)) {
-    auto launch = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, (const uint16_t*)x,
-                         (const uint16_t*)gamma, (uint8_t*)out, H, eps, lower_bound);
-    };
-    const int64_t chunks = (H + RQ_THREADS * 8 - 1) / (RQ_THREADS * 8);
-    if (chunks <= 1) launch(rmsnorm_quant_row_bf16_kernel<1>);
-    else if (chunks <= 2) launch(rmsnorm_quant_row_bf16_kernel<2>);
-    else if (chunks <= 4) launch(rmsnorm_quant_row_bf16_kernel<4>);
-    else launch(rmsnorm_quant_row_bf16_kernel<8>);
+    launch_bf16_front_end<0>(x, gamma, nullptr, out, rows, H, eps, lower_bound, (hipStream_t)stream);
     MOE_CHECK_LAUNCH();
     return MOE_OK;
   }
@@ -547,6 +562,11 @@ extern "C" int moe_rmsnorm_quant_fp8_static(const void* x, int x_dtype, const vo
   if (H > RQ_MAX_H) return MOE_E_BAD_SHAPE;
   if (rows == 0) return MOE_OK;
   const int vec_ok = (H % 8 == 0) && (((uintptr_t)x & 15) == 0) && (!do_norm || ((uintptr_t)gamma & 15) == 0);
+  if (vec_ok && do_norm && x_dtype == MOE_DT_BF16 && gamma_dtype == MOE_DT_BF16 && (((uintptr_t)out & 3) == 0)) {
+    launch_bf16_front_end<1>(x, gamma, input_dequant_scale, out, rows, H, eps, 0.f, (hipStream_t)stream);
+    MOE_CHECK_LAUNCH();
+    return MOE_OK;
+  }
   hipLaunchKernelGGL(rmsnorm_quant_fp8_kernel<1>, dim3((unsigned)rows), dim3(RQ_THREADS), 0, (hipStream_t)stream, x,
                      x_dtype, gamma, gamma_dtype, input_dequant_scale, (uint8_t*)out, H, H, eps, 0.f, do_norm, vec_ok);
   MOE_CHECK_LAUNCH();

@@ -108,6 +108,13 @@ def test_row_quant_bf16_kernel_equals_the_general_one(rows, H, lower_bound):
     fast = rmsnorm_quant_kernel(xt, gt, kargs).view(torch.uint8)
     general = rmsnorm_quant_kernel(xt, gt.float(), kargs).view(torch.uint8)
     assert torch.equal(fast, general)
+    # the same pair of kernels with a static scale
+    from nkilib.core.utils.common_types import QuantizationType
+    kargs = RmsNormQuantKernelArgs(quantization_type=QuantizationType.STATIC)
+    sc = f32_tensor(np.full((128, 1), 0.017, np.float32), dev)
+    fast = rmsnorm_quant_kernel(xt, gt, kargs, sc).view(torch.uint8)
+    general = rmsnorm_quant_kernel(xt, gt.float(), kargs, sc).view(torch.uint8)
+    assert tuple(fast.shape)[-1] == H and torch.equal(fast, general)
 
 
 @pytest.mark.parametrize("rows,H,quant_only", [(2, 16384, True), (160, 16384, False), (64, 4096, False)])
