@@ -127,6 +127,24 @@ def test_dense_variants(T, H, I, E, k, B, impl, act, mode, bias, skip, clamp):
     _check(o, g, f"dense {impl} act={act} mode={mode}")
 
 
+@pytest.mark.parametrize("fp8_weights", [False, True])
+def test_dense_down_weight_padded_on_I_large_tile_shape(fp8_weights):
+    """down_proj_weight [E, I_pad, H] with I_pad > I (test_moe_cte_common.py:645,663) on a shape of the large-tile
+    kernels: rows I.. of every expert's down weights hold junk that must not reach the result."""
+    c = dense_case(256, 512, 128, 4, 2, 128, seed=21, quant=fp8_weights, hidden_std=1.0)
+    rng = np.random.default_rng(21)
+    pad = 32
+    if fp8_weights:
+        junk = rng.integers(0, 0x7e, size=(4, pad, 512)).astype(np.uint8)
+        c["down_q"] = np.concatenate([c["down_q"], junk], axis=1)
+        c["down_w"] = np.concatenate([c["down_w"], np.full((4, pad, 512), 3.0, np.float32)], axis=1)
+    else:
+        c["down_w"] = np.concatenate([c["down_w"], np.full((4, pad, 512), 3.0, np.float32)], axis=1)
+    out = _run_dense(c, impl="shard_on_block", fp8_weights=fp8_weights)
+    o = from_bf16_tensor(out)[:, 0]
+    _check(o[:256], _golden_dense(c, fp8_weights=fp8_weights)[:256], f"padded I, fp8 weights {fp8_weights}")
+
+
 def _run_checkpointed(c, impl, act=0, mode=1, clamps=None, on_I=False, tp2id=None, b2e=None, fp8_weights=False):
     import torch
     from nkilib.core.moe.moe_cte import (MoECTEImplementation, MoECTESpec, QuantizationConfig, ShardOnIConfig, SkipMode,
