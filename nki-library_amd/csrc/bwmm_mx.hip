@@ -385,7 +385,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
 #pragma unroll
     for (int j = 0; j < (ROWS2 ? 2 : 1); ++j) {
       const int r = tid + 256 * j;
-      if (r < NMT * 16) s_tok[buf][r] = (r < nrows && raw[j] >= 0 && raw[j] < a.n_real) ? raw[j] : -1;
+      if (r < Cfg::ROWS) s_tok[buf][r] = (r < nrows && raw[j] >= 0 && raw[j] < a.n_real) ? raw[j] : -1;
     }
   };
   // (No branch may surround such a load: where two paths that load into the same variable meet, the compiler
@@ -956,7 +956,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       su[0] = vu.x; su[1] = vu.y; su[2] = vu.z; su[3] = vu.w;
     }
     const int pl0 = 4 * cl_e;
-    constexpr int NPS = NMT / 4;
+    constexpr int NPS = (NMT + 3) / 4;  // passes of 64 rows (the last one may hold two row tiles only)
     // Clamps as unconditional min/max against +-inf, and the activation kind as a compile-time
     // constant of the pass: a lane evaluates 128 elements here, and per-element decisions made this
     // code longer (and slower) than the K loop.
@@ -981,6 +981,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
         static_for<0, 4>([&](auto m_) {
           constexpr int ml = decltype(m_)::value;
           constexpr int mt = ps * 4 + ml;
+          if constexpr (mt < NMT) {
           // Lane c < 8 holds gate, lane c + 8 up, of the same four partitions and the same four rows.
           // The pair splits the rows: the gate lane finishes rows 0,1 of its four, the up lane rows
           // 2,3; each hands the other the two values it needs (a rotation by 8 within the 16 lanes).
@@ -1019,6 +1020,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
           for (int k = 0; k < 2; ++k) {
             const int rl = ml * 16 + 4 * g_e + 2 * hcol_e + k;
             *(float4*)(E + rl * MX_EP + q * 32 + pl0) = make_float4(y[k][0], y[k][1], y[k][2], y[k][3]);
+          }
           }
         });
         lds_barrier();
@@ -1198,26 +1200,30 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int qbase = __builtin_amdgcn_readfirstlane(qo[0]);
   const int interleave = __builtin_amdgcn_readfirstlane(a.q_off[8 * (CHUNK_CLASSES + 1)]);
   int L = w;
-  // classes in queue order (chunk_class): row-tile variants 20, 16, 8, 4, each first "not the last chunk of
-  // its expert", then "last"
-#define MX_RUN_CLASS(CLS_, NMT_, LAST_)                                                                        \
+  // classes in queue order (CHUNK_CLASS_TILES / CHUNK_CLASS_LAST in combine.hpp)
+#define MX_RUN_CLASS(CLS_)                                                                                     \
   {                                                                                                            \
     const int startL = (__builtin_amdgcn_readfirstlane(qo[CLS_]) - qbase) * a.col_tiles;                       \
     const int endL = (__builtin_amdgcn_readfirstlane(qo[CLS_ + 1]) - qbase) * a.col_tiles;                     \
     if (L < endL)                                                                                              \
-      L = mx_gemm_tiles<STAGE, NMT_, LAST_, WFMT>(a, smem, s_tok, s_aff, s_bias, (float(*)[MX_ROWS_MAX])s_rs,  \
-                                                  (float(*)[MXT])s_wsc, L, startL, endL, W, qbase,            \
-                                                  interleave);                                                \
+      L = mx_gemm_tiles<STAGE, CHUNK_CLASS_TILES[CLS_], CHUNK_CLASS_LAST[CLS_], WFMT>(                         \
+          a, smem, s_tok, s_aff, s_bias, (float(*)[MX_ROWS_MAX])s_rs, (float(*)[MXT])s_wsc, L, startL, endL,  \
+          W, qbase, interleave);                                                                               \
     __syncthreads();                                                                                           \
   }
-  MX_RUN_CLASS(0, 20, false)
-  MX_RUN_CLASS(1, 20, true)
-  MX_RUN_CLASS(2, 16, false)
-  MX_RUN_CLASS(3, 16, true)
-  MX_RUN_CLASS(4, 8, false)
-  MX_RUN_CLASS(5, 8, true)
-  MX_RUN_CLASS(6, 4, false)
-  MX_RUN_CLASS(7, 4, true)
+  static_assert(CHUNK_CLASSES == 12, "one MX_RUN_CLASS per class");
+  MX_RUN_CLASS(0)
+  MX_RUN_CLASS(1)
+  MX_RUN_CLASS(2)
+  MX_RUN_CLASS(3)
+  MX_RUN_CLASS(4)
+  MX_RUN_CLASS(5)
+  MX_RUN_CLASS(6)
+  MX_RUN_CLASS(7)
+  MX_RUN_CLASS(8)
+  MX_RUN_CLASS(9)
+  MX_RUN_CLASS(10)
+  MX_RUN_CLASS(11)
 #undef MX_RUN_CLASS
 }
 

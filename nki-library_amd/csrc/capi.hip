@@ -121,40 +121,49 @@ int validate(const moe_bwmm_args* a) {
   return MOE_OK;
 }
 
-// The fp8-row kind runs on the large-tile kernels (bwmm_mx.hip, MX_WFMT_ROW8) when the shape is one of theirs and
-// every 32-bit offset they form stays in range; otherwise on the general tiled kernel.  The choice depends on the
-// shape only, because it also decides what the kept weight copies look like.
-bool row8_fast(const moe_bwmm_args* a) {
+// The dense kinds on the large-tile kernels (bwmm_mx.hip).  Two separate questions:
+//   *_shape:     is the expert shape (kind, weight type, H, I, E) one of those kernels', with every 32-bit offset they
+//                form inside one expert's weights and tables in range?  This alone decides what a KEPT weight copy
+//                holds (x4 read order, or K-contiguous rows for the general kernel): a copy prepared in one call must
+//                mean the same in every other call with the same weights, whatever its token count.
+//   *_call_fits: do this call's activations (token count, number of blocks) fit the kernels' 32-bit row offsets?
+// A call runs there when both hold (and, for bf16, it asks for no activation checkpoints, which those epilogues do not
+// write).  A call on such a shape that cannot run there uses the general kernel on K-contiguous copies of its own,
+// made per call in the workspace: kept copies are in the other order and are ignored (*_kept_usable).
+bool row8_shape(const moe_bwmm_args* a) {
   if (a->kind != MOE_KIND_FP8_ROW || !mx_fast_path_ok(a->H, a->I)) return false;
   const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
-  const int64_t slots = a->N * a->B, Iw = (a->I + 127) / 128 * 128;
   const int64_t pI = a->I > 512 ? 128 : a->I / 4, nI = (a->I + 511) / 512;
-  if (a->T1 * (a->H + 4) >= lim32 || slots * Iw >= lim32) return false;
   if (2 * a->H * a->I >= lim31 || pI * nI * a->H * 4 >= lim31) return false;
-  if (slots * 4 >= lim32 || a->T1 * a->E * 4 >= lim32 || a->E * 2 * a->I * 4 >= lim32 || a->E * a->H * 4 >= lim32)
-    return false;
+  if (a->E * 2 * a->I * 4 >= lim32 || a->E * a->H * 4 >= lim32) return false;
   return true;
 }
-// The bf16 kind (bf16 weights, or fp8 weights widened to bf16 in the copy) runs there too (MX_WFMT_BF16) when the K extents in bytes (2H, 2I) are shapes of
-// those kernels and the offsets fit -- which, as above, also decides what kept weight copies look like -- except for
-// calls that ask for activation checkpoints, which their epilogues do not write: those run the general kernel on
-// copies of their own, made per call (kept copies are in the other order).
+bool row8_call_fits(const moe_bwmm_args* a) {
+  const int64_t lim32 = (int64_t)1 << 32;
+  const int64_t slots = a->N * a->B, Iw = (a->I + 127) / 128 * 128;
+  return a->T1 * (a->H + 4) < lim32 && slots * Iw < lim32 && slots * 4 < lim32 && a->T1 * a->E * 4 < lim32;
+}
+bool row8_fast(const moe_bwmm_args* a) { return row8_shape(a) && row8_call_fits(a); }
+bool row8_kept_usable(const moe_bwmm_args* a) { return row8_fast(a) || !row8_shape(a); }
+// (bf16 weights, or fp8 weights widened to bf16 in the copy; K extents in bytes: 2H, 2I)
 bool bf16_fast_shape(const moe_bwmm_args* a) {
   if (a->kind != MOE_KIND_BF16 || (a->weight_dtype != MOE_DT_BF16 && a->weight_dtype != MOE_DT_FP8_E4M3)) return false;
   if (a->H % 256 != 0 || a->I % 128 != 0) return false;
   const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
-  const int64_t slots = a->N * a->B, Ib = 2 * a->I, Hb = 2 * a->H;
+  const int64_t Ib = 2 * a->I, Hb = 2 * a->H;
   const int64_t pI = Ib > 512 ? 128 : Ib / 4, nI = (Ib + 511) / 512;
-  if (a->T1 * Hb >= lim32 || slots * Ib >= lim32) return false;
   if (2 * Hb * a->I >= lim31 || pI * nI * a->H * 4 >= lim31) return false;
-  if (slots * 4 >= lim32 || a->T1 * a->E * 4 >= lim32 || a->E * 2 * a->I * 4 >= lim32 || a->E * a->H * 4 >= lim32)
-    return false;
+  if (a->E * 2 * a->I * 4 >= lim32 || a->E * a->H * 4 >= lim32) return false;
   return true;
 }
-bool bf16_fast(const moe_bwmm_args* a) {
-  return bf16_fast_shape(a) && !a->gate_up_activations_T && !a->down_activations;
+bool bf16_call_fits(const moe_bwmm_args* a) {
+  const int64_t lim32 = (int64_t)1 << 32;
+  const int64_t slots = a->N * a->B;
+  return a->T1 * 2 * a->H < lim32 && slots * 2 * a->I < lim32 && slots * 4 < lim32 && a->T1 * a->E * 4 < lim32;
 }
-// kept copies of the bf16 kind's weights are in the order this call reads
+bool bf16_fast(const moe_bwmm_args* a) {
+  return bf16_fast_shape(a) && bf16_call_fits(a) && !a->gate_up_activations_T && !a->down_activations;
+}
 bool bf16_kept_usable(const moe_bwmm_args* a) { return bf16_fast(a) || !bf16_fast_shape(a); }
 // What a kept copy of the fp8-row (bf16) weights holds on that path: the weights in x4 order, one expert's worth of
 // E8M0 block scales of 127 (2^0) that serves every expert, and one row of activation block scales of 127 (the bf16
@@ -223,10 +232,11 @@ Plan make_plan(const moe_bwmm_args* a) {
       p.nI = (a->I + 511) / 512;
       p.pI = a->I > 512 ? 128 : a->I / 4;
     }
-    if (!a->gate_up_proj_weight_kmajor) {
+    const bool kept = row8_kept_usable(a);
+    if (!(a->gate_up_proj_weight_kmajor && kept)) {
       p.wt1 = off; off += al256(r8 ? row8_copy(a, 0).total : (size_t)a->E * 2 * a->I * p.Hk);
     }
-    if (!a->down_proj_weight_kmajor) {
+    if (!(a->down_proj_weight_kmajor && kept)) {
       p.wt2 = off; off += al256(r8 ? row8_copy(a, 1).total : (size_t)a->E * a->H * p.Iw);
     }
   }
@@ -235,11 +245,11 @@ Plan make_plan(const moe_bwmm_args* a) {
   return p;
 }
 
-// K-contiguous copy of the gate/up (which == 0) or down (which == 1) weights of the BF16 / FP8_ROW kinds.
-// (bf16_x4: the bf16 kind's copy in the large-tile kernels' order rather than K-contiguous)
-int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hipStream_t s, bool bf16_x4) {
+// Copy of the gate/up (which == 0) or down (which == 1) weights of the BF16 / FP8_ROW kinds: in the large-tile
+// kernels' x4 read order (x4), else K-contiguous rows for the general kernel.
+int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hipStream_t s, bool x4) {
   const int64_t Ipad = a->I_pad > 0 ? a->I_pad : a->I;
-  if (bf16_x4) {
+  if (x4 && a->kind == MOE_KIND_BF16) {
     const Row8Copy c = row8_copy(a, which);
     int rc = launch_relayout_x4_bf16(a->gate_up_proj_weight, a->down_proj_weight, a->weight_dtype == MOE_DT_FP8_E4M3,
                                      (uint8_t*)dst, which, a->E, a->H, a->I, Ipad, s);
@@ -253,7 +263,7 @@ int kmajor_copy(const moe_bwmm_args* a, const Plan& p, int which, void* dst, hip
                                   a->H * 2 * a->I, a->I, s);
     return launch_transpose_w16(a->down_proj_weight, w8, (uint16_t*)dst, a->I, a->H, a->H, p.Iw, a->E, 1, Ipad * a->H, 0, s);
   }
-  if (row8_fast(a)) {
+  if (x4) {
     const Row8Copy c = row8_copy(a, which);
     int rc = launch_relayout_x4((const uint8_t*)a->gate_up_proj_weight, (const uint8_t*)a->down_proj_weight,
                                 (uint8_t*)dst, which, a->E, a->H, a->I, Ipad, s);
@@ -284,7 +294,7 @@ extern "C" size_t moe_kmajor_weights_bytes(const moe_bwmm_args* a, int which) {
                                  : 0;
   const Plan p = make_plan(a);
   const size_t es = a->kind == MOE_KIND_BF16 ? 2 : 1;
-  if (row8_fast(a) || bf16_fast_shape(a)) return row8_copy(a, which).total;
+  if (row8_shape(a) || bf16_fast_shape(a)) return row8_copy(a, which).total;
   return which == 0 ? (size_t)a->E * 2 * a->I * p.Hk * es : (size_t)a->E * a->H * p.Iw * es;
 }
 
@@ -303,9 +313,10 @@ extern "C" int moe_prepare_kmajor_weights(const moe_bwmm_args* a, void* gate_up_
   if (!gate_up_kmajor || !down_kmajor) return MOE_E_BAD_ARG;
   if ((((uintptr_t)gate_up_kmajor) & 255) != 0 || (((uintptr_t)down_kmajor) & 255) != 0) return MOE_E_BAD_ARG;
   const Plan p = make_plan(a);
-  rc = kmajor_copy(a, p, 0, gate_up_kmajor, (hipStream_t)stream, bf16_fast_shape(a));
+  const bool x4 = row8_shape(a) || bf16_fast_shape(a);  // from the expert shape alone, see row8_shape
+  rc = kmajor_copy(a, p, 0, gate_up_kmajor, (hipStream_t)stream, x4);
   if (rc != MOE_OK) return rc;
-  return kmajor_copy(a, p, 1, down_kmajor, (hipStream_t)stream, bf16_fast_shape(a));
+  return kmajor_copy(a, p, 1, down_kmajor, (hipStream_t)stream, x4);
 }
 
 extern "C" size_t moe_blockwise_workspace_bytes(const moe_bwmm_args* a) {
@@ -411,16 +422,18 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     gx1 = (unsigned)((a->I + 127) / 128);
     // the reference stores the weights N-contiguous ([E, H, 2, I], [E, I_pad, H]); both MFMA operands are read
     // along K, so each stage first writes a K-contiguous copy of its weights
-    g1.W = a->gate_up_proj_weight_kmajor ? (const uint8_t*)a->gate_up_proj_weight_kmajor : ws + p.wt1;
-    g2.W = a->down_proj_weight_kmajor ? (const uint8_t*)a->down_proj_weight_kmajor : ws + p.wt2;
+    const bool kept = row8_kept_usable(a);
+    const bool have1 = a->gate_up_proj_weight_kmajor && kept, have2 = a->down_proj_weight_kmajor && kept;
+    g1.W = have1 ? (const uint8_t*)a->gate_up_proj_weight_kmajor : ws + p.wt1;
+    g2.W = have2 ? (const uint8_t*)a->down_proj_weight_kmajor : ws + p.wt2;
     g1.Kp = p.Hk;
     g2.Kp = p.Iw;
-    if ((stages & MOE_STAGE_GATE_UP) && !a->gate_up_proj_weight_kmajor) {
-      rc = kmajor_copy(a, p, 0, ws + p.wt1, s, false);
+    if ((stages & MOE_STAGE_GATE_UP) && !have1) {
+      rc = kmajor_copy(a, p, 0, ws + p.wt1, s, row8_fast(a));
       if (rc != MOE_OK) return rc;
     }
-    if ((stages & MOE_STAGE_DOWN) && !a->down_proj_weight_kmajor) {
-      rc = kmajor_copy(a, p, 1, ws + p.wt2, s, false);
+    if ((stages & MOE_STAGE_DOWN) && !have2) {
+      rc = kmajor_copy(a, p, 1, ws + p.wt2, s, row8_fast(a));
       if (rc != MOE_OK) return rc;
     }
   }

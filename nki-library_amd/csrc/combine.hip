@@ -161,10 +161,7 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     if (in_lds) s_cx[i] = v;
     else chunk_xcd[i] = v;
   };
-  auto work_of = [&](int i) {
-    const int r = rows_of(i);
-    return r <= 64 ? 4 : r <= 128 ? 8 : r <= 256 ? 16 : 20;
-  };
+  auto work_of = [&](int i) { return chunk_row_tiles(rows_of(i), true); };
   int wcarry = 0;
   for (int i0 = 0; i0 < n; i0 += 1024) {
     const int i = i0 + threadIdx.x;

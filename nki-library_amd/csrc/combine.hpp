@@ -30,12 +30,25 @@ struct Bookkeeping {
   int64_t max_chunks;
 };
 
-constexpr int CHUNK_CLASSES = 8;
-// class of a chunk: its row-tile variant (0: up to 64 rows, 1: 128, 2: 256, 3: 320), largest first, then whether
-// it is the last chunk of its expert
+// Classes of chunks = instances of the large-tile kernels' tile loop: how many 16-row tiles the instance multiplies
+// (at least the chunk's rows / 16) and whether the chunk is the last one of its expert (its weights are then
+// streamed past the L2).  Last chunks, which carry an expert's ragged remainder, choose among eight row-tile counts,
+// so that at most one or two tiles of a chunk multiply padding (a router's 256 +- 15 rows per expert made one MFMA in
+// eight multiply padding with the counts 4 / 8 / 16 / 20 alone); chunks that are not the last of their expert hold
+// exactly CHUNK_ROWS rows unless chunks are interleaved (see build_chunks), and choose among four.  Queue order =
+// class order: largest tiles first, so that a launch ends on its small ones.
+constexpr int CHUNK_CLASSES = 12;
+constexpr int CHUNK_CLASS_TILES[CHUNK_CLASSES] = {20, 20, 18, 16, 16, 14, 12, 10, 8, 8, 4, 4};
+constexpr bool CHUNK_CLASS_LAST[CHUNK_CLASSES] = {false, true, true, false, true, true, true, true, false, true, false, true};
+// 16-row tiles of the instance that runs a chunk of `rows` rows
+__host__ __device__ inline int chunk_row_tiles(int rows, bool last) {
+  if (!last) return rows <= 64 ? 4 : rows <= 128 ? 8 : rows <= 256 ? 16 : 20;
+  return rows <= 64 ? 4 : rows <= 128 ? 8 : 2 * ((rows + 31) / 32);
+}
 __host__ __device__ inline int chunk_class(int rows, bool last) {
-  const int v = rows <= 64 ? 0 : rows <= 128 ? 1 : rows <= 256 ? 2 : 3;
-  return (3 - v) * 2 + (last ? 1 : 0);
+  const int t = chunk_row_tiles(rows, last);
+  if (!last) return t == 20 ? 0 : t == 16 ? 3 : t == 8 ? 8 : 10;
+  return t == 20 ? 1 : t == 18 ? 2 : t == 16 ? 4 : t == 14 ? 5 : t == 12 ? 6 : t == 10 ? 7 : t == 8 ? 9 : 11;
 }
 
 constexpr int CHUNK_ROWS = 256;      // rows of every chunk of a run but the last

@@ -133,3 +133,33 @@ def test_static_scratch_entry_point_rejects_sizes_beyond_its_scratch():
     assert rc == -7 and b"allocates nothing" in L.moe_error_string(rc)
     assert L.moe_build_blocks_static(None, 4, 2, 256, 128, 600, 0, 0, fake, fake, None, 0, None, None) == -1
     assert L.moe_build_blocks_workspace_bytes(512) == 133136  # MOE_BUILD_BLOCKS_STATIC_BYTES in the header
+
+
+@pytest.mark.parametrize("kind,shape", [("KIND_FP8_ROW", (4096, 14336, 8)), ("KIND_BF16", (2048, 14336, 8))])
+def test_kept_weight_copies_depend_on_the_expert_shape_only(kind, shape):
+    """What a kept weight copy holds (x4 read order or K-contiguous rows) follows from kind, weight type and
+    (H, I, E) alone.  A call whose activations outgrow the large-tile kernels' 32-bit row offsets must not change the
+    meaning of the copies: it ignores them and plans K-contiguous copies of its own in the workspace."""
+    from nkilib import _native as nv
+
+    L = nv.lib()
+    H, I, E = shape
+    kind = getattr(nv, kind)
+    es = 2 if kind == nv.KIND_BF16 else 1
+    small = _valid_args(nv, kind, 4097, H, I, E, 128, 71)
+    n_big = 2**32 // (128 * I * es) + 1  # N * B * I * es >= 2^32: past the large-tile kernels' offsets
+    big = _valid_args(nv, kind, 150001, H, I, E, 128, n_big)
+    nbytes = lambda a, which: L.moe_kmajor_weights_bytes(ctypes.byref(a), which)
+    ws = lambda a: L.moe_blockwise_workspace_bytes(ctypes.byref(a))
+    for which in (0, 1):
+        assert nbytes(small, which) > 0
+        assert nbytes(small, which) == nbytes(big, which)
+        # the x4 copies carry their unit scale tables behind the weights: more bytes than bare K-contiguous rows
+        assert nbytes(small, which) > E * (2 if which == 0 else 1) * I * H * es
+    fake = ctypes.c_void_p(4096)
+    ws_small, ws_big = ws(small), ws(big)
+    for a in (small, big):
+        a.gate_up_proj_weight_kmajor = fake
+        a.down_proj_weight_kmajor = fake
+    assert ws(small) < ws_small - 2 * E * I * H * es  # kept copies used: none planned in the workspace
+    assert ws(big) == ws_big  # kept copies ignored: the call still plans its own
