@@ -67,6 +67,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sustain-seconds", type=float, default=2.0,
+                    help="after the timed steps keep running the same step for at least this long and report its pace "
+                         "and the shader clock the GEMMs held (extra keys; 0 skips it)")
     ap.add_argument("--cpu-blocks", type=int, default=48, help="blocks of the workload timed on the CPU oracle (48: 10-20 s)")
     ap.add_argument("--with-router", action="store_true",
                     help="start from hidden states: time the router top-k front end (synthetic router weights) as a "
@@ -379,6 +382,30 @@ def main():
             stage_ms[n] += evs[i].elapsed_time(evs[i + 1])
     stage_ms = {n: v / args.steps for n, v in stage_ms.items()}
 
+    # Sustained pace: the same step, back to back, for at least --sustain-seconds more (the clock under load is a
+    # power-management outcome with a time constant far beyond the 20 timed steps).  Workgroup 0 of each GEMM launch
+    # reports its shader cycles and the ticks of the constant 100 MHz counter: their ratio is the clock it ran at.
+    sustained = None
+    if args.sustain_seconds > 0:
+        clk = torch.zeros(4, dtype=torch.int64, device=dev)
+        _launch.gemm_clock_probe = clk
+        n_sus = 0
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        while True:
+            for _ in range(args.steps):
+                step(False)
+            n_sus += args.steps
+            torch.cuda.synchronize()
+            if time.perf_counter() - t1 >= args.sustain_seconds:
+                break
+        sus_ms = (time.perf_counter() - t1) * 1e3 / n_sus
+        _launch.gemm_clock_probe = None
+        c = [int(v) for v in clk.cpu().tolist()]
+        sustained = {"ms_per_step": sus_ms, "steps": n_sus,
+                     "ghz_gate_up": (c[0] / c[1] * 0.1) if c[1] else None,
+                     "ghz_down": (c[2] / c[3] * 0.1) if c[3] else None}
+
     routed = int((tp2id.reshape(-1) < T).sum().item())  # == T*k
     flops_layer = 6.0 * routed * H * I
     flops_gate_up = 4.0 * routed * H * I
@@ -420,6 +447,10 @@ def main():
         # 256 CUs x 4 SIMDs, one 16x16x128 MFMA (65536 flop) per 32 cycles and SIMD
         roofline["sclk_ghz_profiled"] = sclk_ghz
         roofline["mfma_peak_at_that_clock_TFLOPs"] = round(1024 * 2048 * sclk_ghz / 1e3, 1)
+    if sustained and sustained["ghz_gate_up"]:
+        # the clock the gate/up launch itself reported at the end of the sustained run
+        roofline["sclk_ghz_sustained"] = round(sustained["ghz_gate_up"], 3)
+        roofline["mfma_peak_at_sustained_clock_TFLOPs"] = round(1024 * 2048 * sustained["ghz_gate_up"] / 1e3, 1)
 
     res = {
         "metric": METRIC,
@@ -451,6 +482,12 @@ def main():
         },
         "roofline": roofline,
     }
+    if sustained:
+        res["sustained_ms_per_step"] = round(sustained["ms_per_step"], 4)
+        res["sustained_steps"] = sustained["steps"]
+        res["sustained_TFLOPs"] = round(flops_layer / (sustained["ms_per_step"] * 1e-3) / 1e12, 2)
+        res["sustained_sclk_ghz"] = {"gate_up": round(sustained["ghz_gate_up"], 3) if sustained["ghz_gate_up"] else None,
+                                     "down": round(sustained["ghz_down"], 3) if sustained["ghz_down"] else None}
     if not args.no_cpu_baseline and not fp4:
         res["cpu_baseline"] = cpu_baseline(cfg, t, tp2id, b2e, args.cpu_blocks)
     print(json.dumps(res), flush=True)

@@ -81,10 +81,15 @@ int moe_rmsnorm_quant_fp8_static(const void* x, int x_dtype, const void* gamma, 
  * n = bf16(x * (1/sqrt(sum(x^2)/hidden_actual + eps)) * gamma) when do_norm, else bf16(x);
  * then MXFP8-e4m3 with one E8M0 scale per 32 consecutive k', k' = tile*512 + p*4 + q for
  * h = q*(H/4) + tile*128 + p.  H % 512 == 0, H <= 16384.
- * out_norm (nullable): bf16 [128, rows, H/128], element [p, t, h1] = n[t, h1*128 + p]. */
-int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out_q,
-                            void* out_scale, void* out_norm, int64_t rows, int64_t H, float eps,
-                            int64_t hidden_actual, int do_norm, int layout, void* stream);
+ * out_norm (nullable): bf16 [128, rows, H/128], element [p, t, h1] = n[t, h1*128 + p].
+ * residual / out_residual (both or neither; [rows, H] of x's type): the fused residual add of
+ * rmsnorm_mx_quantize_tkg.py:29-40,214-232 (golden test_rmsnorm_mx_quantize_tkg.py:104-117):
+ * hidden = x + residual rounded to x's type is what is normalised and quantised, and it is written to
+ * out_residual.  (The reference's hidden_dim_tp=False has no kernel behind it there either:
+ * "Only hidden_dim_tp=True is supported", norm_tkg_utils.py:467.) */
+int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* residual, void* out_residual, const void* gamma,
+                            int gamma_dtype, void* out_q, void* out_scale, void* out_norm, int64_t rows, int64_t H,
+                            float eps, int64_t hidden_actual, int do_norm, int layout, void* stream);
 
 /* ---- router top-k front end ----------------------------------------------------------- */
 
@@ -267,6 +272,11 @@ typedef struct moe_bwmm_args {
    * output_shard1 + t*out_row_stride elements and the combine pass writes it as zeros along with row t of
    * `output`, so the caller needs no separate clear. */
   void* output_shard1;
+  /* Nullable, no counterpart in the reference: device int64 [4].  Workgroup 0 of the large-tile gate/up GEMM writes
+   * [0] = shader clock cycles and [1] = ticks of the constant 100 MHz counter between its first and last
+   * instruction, the down GEMM the same into [2], [3]: cycles / ticks x 0.1 is the shader clock in GHz that the
+   * part held under that launch (it is set by power management, not by the data sheet).  Read by bench.py. */
+  int64_t* gemm_clocks;
 } moe_bwmm_args;
 
 /* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /

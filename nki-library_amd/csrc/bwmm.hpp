@@ -81,6 +81,7 @@ struct MxArgs {
                            // of constants for every row)
   float* Y32;              // stage 1 output of this format: fp32 [N*B, y32_stride], columns in natural order
   int64_t y32_stride;
+  int64_t* clk;            // nullable: workgroup 0 stores its shader cycles and 100 MHz ticks from start to end here
   // MX_WFMT_BF16 (the bf16 kind on these kernels): both operands bf16, read as bytes exactly like the 8-bit formats
   // (a 128-byte K slice is 64 elements, multiplied by two v_mfma_f32_16x16x32_bf16 where the 8-bit formats issue
   // one 128-deep MFMA), so H (gate/up) and I (down) are the K extents in BYTES; no scales of any kind (w_cscale

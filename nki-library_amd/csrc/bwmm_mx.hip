@@ -1196,6 +1196,8 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // consecutive items are of one class, i.e. one instance of the code below, which carries its loads from tile
   // to tile.
   const int xcd = blockIdx.x & 7, w = blockIdx.x >> 3, W = gridDim.x >> 3;
+  // (for a caller that wants to know the clock the part held under this launch, see MxArgs::clk)
+  const long long clk0 = a.clk ? clock64() : 0, tick0 = a.clk ? wall_clock64() : 0;
   const int32_t* qo = a.q_off + xcd * (CHUNK_CLASSES + 1);
   const int qbase = __builtin_amdgcn_readfirstlane(qo[0]);
   const int interleave = __builtin_amdgcn_readfirstlane(a.q_off[8 * (CHUNK_CLASSES + 1)]);
@@ -1225,6 +1227,10 @@ __global__ __launch_bounds__(MXT) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   MX_RUN_CLASS(10)
   MX_RUN_CLASS(11)
 #undef MX_RUN_CLASS
+  if (a.clk && blockIdx.x == 0 && threadIdx.x == 0) {
+    a.clk[0] = clock64() - clk0;
+    a.clk[1] = wall_clock64() - tick0;
+  }
 }
 
 #define MX_CAT_(a, b, c, d) a##b##c##d

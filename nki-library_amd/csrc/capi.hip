@@ -6,8 +6,8 @@
 
 using namespace moe;
 
-extern "C" int moe_rmsnorm_quant_mxfp8(const void*, int, const void*, int, void*, void*, void*, int64_t, int64_t, float,
-                                       int64_t, int, int, void*);
+extern "C" int moe_rmsnorm_quant_mxfp8(const void*, int, const void*, void*, const void*, int, void*, void*, void*, int64_t,
+                                       int64_t, float, int64_t, int, int, void*);
 
 extern "C" const char* moe_error_string(int code) {
   switch (code) {
@@ -24,7 +24,7 @@ extern "C" const char* moe_error_string(int code) {
   }
 }
 
-extern "C" int moe_abi_version(void) { return 5; }
+extern "C" int moe_abi_version(void) { return 6; }
 
 extern "C" int moe_check_device(void) {
   int dev = 0;
@@ -384,8 +384,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     if (!xs) {
       // online activation quantisation (moe_cte_mx_utils.py:730-771): bf16 rows -> MXFP8 in k' order
       if (stages & MOE_STAGE_ACT_QUANT) {
-        rc = moe_rmsnorm_quant_mxfp8(a->hidden_states, MOE_DT_BF16, nullptr, MOE_DT_BF16, ws + p.xq, ws + p.xs,
-                                     nullptr, a->T1, a->H, 0.f, a->H, 0, MOE_MX_LAYOUT_TOKEN_MAJOR, stream);
+        rc = moe_rmsnorm_quant_mxfp8(a->hidden_states, MOE_DT_BF16, nullptr, nullptr, nullptr, MOE_DT_BF16, ws + p.xq,
+                                     ws + p.xs, nullptr, a->T1, a->H, 0.f, a->H, 0, MOE_MX_LAYOUT_TOKEN_MAJOR, stream);
         if (rc != MOE_OK) return rc;
       }
       xq = ws + p.xq;
@@ -507,6 +507,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
         m1.w_cscale = (const float*)a->gate_up_proj_scale;
       }
       if (bf_fast) m1.H = 2 * a->H;  // K in bytes
+      m1.clk = a->gemm_clocks;
 
       // column tiles of 32 partitions x 4 q, gate and up: 4 per full intermediate tile + those of a short last one
       rc = launch_mx_gemm(1, m1, (unsigned)((a->I / 512) * 4 + (a->I % 512) / 128), gyc, s);
@@ -543,6 +544,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
         m2.I = 2 * a->I;  // K in bytes
         m2.a_rscale = nullptr;
       }
+      m2.clk = a->gemm_clocks ? a->gemm_clocks + 2 : nullptr;
 
       rc = launch_mx_gemm(2, m2, (unsigned)(a->H / 256), gyc, s);
     } else {

@@ -268,6 +268,69 @@ __global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
     inv_scan(cnt, off, n_real, s_ws);
 }
 
+// The whole bookkeeping of a small problem (decode-sized: a few ten thousand slots) by ONE workgroup of 1024
+// threads in one launch: clear the per-token counts, find the active blocks and their valid rows, count the slots
+// per token, build the expert chunks and the work queues, scan the counts and fill the token -> slot lists.  The
+// four launches it replaces take longer to start than to run at such sizes.  Steps communicate through global
+// memory that this workgroup alone writes and reads, ordered by workgroup barriers.
+__global__ __launch_bounds__(1024) void prep_small_kernel(
+    const int32_t* __restrict__ tp2id, const int32_t* __restrict__ b2e, const int32_t* __restrict__ conditions,
+    int64_t n_conditions, int64_t N, int64_t B, int64_t E, int64_t n_real, int32_t* __restrict__ n_active,
+    int32_t* __restrict__ valid_rows, int32_t* __restrict__ cnt, int64_t clear_words, int32_t* __restrict__ n_chunks,
+    int32_t* __restrict__ chunk_slot, int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
+    int32_t* __restrict__ chunk_xcd, int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off, int64_t max_chunks,
+    int32_t* __restrict__ off, int32_t* __restrict__ cursor, int32_t* __restrict__ list) {
+  __shared__ int s_ws[16];
+  __shared__ int s_first_zero;
+  for (int64_t i = threadIdx.x; i < clear_words; i += blockDim.x) cnt[i] = 0;  // cnt and cursor are adjacent
+  if (threadIdx.x == 0) s_first_zero = (int)N;
+  __threadfence_block();
+  __syncthreads();
+  if (conditions) {
+    const int64_t lim = n_conditions < N ? n_conditions : N;
+    for (int64_t i = threadIdx.x; i < lim; i += blockDim.x)
+      if (conditions[i] == 0) atomicMin(&s_first_zero, (int)i);
+  }
+  __syncthreads();
+  const int na = s_first_zero;
+  if (threadIdx.x == 0) *n_active = na;
+  // a wave per block: valid rows = 1 + last row with a real token; slots per token
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  for (int64_t b = wave; b < N; b += nwaves) {
+    int v = 0;
+    const int e = b2e[b];
+    if (b < na && e >= 0 && e < E) {
+      for (int64_t r = lane; r < B; r += 64) {
+        const int id = tp2id[b * B + r];
+        if (id >= 0 && id < n_real) {
+          v = (int)r + 1;
+          atomicAdd(&cnt[id], 1);
+        }
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+    if (lane == 0) valid_rows[b] = v;
+  }
+  __threadfence_block();
+  __syncthreads();
+  build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, chunk_xcd, q_chunk,
+               q_off, max_chunks, s_ws);
+  __syncthreads();
+  inv_scan(cnt, off, n_real, s_ws);
+  __threadfence_block();
+  __syncthreads();
+  for (int64_t s = threadIdx.x; s < N * B; s += blockDim.x) {
+    const int64_t b = s / B, r = s % B;
+    if (r >= valid_rows[b]) continue;
+    const int id = tp2id[s];
+    if (id >= 0 && id < n_real) {
+      const int p = atomicAdd(&cursor[id], 1);
+      list[off[id] + p] = (int32_t)s;
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict__ tp2id,
                                                        const int32_t* __restrict__ valid_rows, int64_t N, int64_t B,
                                                        int64_t n_real, const int32_t* __restrict__ off,
@@ -380,10 +443,21 @@ Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
   return k;
 }
 
+// up to this many slots and tokens the bookkeeping is one launch of one workgroup (prep_small_kernel)
+constexpr int64_t PREP_SMALL_SLOTS = 40960, PREP_SMALL_TOKENS = 4096;
+
 int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hipStream_t s) {
   // cnt and cursor are adjacent: one clear covers both.  A fill kernel rather than a memset
   // node, so that the sequence stays safe to record into a HIP graph.
   const int64_t clear_words = (int64_t)((uint8_t*)k.off - (uint8_t*)k.cnt) / 4;
+  if (a->N * a->B <= PREP_SMALL_SLOTS && n_real <= PREP_SMALL_TOKENS) {
+    hipLaunchKernelGGL(prep_small_kernel, dim3(1), dim3(1024), 0, s, a->token_position_to_id, a->block_to_expert,
+                       a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows, k.cnt,
+                       clear_words, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.chunk_xcd, k.q_chunk,
+                       k.q_off, k.max_chunks, k.off, k.cursor, k.list);
+    MOE_CHECK_LAUNCH();
+    return MOE_OK;
+  }
   hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((clear_words + 255) / 256)), dim3(256), 0, s, k.cnt,
                      clear_words);
   MOE_CHECK_LAUNCH();

@@ -285,15 +285,38 @@ __device__ __forceinline__ void unpack8(const uint4& a, int dtype, float* v) {
   }
 }
 
+// Fused residual add of the MXFP8 front end (rmsnorm_mx_quantize_tkg.py:29-40,214-232): hidden = input + residual,
+// rounded to the input type (the reference adds into a buffer of the residual's type; its golden adds the two arrays
+// in their own type, test_rmsnorm_mx_quantize_tkg.py:104-117), kept as the row that is normalised and written out
+// as output_residual.  Eight packed 16-bit values at a time.
+__device__ __forceinline__ uint4 add8_16(const uint4& a, const uint4& b, int dtype) {
+  float x[8], y[8];
+  unpack8(a, dtype, x);
+  unpack8(b, dtype, y);
+  uint32_t w[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float s0 = x[2 * k] + y[2 * k], s1 = x[2 * k + 1] + y[2 * k + 1];
+    if (dtype == MOE_DT_BF16) {
+      w[k] = pack2_bf16(s0, s1);
+    } else {
+      const _Float16 h0 = (_Float16)s0, h1 = (_Float16)s1;  // round to nearest even
+      w[k] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+    }
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // MAXB = MX blocks per thread (1 for H <= 32 * RQ_THREADS).  A row is one load round trip, one reduction and one
 // store, so the rows in flight per CU are what fills the memory pipeline, and registers decide how many those are:
 // 16-bit inputs (X16) stay packed as loaded (16 registers per MX block instead of 32) and the normalised values,
 // which are bf16 by definition, are kept as bf16 pairs.
 template <int MAXB, bool X16>
 __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? (X16 ? 6 : 5) : 3, 8))) void rmsnorm_quant_mx_kernel(
-    const void* __restrict__ x, int x_dtype, const void* __restrict__ gamma, int gamma_dtype,
-    uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, uint16_t* __restrict__ out_norm, int64_t rows,
-    int64_t H, float eps, float hidden_actual, int do_norm, int layout, int tpr) {
+    const void* __restrict__ x, int x_dtype, const void* __restrict__ residual, void* __restrict__ out_res,
+    const void* __restrict__ gamma, int gamma_dtype, uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale,
+    uint16_t* __restrict__ out_norm, int64_t rows, int64_t H, float eps, float hidden_actual, int do_norm, int layout,
+    int tpr) {
   __shared__ double redd[16];
   // tpr = threads per row (64, 128 or 256): short rows share a workgroup, RQ_THREADS / tpr of them
   const int tpr_lg = (tpr == 64) ? 6 : ((tpr == 128) ? 7 : 8);
@@ -303,6 +326,8 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
   const int64_t row = row_ok ? row_raw : rows - 1;
   const int es = X16 ? 2 : 4;
   const void* xr = (const uint8_t*)x + row * H * es;
+  const void* rr = residual ? (const uint8_t*)residual + row * H * es : nullptr;
+  void* orr = out_res ? (uint8_t*)out_res + row * H * es : nullptr;
   const int nblk = row_ok ? (int)(H / 32) : 0;  // threads of a row past the end own no block
   const int nT = (int)(H / 512);
   const int64_t Hq = H / 4;
@@ -320,11 +345,23 @@ __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB
         float t[8];
         if constexpr (X16) {
           raw[j][q] = *(const uint4*)((const uint16_t*)xr + i);
+          if (rr) {
+            raw[j][q] = add8_16(raw[j][q], *(const uint4*)((const uint16_t*)rr + i), x_dtype);
+            if (orr) *(uint4*)((uint16_t*)orr + i) = raw[j][q];
+          }
           unpack8(raw[j][q], x_dtype, t);
         } else {
           raw[j][2 * q] = *(const uint4*)((const float*)xr + i);
           raw[j][2 * q + 1] = *(const uint4*)((const float*)xr + i + 4);
           __builtin_memcpy(t, &raw[j][2 * q], 32);
+          if (rr) {
+            float rv[8];
+            __builtin_memcpy(rv, (const float*)rr + i, 32);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) t[r] += rv[r];
+            __builtin_memcpy(&raw[j][2 * q], t, 32);
+            if (orr) __builtin_memcpy((float*)orr + i, t, 32);
+          }
         }
 #pragma unroll
         for (int r = 0; r < 8; ++r) ss += (double)t[r] * (double)t[r];
@@ -417,7 +454,8 @@ __device__ __forceinline__ uint32_t nan_to_max(uint32_t d) {
 
 template <int MAXB>
 __global__ __launch_bounds__(RQ_THREADS) __attribute__((amdgpu_waves_per_eu(MAXB == 1 ? 6 : 3, 8))) void
-rmsnorm_quant_mx_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
+rmsnorm_quant_mx_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual,
+                             uint16_t* __restrict__ out_res, const uint16_t* __restrict__ gamma,
                              uint8_t* __restrict__ out_q, uint8_t* __restrict__ out_scale, int64_t rows, int64_t H,
                              float eps, float hidden_actual, int tpr) {
   typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
@@ -440,6 +478,19 @@ rmsnorm_quant_mx_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __r
     if (blk < nblk) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) raw[j][q] = *(const uint4*)(xr + q * Hq + blk * 8);  // tile*128 + p8*8 == blk*8
+    }
+  }
+  if (residual != nullptr) {  // hidden = bf16(input + residual): the row that is normalised and written back
+#pragma unroll
+    for (int j = 0; j < MAXB; ++j) {
+      const int blk = j * tpr + lt;
+      if (blk < nblk) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          raw[j][q] = add8_16(raw[j][q], *(const uint4*)(residual + row * H + q * Hq + blk * 8), MOE_DT_BF16);
+          if (out_res != nullptr) *(uint4*)(out_res + row * H + q * Hq + blk * 8) = raw[j][q];
+        }
+      }
     }
   }
 #pragma unroll
@@ -573,10 +624,15 @@ extern "C" int moe_rmsnorm_quant_fp8_static(const void* x, int x_dtype, const vo
   return MOE_OK;
 }
 
-extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* gamma, int gamma_dtype, void* out_q,
-                                       void* out_scale, void* out_norm, int64_t rows, int64_t H, float eps,
-                                       int64_t hidden_actual, int do_norm, int layout, void* stream) {
+extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* residual, void* out_residual,
+                                       const void* gamma, int gamma_dtype, void* out_q, void* out_scale,
+                                       void* out_norm, int64_t rows, int64_t H, float eps, int64_t hidden_actual,
+                                       int do_norm, int layout, void* stream) {
   if (!x || !out_q || !out_scale || rows < 0 || H <= 0 || !valid_in_dtype(x_dtype)) return MOE_E_BAD_ARG;
+  // the sum is needed by the caller's residual stream: the reference requires output_residual with residual
+  // (norm_tkg_utils.py:473-476)
+  if ((residual != nullptr) != (out_residual != nullptr)) return MOE_E_BAD_ARG;
+  if (residual && ((((uintptr_t)residual) & 15) != 0 || (((uintptr_t)out_residual) & 15) != 0)) return MOE_E_BAD_ARG;
   if (do_norm && (!gamma || !valid_in_dtype(gamma_dtype))) return MOE_E_BAD_ARG;
   if (layout < 0 || layout > 2 || eps < 0.f) return MOE_E_BAD_ARG;
   if (H % 512 != 0 || H > RQ_MAX_H) return MOE_E_BAD_SHAPE;
@@ -590,15 +646,17 @@ extern "C" int moe_rmsnorm_quant_mxfp8(const void* x, int x_dtype, const void* g
   const int rpw = RQ_THREADS / tpr;  // rows per workgroup
   const dim3 grid((unsigned)((rows + rpw - 1) / rpw)), block(RQ_THREADS);
   auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, x, x_dtype, gamma, gamma_dtype, (uint8_t*)out_q,
-                       (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H, eps, ha, do_norm, layout, tpr);
+    hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, x, x_dtype, residual, out_residual, gamma,
+                       gamma_dtype, (uint8_t*)out_q, (uint8_t*)out_scale, (uint16_t*)out_norm, rows, H, eps, ha, do_norm,
+                       layout, tpr);
   };
   const bool fast = x_dtype == MOE_DT_BF16 && do_norm && gamma_dtype == MOE_DT_BF16 && !out_norm &&
                     layout == MOE_MX_LAYOUT_TOKEN_MAJOR;
   if (fast) {
     auto launch_fast = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, (const uint16_t*)x, (const uint16_t*)gamma,
-                         (uint8_t*)out_q, (uint8_t*)out_scale, rows, H, eps, ha, tpr);
+      hipLaunchKernelGGL(kernel, grid, block, 0, (hipStream_t)stream, (const uint16_t*)x, (const uint16_t*)residual,
+                         (uint16_t*)out_residual, (const uint16_t*)gamma, (uint8_t*)out_q, (uint8_t*)out_scale, rows, H,
+                         eps, ha, tpr);
     };
     if (H <= 32 * RQ_THREADS) launch_fast(rmsnorm_quant_mx_bf16_kernel<1>);
     else launch_fast(rmsnorm_quant_mx_bf16_kernel<MXQ_MAX_BLK>);

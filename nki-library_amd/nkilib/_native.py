@@ -99,6 +99,7 @@ class BwmmArgs(ctypes.Structure):
         ("gate_up_proj_weight_kmajor", c_void_p),
         ("down_proj_weight_kmajor", c_void_p),
         ("output_shard1", c_void_p),
+        ("gemm_clocks", c_void_p),
     ]
 
 
@@ -130,8 +131,8 @@ def lib():
     L.moe_rmsnorm_quant_fp8_static.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64,
                                                c_float, c_int, c_void_p]
     L.moe_rmsnorm_quant_mxfp8.restype = c_int
-    L.moe_rmsnorm_quant_mxfp8.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
-                                          c_int64, c_float, c_int64, c_int, c_int, c_void_p]
+    L.moe_rmsnorm_quant_mxfp8.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                          c_void_p, c_int64, c_int64, c_float, c_int64, c_int, c_int, c_void_p]
     L.moe_build_blocks_workspace_bytes.restype = c_size_t
     L.moe_build_blocks_workspace_bytes.argtypes = [c_int64]
     L.moe_build_blocks.restype = c_int

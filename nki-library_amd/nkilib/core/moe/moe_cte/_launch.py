@@ -42,6 +42,9 @@ kmajor_weight_cache = True
 # copy of the gate/up weights in HBM, made on the first call with a weight tensor pair; ``mx_weight_copies =
 # False`` reads the reference layout in place.
 mx_weight_copies = True
+# Measurement hook: an int64 device tensor of 4 elements that the large-tile GEMMs fill with the shader cycles and
+# the 100 MHz ticks of their workgroup 0 (gate/up, then down): cycles / ticks * 0.1 = the clock in GHz under load.
+gemm_clock_probe = None
 _KMAJOR_MAX_ENTRIES = 64
 _kmajor = {}
 
@@ -209,6 +212,10 @@ def run_blockwise(
         ck_down = torch.empty((N, B, H), dtype=torch.bfloat16, device=dev)
         a.down_activations = nv.ptr(ck_down)
 
+    if gemm_clock_probe is not None:
+        kernel_assert(gemm_clock_probe.dtype == torch.int64 and gemm_clock_probe.numel() >= 4 and gemm_clock_probe.is_cuda,
+                      "gemm_clock_probe must be a device int64 tensor of 4 elements")
+        a.gemm_clocks = gemm_clock_probe.data_ptr()
     kmajor = (None, None)
     if (kmajor_weight_cache and kind in (nv.KIND_BF16, nv.KIND_FP8_ROW)) or (mx_weight_copies and kind == nv.KIND_MXFP8):
         # (weight_objects: the caller's own tensor objects where the operator had to make views of them)

@@ -90,7 +90,7 @@ def mx_k_order(H):
     return (q * (H // 4) + tile * 128 + p).reshape(-1)
 
 
-def rmsnorm_mx_quant_ref(inp, gamma, eps=1e-6, hidden_actual=None, do_norm=True):
+def rmsnorm_mx_quant_ref(inp, gamma, eps=1e-6, hidden_actual=None, do_norm=True, residual=None):
     """[T, H] -> dict of the RMSNorm->MXFP8 front end outputs.
 
     Returns
@@ -101,8 +101,15 @@ def rmsnorm_mx_quant_ref(inp, gamma, eps=1e-6, hidden_actual=None, do_norm=True)
 
     The normalised value is rounded to bf16 before quantisation, as in the golden
     (``.astype(out_dtype)`` at test_rmsnorm_mx_quantize_tkg.py:118).
+
+    residual ([T, H], bf16-valued like inp): the golden's residual branch (`:104-109`): ``hidden = inp + residual`` as a
+    sum of two bf16 arrays, i.e. rounded to bf16, replaces inp and is returned as "out_residual" [T, H].
     """
     inp = np.asarray(inp, dtype=np.float32)
+    out_residual = None
+    if residual is not None:
+        inp = to_bf16(inp + np.asarray(residual, dtype=np.float32))
+        out_residual = inp
     T, H = inp.shape
     nt = H // 512
     norm = rms_norm(inp, gamma, eps, hidden_actual) if do_norm else inp
@@ -115,4 +122,7 @@ def rmsnorm_mx_quant_ref(inp, gamma, eps=1e-6, hidden_actual=None, do_norm=True)
     scale = scale.reshape(16, nt, T)
     tok_quant = data.transpose(2, 1, 0, 3).reshape(T, H)
     tok_scale = scale.transpose(2, 1, 0).reshape(T, H // 32)
-    return {"out": out, "out_quant": data, "out_scale": scale, "tok_quant": tok_quant, "tok_scale": tok_scale}
+    res = {"out": out, "out_quant": data, "out_scale": scale, "tok_quant": tok_quant, "tok_scale": tok_scale}
+    if out_residual is not None:
+        res["out_residual"] = out_residual
+    return res

@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported():
     for name in declared:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
     assert set(nv.EXPORTED_SYMBOLS) == set(declared)
-    assert L.moe_abi_version() == 5
+    assert L.moe_abi_version() == 6
     assert b"workspace" in L.moe_error_string(-3)
 
 
@@ -62,8 +62,11 @@ def test_argument_validation_runs_without_a_gpu():
     assert L.moe_blockwise_workspace_bytes(ctypes.byref(a)) == 0
     assert L.moe_blockwise(ctypes.byref(a), None) == -1  # MOE_E_BAD_ARG: null tensors
     assert L.moe_rmsnorm_quant_fp8_row(None, 0, None, 0, None, 1, 8, 1e-6, 0.0, 0, None) == -1
-    assert L.moe_rmsnorm_quant_mxfp8(ctypes.c_void_p(256), 0, None, 0, ctypes.c_void_p(256), ctypes.c_void_p(256), None,
-                                     4, 500, 1e-6, 500, 0, 0, None) == -2  # H % 512
+    assert L.moe_rmsnorm_quant_mxfp8(ctypes.c_void_p(256), 0, None, None, None, 0, ctypes.c_void_p(256),
+                                     ctypes.c_void_p(256), None, 4, 500, 1e-6, 500, 0, 0, None) == -2  # H % 512
+    # a residual without a place for the sum (or the reverse) is refused
+    assert L.moe_rmsnorm_quant_mxfp8(ctypes.c_void_p(256), 0, ctypes.c_void_p(256), None, None, 0, ctypes.c_void_p(256),
+                                     ctypes.c_void_p(256), None, 4, 512, 1e-6, 512, 0, 0, None) == -1
     assert L.moe_rmsnorm_quant_fp8_row(ctypes.c_void_p(256), 0, None, 0, ctypes.c_void_p(256), 4, 32768, 1e-6, 0.0, 0,
                                        None) == -2  # H > 16384
     assert L.moe_build_blocks_workspace_bytes(256) >= 2 * 256 * 4

@@ -159,13 +159,60 @@ def test_zero_row_follows_kernel_rule():
     assert torch.equal(scale.cpu(), torch.full((3, 1), 1e-6, dtype=torch.float32))
 
 
+def _mx_blocks_explained_by_bf16_ties(norm32_k, q, s, g_q, g_s, window=8):
+    """Every MX block (32 consecutive k') in which the kernel's codes or scale byte differ from the oracle's must be
+    explained by a rounding tie: the oracle rounds its fp32 normalised value to bf16 before quantising, and a value
+    within `window` fp32 ulps of a bf16 rounding boundary may legitimately round the other way when the row's sum of
+    squares is accumulated in another order.  The fp8 rounding behind it is exact in both (a bf16 value times a power
+    of two), so nothing else may differ: for each differing block some choice of "other neighbour" for its
+    boundary values must reproduce the kernel's 32 codes and its scale byte exactly.
+
+    norm32_k: the oracle's unrounded fp32 normalised values [T, H] in k' order.  Returns (number of differing blocks,
+    number of differing codes, number of differing scale bytes, unexplained blocks)."""
+    from oracle.mx import quantize_mx
+
+    T, H = norm32_k.shape
+    bits = norm32_k.view(np.uint32)
+    low = (bits & 0xFFFF).astype(np.int64)
+    near = np.abs(low - 0x8000) <= window
+    trunc = bits & np.uint32(0xFFFF0000)
+    up = trunc + np.uint32(0x10000)
+    rne_up = (low > 0x8000) | ((low == 0x8000) & (((bits >> 16) & 1) == 1))
+    b0 = np.where(rne_up, up, trunc).view(np.float32)
+    b1 = np.where(rne_up, trunc, up).view(np.float32)
+    diff_codes = q != g_q
+    diff_scale = s != g_s
+    blk = diff_codes.reshape(T, H // 32, 32).any(axis=2) | diff_scale
+    unexplained = []
+    for t, j in zip(*np.nonzero(blk)):
+        sl = slice(32 * j, 32 * j + 32)
+        cand = np.nonzero(near[t, sl])[0]
+        ok = False
+        if 0 < cand.size <= 8:
+            for mask in range(1, 1 << cand.size):
+                v = b0[t, sl].copy()
+                for bit, idx in enumerate(cand):
+                    if mask >> bit & 1:
+                        v[idx] = b1[t, sl][idx]
+                cq, cs = quantize_mx(v.reshape(8, 4))
+                if np.array_equal(cq.reshape(-1), q[t, sl]) and cs.reshape(-1)[0] == s[t, j]:
+                    ok = True
+                    break
+        if not ok:
+            unexplained.append((int(t), int(j), int(cand.size)))
+    return int(blk.sum()), int(diff_codes.sum()), int(diff_scale.sum()), unexplained
+
+
 @pytest.mark.parametrize("T,H,do_norm", [(4, 512, True), (64, 2048, True), (33, 7168, True), (16, 16384, True),
                                           (40, 1024, False),
                                           # short rows share a workgroup (four of up to 64 MX blocks, two of up to
                                           # 128): row counts that leave the last workgroup partly empty
-                                          (5, 1536, True), (7, 4096, True), (3, 3072, True)])
+                                          (5, 1536, True), (7, 4096, True), (3, 3072, True),
+                                          # BASELINE config 4's row length, a few hundred rows
+                                          (300, 7168, True)])
 def test_mx_front_end(T, H, do_norm):
-    """RMSNorm -> MXFP8 (token-major and the reference's [128, H/512, T] layouts) vs the oracle."""
+    """RMSNorm -> MXFP8 (token-major and the reference's [128, H/512, T] layouts) vs the oracle: bit exact except
+    where a bf16 rounding tie of the normalised value explains the difference, and those are counted."""
     import torch
     from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize, rmsnorm_mx_quantize_tkg
 
@@ -176,24 +223,18 @@ def test_mx_front_end(T, H, do_norm):
     dev = torch.device("cuda:0")
     q, s = rmsnorm_mx_quantize(bf16_tensor(x, dev), bf16_tensor(g, dev) if do_norm else None, do_norm=do_norm)
     q, s = q.cpu().numpy(), s.cpu().numpy()
-    # scale bytes can only differ where the bf16 rounding of the normalised value differs, i.e. where the fp32
-    # sum-of-squares order decided a tie; count them, then compare values through the dequantised result
-    n_s = int((s != ref["tok_scale"]).sum())
-    assert n_s <= max(2, s.size // 2000), f"{n_s} of {s.size} scale bytes differ"
-    from oracle.numerics import e4m3fn_decode
-
-    deq = e4m3fn_decode(q).astype(np.float64) * np.repeat(np.power(2.0, s.astype(np.float64) - 127), 32, axis=1)
-    gdeq = e4m3fn_decode(ref["tok_quant"]).astype(np.float64) * np.repeat(
-        np.power(2.0, ref["tok_scale"].astype(np.float64) - 127), 32, axis=1)
-    mism = q != ref["tok_quant"]
-    frac = mism.mean()
-    assert frac < 2e-3, f"{frac:.2e} of codes differ"
-    # every differing code is at most one fp8 step away (one e4m3 ulp = 2^-3 relative)
-    rel = np.abs(deq - gdeq) / np.maximum(np.abs(gdeq), 1e-30)
-    assert (rel[mism & (gdeq != 0)] <= 0.1251).all()
     if not do_norm:
-        assert not mism.any() and n_s == 0  # pure quantisation has no reduction: bit exact
-    if do_norm and T % 4 == 0:
+        # pure quantisation has no reduction: bit exact
+        assert np.array_equal(q, ref["tok_quant"]) and np.array_equal(s, ref["tok_scale"])
+        return
+    norm32 = np.ascontiguousarray(orn.rms_norm(x, g)[:, orn.mx_k_order(H)], dtype=np.float32)
+    n_blk, n_codes, n_scales, unexplained = _mx_blocks_explained_by_bf16_ties(norm32, q, s, ref["tok_quant"], ref["tok_scale"])
+    print(f"MX front end T={T} H={H}: {n_codes} of {q.size} codes and {n_scales} of {s.size} scale bytes differ, in "
+          f"{n_blk} blocks; unexplained: {len(unexplained)}", flush=True)
+    assert not unexplained, f"blocks (token, block, boundary values) that no rounding tie explains: {unexplained[:8]}"
+    assert n_codes <= max(8, q.size // 20000), f"too many tie flips: {n_codes} of {q.size} codes"
+    assert n_scales <= max(2, s.size // 20000), f"too many scale bytes differ: {n_scales} of {s.size}"
+    if T % 4 == 0:
         nT = H // 512
         out = torch.empty((128, T, H // 128), dtype=torch.bfloat16, device=dev)
         oq = torch.empty((128, nT, T), dtype=torch.int32, device=dev)
@@ -206,5 +247,79 @@ def test_mx_front_end(T, H, do_norm):
         assert np.array_equal(osc.cpu().numpy()[rows].transpose(2, 1, 0).reshape(T, H // 32), s)
         from helpers import from_bf16_tensor
 
-        o = from_bf16_tensor(out)
-        assert np.mean(o != ref["out"]) < 2e-3
+        # the normalised bf16 copy: equal to the oracle's except at the same rounding boundaries
+        o = from_bf16_tensor(out)                       # [128, T, H/128], h = h1*128 + p
+        o_th = o.transpose(1, 2, 0).reshape(T, H)
+        g_th = ref["out"].transpose(1, 2, 0).reshape(T, H)
+        n32 = orn.rms_norm(x, g).astype(np.float32)
+        low = (n32.view(np.uint32) & 0xFFFF).astype(np.int64)
+        bad = o_th != g_th
+        assert (np.abs(low[bad] - 0x8000) <= 8).all(), "a normalised value differs away from a bf16 rounding boundary"
+        assert int(bad.sum()) <= max(8, o.size // 20000), f"{int(bad.sum())} of {o.size} normalised values differ"
+
+
+@pytest.mark.parametrize("T,H,dtype", [(256, 2048, "bf16"), (260, 7168, "bf16"), (8, 16384, "bf16"), (12, 1024, "fp16"),
+                                        (16, 1536, "fp32")])
+def test_mx_front_end_residual(T, H, dtype):
+    """Fused residual add (rmsnorm_mx_quantize_tkg.py:29-40; golden test_rmsnorm_mx_quantize_tkg.py:104-117), on the
+    token-major layout and on the reference's [128, H/512, T] layout: output_residual is the sum rounded to the
+    input type, bit for bit, and codes, scales and the normalised copy are bit-equal to the call without residual
+    on that sum (the two calls run the same kernel arithmetic on the same row)."""
+    import torch
+    from helpers import from_bf16_tensor
+    from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize, rmsnorm_mx_quantize_tkg
+
+    rng = np.random.default_rng(5)
+    dev = torch.device("cuda:0")
+    tdt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[dtype]
+    x = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(tdt).to(dev)
+    r = torch.from_numpy((rng.standard_normal((T, H)) * 3).astype(np.float32)).to(tdt).to(dev)
+    g = torch.from_numpy(rng.random((1, H)).astype(np.float32) + 0.5).to(tdt).to(dev)
+    q, s, new_res = rmsnorm_mx_quantize(x, g, residual=r)
+    want = x + r  # torch rounds the sum to the tensors' type
+    assert new_res.dtype == tdt and torch.equal(new_res, want)
+    q0, s0 = rmsnorm_mx_quantize(want, g)
+    assert torch.equal(q, q0) and torch.equal(s, s0)
+    if dtype == "bf16":
+        # and against the oracle's residual branch, with the front end's tie rule
+        xf, rf, gf = (from_bf16_tensor(t) for t in (x, r, g))
+        ref = orn.rmsnorm_mx_quant_ref(xf, gf, residual=rf)
+        assert np.array_equal(from_bf16_tensor(new_res), ref["out_residual"])
+        norm32 = np.ascontiguousarray(orn.rms_norm(ref["out_residual"], gf)[:, orn.mx_k_order(H)], dtype=np.float32)
+        n_blk, n_codes, n_scales, unexplained = _mx_blocks_explained_by_bf16_ties(
+            norm32, q.cpu().numpy(), s.cpu().numpy(), ref["tok_quant"], ref["tok_scale"])
+        print(f"residual front end T={T} H={H}: {n_codes} codes / {n_scales} scale bytes differ, unexplained {len(unexplained)}")
+        assert not unexplained and n_codes <= max(8, q.numel() // 20000)
+    if T % 4 == 0 and dtype != "fp32":
+        nT = H // 512
+        out = torch.empty((128, T, H // 128), dtype=torch.bfloat16, device=dev)
+        oq = torch.empty((128, nT, T), dtype=torch.int32, device=dev)
+        osc = torch.zeros((128, nT, T), dtype=torch.uint8, device=dev)
+        ores = torch.empty((T, H), dtype=tdt, device=dev)
+        res = rmsnorm_mx_quantize_tkg(x.reshape(1, T, H), g, out, oq, osc, residual=r.reshape(1, T, H), output_residual=ores)
+        assert len(res) == 4 and res[3] is ores and torch.equal(ores, want)
+        out0, oq0, osc0 = torch.empty_like(out), torch.empty_like(oq), torch.zeros_like(osc)
+        rmsnorm_mx_quantize_tkg(want.reshape(1, T, H), g, out0, oq0, osc0)
+        assert torch.equal(oq, oq0) and torch.equal(osc, osc0) and torch.equal(out, out0)
+        oq_b = oq.cpu().numpy().view(np.uint8).reshape(128, nT, T, 4)
+        assert np.array_equal(oq_b.transpose(2, 1, 0, 3).reshape(T, H), q.cpu().numpy())
+
+
+def test_mx_front_end_residual_argument_rules():
+    """The reference's argument rules for the residual pair (norm_tkg_utils.py:467,473-476)."""
+    import torch
+    from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize_tkg
+
+    dev = torch.device("cuda:0")
+    T, H = 4, 512
+    x = torch.zeros((1, T, H), dtype=torch.bfloat16, device=dev)
+    g = torch.ones((1, H), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((128, T, H // 128), dtype=torch.bfloat16, device=dev)
+    oq = torch.empty((128, 1, T), dtype=torch.int32, device=dev)
+    osc = torch.zeros((128, 1, T), dtype=torch.uint8, device=dev)
+    with pytest.raises(AssertionError, match="output_residual required"):
+        rmsnorm_mx_quantize_tkg(x, g, out, oq, osc, residual=x)
+    with pytest.raises(AssertionError, match="shapes must match"):
+        rmsnorm_mx_quantize_tkg(x, g, out, oq, osc, residual=x[:, :2], output_residual=torch.empty((T, H), dtype=torch.bfloat16, device=dev))
+    with pytest.raises(AssertionError, match="Only hidden_dim_tp=True is supported"):
+        rmsnorm_mx_quantize_tkg(x, g, out, oq, osc, hidden_dim_tp=False)

@@ -261,6 +261,28 @@ def test_mx_front_end_is_norm_then_online_quantisation():
     assert np.mean(bf16_bits(n64.astype(np.float32)) != bf16_bits(normed)) < 5e-3
 
 
+def test_mx_front_end_residual_branch_closed_forms():
+    """The residual branch of the RMSNorm -> MXFP8 golden (test_rmsnorm_mx_quantize_tkg.py:104-117): the new residual
+    stream is bf16(x + r) -- checked against torch's bf16 addition, an independent routine -- and everything behind
+    it equals the plain front end applied to that sum.  A branch that normalised x alone, or that kept the sum
+    unrounded, fails one of the two."""
+    import torch
+
+    rng = np.random.default_rng(12)
+    T, H = 12, 1024
+    x = to_bf16(rng.standard_normal((T, H)).astype(np.float32))
+    r = to_bf16((rng.standard_normal((T, H)) * 3).astype(np.float32))
+    g = to_bf16(rng.random((1, H)).astype(np.float32) + 0.5)
+    got = orn.rmsnorm_mx_quant_ref(x, g, residual=r)
+    tsum = (torch.from_numpy(x).to(torch.bfloat16) + torch.from_numpy(r).to(torch.bfloat16)).float().numpy()
+    assert np.array_equal(bf16_bits(got["out_residual"]), bf16_bits(tsum))
+    assert (got["out_residual"] != (x + r)).any(), "the case must need the rounding"
+    plain = orn.rmsnorm_mx_quant_ref(tsum, g)
+    for k in ("out", "out_quant", "out_scale", "tok_quant", "tok_scale"):
+        assert np.array_equal(got[k], plain[k]), k
+    assert not np.array_equal(got["tok_quant"], orn.rmsnorm_mx_quant_ref(x, g)["tok_quant"])
+
+
 def test_committed_fixtures():
     fx = np.load(os.path.join(GOLDEN, "small_cases.npz"))
     c = mx_case(128, 512, 512, 4, 2, 128, seed=21)
