@@ -81,6 +81,8 @@ struct MxArgs {
                            // of constants for every row)
   float* Y32;              // stage 1 output of this format: fp32 [N*B, y32_stride], columns in natural order
   int64_t y32_stride;
+  uint16_t* ckpt;          // MX_WFMT_BF16, nullable: stage 1 gate/up checkpoint [N, 2, I, B], stage 2 down checkpoint [N, B, H]
+  int64_t ckpt_B, ckpt_I;  // block size and intermediate size of the checkpoint layout (elements)
   int64_t* clk;            // nullable: workgroup 0 stores its shader cycles and 100 MHz ticks from start to end here
   // MX_WFMT_BF16 (the bf16 kind on these kernels): both operands bf16, read as bytes exactly like the 8-bit formats
   // (a 128-byte K slice is 64 elements, multiplied by two v_mfma_f32_16x16x32_bf16 where the 8-bit formats issue

@@ -508,9 +508,8 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   constexpr int NAJ = NMT / 2;  // 32-row groups that hold rows of the NMT tiles
   // Per-lane 32-bit byte offsets (row * stride + chunk); the K offset is wave-uniform and is added
   // to the scalar base, so a load needs one VGPR of address.  Rows without a token (padding
-  // slots, rows past the end of the chunk) read some valid row instead of being zeroed: rows are
-  // independent in a GEMM and the results of such rows are never written out, so what they hold
-  // does not matter -- and the loads stay free of branches.
+  // slots, rows past the end of the chunk) point past the end of the buffer and load as zero rows,
+  // without a branch (see aim_loads_at).
   // (down stage: the rows are consecutive slots, so one per-lane offset serves all row groups and the group goes
   // into the scalar offset; rows past the chunk's end may then lie past the end of the buffer, where the range
   // check of the descriptor returns zeros)
@@ -592,7 +591,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     RawLoad d[NBL];
     int sc;
   };
-  v4i ra_ = make_rsrc(a.A, (STAGE == 1) ? 0xffffffffu : (uint32_t)(a.a_rows * a.a_stride)),
+  v4i ra_ = make_rsrc(a.A, (uint32_t)(a.a_rows * a.a_stride)),
       ras_ = make_rsrc(a.A_scale, (uint32_t)(a.a_scale_bytes ? a.a_scale_bytes : a.a_rows * a.a_scale_stride));
   const int ra_rec = ra_[2], ras_rec = ras_[2];
   int rw_rec = 0, rs_rec = 0;
@@ -610,8 +609,11 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       const int row = arow0 + 32 * j;
       uint32_t r;
       if (STAGE == 1) {
+        // a row without a token (padding slot, row past the end of the chunk) points past the end of the buffer:
+        // the range check of the descriptor turns such a load into zeros without any traffic, so the row is a zero
+        // row (what the activation checkpoints must show for it) and its MFMAs multiply zeros
         const int tok = s_tok[buf][row];
-        r = (tok >= 0) ? (uint32_t)tok : 0u;
+        r = (tok >= 0) ? (uint32_t)tok : (uint32_t)a.a_rows;
       } else {
         r = (uint32_t)(t.slot0 + row);
       }
@@ -992,6 +994,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
             else av[i / 4][i % 4] = accv[mt - 16][i / 4][i % 4];
           });
           float y[2][4];
+          float ckg[4][2], cku[4][2];  // bf16 kind: gate / up ahead of the activation, for the checkpoint
           float rsk[2] = {1.f, 1.f};  // fp8-row kind: the scales of the lane's two rows
           if constexpr (ROW8) {
             const float2 rr = *(const float2*)(s_rs[buf] + ps * 64 + ml * 16 + 4 * g_e + 2 * hcol_e);
@@ -1014,6 +1017,40 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
               const float gg = fminf(fmaxf(gv + bg[t], g_lo), g_hi);
               const float uu = fminf(fmaxf(uv + bu[t], u_lo), u_hi);
               y[k][t] = act_apply(gg, ACT) * uu;
+              if constexpr (BF16) {
+                ckg[t][k] = gg;
+                cku[t][k] = uu;
+              }
+            }
+          }
+          if constexpr (BF16) {
+            // activation checkpoint [N, 2, I, B] (bwmm_shard_on_I.py:160-176): gate / up projections after scale, bias
+            // and clamp, transposed: the lane's two rows are neighbours along B
+            const int row = ps * 64 + ml * 16 + 4 * g_e + 2 * hcol_e;
+            if (a.ckpt != nullptr && row < cur.nrows) {
+              const uint32_t slot = (uint32_t)(cur.slot0 + row);
+              const uint32_t n = slot / (uint32_t)a.ckpt_B, r = slot - n * (uint32_t)a.ckpt_B;
+              const int64_t col = (int64_t)tile_tI(cur) * 512 + (int64_t)q * tile_Pt(cur) + tile_p0(cur) + pl0;
+              uint16_t* ck = a.ckpt + (((int64_t)n * 2) * a.ckpt_I + col) * a.ckpt_B + r;
+              // (an even block size keeps the pair inside one block and the store aligned; otherwise row by row)
+              const bool pair = (a.ckpt_B & 1) == 0;
+              const uint32_t slot1 = slot + 1, n1 = slot1 / (uint32_t)a.ckpt_B, r1 = slot1 - n1 * (uint32_t)a.ckpt_B;
+              uint16_t* ck1 = a.ckpt + (((int64_t)n1 * 2) * a.ckpt_I + col) * a.ckpt_B + r1;
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                const uint32_t gp = pack2_bf16(ckg[t][0], ckg[t][1]), up = pack2_bf16(cku[t][0], cku[t][1]);
+                if (pair) {
+                  *(uint32_t*)(ck + (int64_t)t * a.ckpt_B) = gp;
+                  *(uint32_t*)(ck + ((int64_t)a.ckpt_I + t) * a.ckpt_B) = up;
+                } else {
+                  ck[(int64_t)t * a.ckpt_B] = (uint16_t)gp;
+                  ck[((int64_t)a.ckpt_I + t) * a.ckpt_B] = (uint16_t)up;
+                  if (row + 1 < cur.nrows) {
+                    ck1[(int64_t)t * a.ckpt_B] = (uint16_t)(gp >> 16);
+                    ck1[((int64_t)a.ckpt_I + t) * a.ckpt_B] = (uint16_t)(up >> 16);
+                  }
+                }
+              }
             }
           }
 #pragma unroll
@@ -1109,6 +1146,10 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     // are dropped by the range check and the stores need no branches.  (Rows of padding slots
     // inside the chunk are written too: nothing reads the contributions of such slots.)
     const v4i rd = make_rsrc(a.D + (int64_t)cur.slot0 * a.H, (uint32_t)((int64_t)cur.nrows * a.H * 2));
+    // bf16 kind: the down checkpoint [N, B, H] = [slots, H] (bwmm_shard_on_I.py:160-176) takes the same rows ahead of
+    // the affinity (a descriptor of zero records when there is none: the stores then go nowhere)
+    const v4i rdc = make_rsrc((BF16 && a.ckpt) ? a.ckpt + (int64_t)cur.slot0 * a.H : a.D,
+                              (BF16 && a.ckpt) ? (uint32_t)((int64_t)cur.nrows * a.H * 2) : 0u);
     const uint32_t d_voff = (uint32_t)((4 * g_e * a.H + col0) * 2);
     const int rowb = uni(a.H * 2);
     typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
@@ -1143,6 +1184,15 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
           for (int t = 0; t < 4; ++t) av[t][r] = (av[t][r] * sd[t]) * rs;
         }
         v2i o;
+        if constexpr (BF16) {
+          v2i oc;
+#pragma unroll
+          for (int t = 0; t < 4; t += 2) {
+            const v2f d = {av[t][r] + bd[t], av[t + 1][r] + bd[t + 1]};
+            oc[t >> 1] = __builtin_bit_cast(int, __builtin_convertvector(d, v2bf));
+          }
+          st_b64(oc, d_voff, rdc, (mt * 16 + r) * rowb);
+        }
 #pragma unroll
         for (int t = 0; t < 4; t += 2) {
           const v2f d = {(av[t][r] + bd[t]) * af, (av[t + 1][r] + bd[t + 1]) * af};

@@ -127,9 +127,9 @@ int validate(const moe_bwmm_args* a) {
 //                holds (x4 read order, or K-contiguous rows for the general kernel): a copy prepared in one call must
 //                mean the same in every other call with the same weights, whatever its token count.
 //   *_call_fits: do this call's activations (token count, number of blocks) fit the kernels' 32-bit row offsets?
-// A call runs there when both hold (and, for bf16, it asks for no activation checkpoints, which those epilogues do not
-// write).  A call on such a shape that cannot run there uses the general kernel on K-contiguous copies of its own,
-// made per call in the workspace: kept copies are in the other order and are ignored (*_kept_usable).
+// A call runs there when both hold (activation checkpoints of the bf16 kind included: those epilogues write them).
+// A call on such a shape that cannot run there uses the general kernel on K-contiguous copies of its own, made per
+// call in the workspace: kept copies are in the other order and are ignored (*_kept_usable).
 bool row8_shape(const moe_bwmm_args* a) {
   if (a->kind != MOE_KIND_FP8_ROW || !mx_fast_path_ok(a->H, a->I)) return false;
   const int64_t lim32 = (int64_t)1 << 32, lim31 = (int64_t)1 << 31;
@@ -161,9 +161,7 @@ bool bf16_call_fits(const moe_bwmm_args* a) {
   const int64_t slots = a->N * a->B;
   return a->T1 * 2 * a->H < lim32 && slots * 2 * a->I < lim32 && slots * 4 < lim32 && a->T1 * a->E * 4 < lim32;
 }
-bool bf16_fast(const moe_bwmm_args* a) {
-  return bf16_fast_shape(a) && bf16_call_fits(a) && !a->gate_up_activations_T && !a->down_activations;
-}
+bool bf16_fast(const moe_bwmm_args* a) { return bf16_fast_shape(a) && bf16_call_fits(a); }
 bool bf16_kept_usable(const moe_bwmm_args* a) { return bf16_fast(a) || !bf16_fast_shape(a); }
 // What a kept copy of the fp8-row (bf16) weights holds on that path: the weights in x4 order, one expert's worth of
 // E8M0 block scales of 127 (2^0) that serves every expert, and one row of activation block scales of 127 (the bf16
@@ -506,7 +504,11 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
         m1.A_scale = g1.W + c.a_scale; m1.a_scale_stride = 0; m1.a_scale_bytes = (int64_t)c.a_scale_bytes;
         m1.w_cscale = (const float*)a->gate_up_proj_scale;
       }
-      if (bf_fast) m1.H = 2 * a->H;  // K in bytes
+      if (bf_fast) {
+        m1.H = 2 * a->H;  // K in bytes
+        m1.ckpt = (uint16_t*)a->gate_up_activations_T;
+        m1.ckpt_B = a->B; m1.ckpt_I = a->I;
+      }
       m1.clk = a->gemm_clocks;
 
       // column tiles of 32 partitions x 4 q, gate and up: 4 per full intermediate tile + those of a short last one
@@ -543,6 +545,8 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
         m2.A = ws + p.y; m2.a_stride = p.Iw * 2;
         m2.I = 2 * a->I;  // K in bytes
         m2.a_rscale = nullptr;
+        m2.ckpt = (uint16_t*)a->down_activations;
+        m2.ckpt_B = a->B; m2.ckpt_I = a->I;
       }
       m2.clk = a->gemm_clocks ? a->gemm_clocks + 2 : nullptr;
 

@@ -63,7 +63,8 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
                                              int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
                                              int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
                                              int32_t* __restrict__ chunk_xcd, int32_t* __restrict__ q_chunk,
-                                             int32_t* __restrict__ q_off, int64_t max_chunks, int* s_ws) {
+                                             int32_t* __restrict__ q_off, int64_t max_chunks, int* s_ws,
+                                             bool whole_blocks) {
   const int64_t na = *n_active;
   // The walk along a run below is a chain of dependent reads, one block after the other: from LDS when the active
   // blocks fit there (a global read per step made the run length the pace of this kernel).
@@ -94,8 +95,10 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
       e = expert_of(b);
       const bool start = (b == 0) || (expert_of(b - 1) != e);
       if (start && e >= 0 && e < E) {
+        // (whole_blocks: activation checkpoints hold every row of every executed block, padding rows included, so
+        // a run's chunks then cover its blocks to the end)
         for (int64_t j = b; j < na && expert_of(j) == e; ++j) {
-          const int v = valid_of(j);
+          const int v = whole_blocks ? (int)B : valid_of(j);
           if (v > 0) last_end = j * B + v;
         }
         // chunks of CHUNK_ROWS rows; the last one absorbs a remainder of up to CHUNK_ROWS_MAX - CHUNK_ROWS
@@ -259,11 +262,11 @@ __global__ __launch_bounds__(1024) void chunks_and_offsets_kernel(
     int64_t N, int64_t B, int64_t E, int32_t* __restrict__ n_chunks, int32_t* __restrict__ chunk_slot,
     int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert, int32_t* __restrict__ chunk_xcd,
     int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off, int64_t max_chunks,
-    const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n_real) {
+    const int32_t* __restrict__ cnt, int32_t* __restrict__ off, int64_t n_real, bool whole_blocks) {
   __shared__ int s_ws[16];
   if (blockIdx.x == 0)
     build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, chunk_xcd, q_chunk,
-                 q_off, max_chunks, s_ws);
+                 q_off, max_chunks, s_ws, whole_blocks);
   else
     inv_scan(cnt, off, n_real, s_ws);
 }
@@ -279,7 +282,7 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
     int32_t* __restrict__ valid_rows, int32_t* __restrict__ cnt, int64_t clear_words, int32_t* __restrict__ n_chunks,
     int32_t* __restrict__ chunk_slot, int32_t* __restrict__ chunk_rows, int32_t* __restrict__ chunk_expert,
     int32_t* __restrict__ chunk_xcd, int32_t* __restrict__ q_chunk, int32_t* __restrict__ q_off, int64_t max_chunks,
-    int32_t* __restrict__ off, int32_t* __restrict__ cursor, int32_t* __restrict__ list) {
+    int32_t* __restrict__ off, int32_t* __restrict__ cursor, int32_t* __restrict__ list, bool whole_blocks) {
   __shared__ int s_ws[16];
   __shared__ int s_first_zero;
   for (int64_t i = threadIdx.x; i < clear_words; i += blockDim.x) cnt[i] = 0;  // cnt and cursor are adjacent
@@ -315,18 +318,21 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
   __threadfence_block();
   __syncthreads();
   build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, chunk_xcd, q_chunk,
-               q_off, max_chunks, s_ws);
+               q_off, max_chunks, s_ws, whole_blocks);
   __syncthreads();
   inv_scan(cnt, off, n_real, s_ws);
   __threadfence_block();
   __syncthreads();
-  for (int64_t s = threadIdx.x; s < N * B; s += blockDim.x) {
-    const int64_t b = s / B, r = s % B;
-    if (r >= valid_rows[b]) continue;
-    const int id = tp2id[s];
-    if (id >= 0 && id < n_real) {
-      const int p = atomicAdd(&cursor[id], 1);
-      list[off[id] + p] = (int32_t)s;
+  // (a wave per block again, over the block's valid rows only: decode-sized problems are mostly padding)
+  for (int64_t b = wave; b < N; b += nwaves) {
+    const int vr = valid_rows[b];
+    for (int64_t r = lane; r < vr; r += 64) {
+      const int64_t s = b * B + r;
+      const int id = tp2id[s];
+      if (id >= 0 && id < n_real) {
+        const int p = atomicAdd(&cursor[id], 1);
+        list[off[id] + p] = (int32_t)s;
+      }
     }
   }
 }
@@ -447,6 +453,7 @@ Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B) {
 constexpr int64_t PREP_SMALL_SLOTS = 40960, PREP_SMALL_TOKENS = 4096;
 
 int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hipStream_t s) {
+  const bool whole_blocks = a->gate_up_activations_T != nullptr || a->down_activations != nullptr;
   // cnt and cursor are adjacent: one clear covers both.  A fill kernel rather than a memset
   // node, so that the sequence stays safe to record into a HIP graph.
   const int64_t clear_words = (int64_t)((uint8_t*)k.off - (uint8_t*)k.cnt) / 4;
@@ -454,7 +461,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
     hipLaunchKernelGGL(prep_small_kernel, dim3(1), dim3(1024), 0, s, a->token_position_to_id, a->block_to_expert,
                        a->conditions, a->n_conditions, a->N, a->B, a->E, n_real, k.n_active, k.valid_rows, k.cnt,
                        clear_words, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.chunk_xcd, k.q_chunk,
-                       k.q_off, k.max_chunks, k.off, k.cursor, k.list);
+                       k.q_off, k.max_chunks, k.off, k.cursor, k.list, whole_blocks);
     MOE_CHECK_LAUNCH();
     return MOE_OK;
   }
@@ -467,7 +474,7 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(chunks_and_offsets_kernel, dim3(2), dim3(1024), 0, s, a->block_to_expert, k.n_active, k.valid_rows,
                      a->N, a->B, a->E, k.n_chunks, k.chunk_slot, k.chunk_rows, k.chunk_expert, k.chunk_xcd, k.q_chunk, k.q_off,
-                     k.max_chunks, k.cnt, k.off, n_real);
+                     k.max_chunks, k.cnt, k.off, n_real, whole_blocks);
   MOE_CHECK_LAUNCH();
   const int64_t slots = a->N * a->B;
   const unsigned gs = (unsigned)((slots + 255) / 256);
