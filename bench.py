@@ -70,6 +70,10 @@ def parse_args():
     ap.add_argument("--sustain-seconds", type=float, default=2.0,
                     help="after the timed steps keep running the same step for at least this long and report its pace "
                          "and the shader clock the GEMMs held (extra keys; 0 skips it)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also record the step into a HIP graph and time its replays (extra key graph_ms_per_step; on by "
+                         "default for the decode-sized workloads c5-<T>, where the eager step is bound by the host's "
+                         "launch path and not by the GPU)")
     ap.add_argument("--cpu-blocks", type=int, default=48, help="blocks of the workload timed on the CPU oracle (48: 10-20 s)")
     ap.add_argument("--with-router", action="store_true",
                     help="start from hidden states: time the router top-k front end (synthetic router weights) as a "
@@ -406,6 +410,33 @@ def main():
                      "ghz_gate_up": (c[0] / c[1] * 0.1) if c[1] else None,
                      "ghz_down": (c[2] / c[3] * 0.1) if c[3] else None}
 
+    # The step recorded once into a HIP graph and replayed: what a decode loop would run.  The library allocates
+    # nothing on the device during a step (workspace and kept weight copies exist after the warm-up), so the recorded
+    # launches are the eager ones; the result of every replay is compared with the eager result.
+    graph_ms = None
+    if (args.graph or args.workload.startswith("c5")) and not args.with_router:
+        ref = out.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(False)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g_out = step(False)[0]
+        for _ in range(max(args.warmup, 1)):
+            graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_out, ref), "a graph replay differs from the eager step"
+        t2 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t2) * 1e3 / args.steps
+        assert torch.equal(g_out, ref), "a graph replay differs from the eager step"
+        del graph
+
     routed = int((tp2id.reshape(-1) < T).sum().item())  # == T*k
     flops_layer = 6.0 * routed * H * I
     flops_gate_up = 4.0 * routed * H * I
@@ -482,6 +513,9 @@ def main():
         },
         "roofline": roofline,
     }
+    if graph_ms is not None:
+        res["graph_ms_per_step"] = round(graph_ms, 4)
+        res["graph_TFLOPs"] = round(flops_layer / (graph_ms * 1e-3) / 1e12, 2)
     if sustained:
         res["sustained_ms_per_step"] = round(sustained["ms_per_step"], 4)
         res["sustained_steps"] = sustained["steps"]

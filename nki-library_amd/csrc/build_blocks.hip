@@ -57,6 +57,17 @@ __device__ __forceinline__ int bb_bits(const uint32_t* bm, int64_t E, int64_t e)
   return n;
 }
 
+// This workgroup's share of the pad ids: 16 bytes per store where the table allows it.
+__device__ __forceinline__ void bb_fill_pad(int32_t* __restrict__ tp2id, int64_t NB, int pad_id, int64_t slab,
+                                            int64_t n_wg) {
+  if ((NB & 3) == 0 && ((uintptr_t)tp2id & 15) == 0) {
+    const int4 v = make_int4(pad_id, pad_id, pad_id, pad_id);
+    for (int64_t i = slab * BB_THREADS + threadIdx.x; i < NB / 4; i += n_wg * BB_THREADS) ((int4*)tp2id)[i] = v;
+  } else {
+    for (int64_t i = slab * BB_THREADS + threadIdx.x; i < NB; i += n_wg * BB_THREADS) tp2id[i] = pad_id;
+  }
+}
+
 // Workgroup = slab of slab_tokens tokens (a multiple of 256).  slab_counts[slab][e] = tokens of the slab that
 // selected e.  All workgroups together also fill token_position_to_id with the pad id, which the scatter
 // overwrites where tokens sit.
@@ -80,7 +91,7 @@ __device__ __forceinline__ void bb_count_body(const int32_t* __restrict__ ids, i
     __syncthreads();
   }
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) slab_counts[slab * E + e] = run[e];
-  for (int64_t i = slab * BB_THREADS + threadIdx.x; i < NB; i += n_wg * BB_THREADS) tp2id[i] = pad_id;
+  bb_fill_pad(tp2id, NB, pad_id, slab, n_wg);
 }
 
 __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __restrict__ ids, int64_t T, int64_t k,
@@ -140,10 +151,18 @@ __device__ __forceinline__ void bb_layout_body(const int32_t* __restrict__ slab_
     carry += total;
   }
   __syncthreads();
-  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
-    const int64_t blk = s_first[e];
-    first_slot[e] = (int32_t)(blk * B);
-    for (int64_t j = 0; j < s_nb[e] && blk + j < N; ++j) block_to_expert[blk + j] = (int32_t)e;
+  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) first_slot[e] = (int32_t)((int64_t)s_first[e] * B);
+  // A block's expert is the last one whose first block is not beyond it (experts without blocks share their first
+  // block with the next expert, so the last of equals is the one that owns the block).  A search per block: the
+  // padding blocks of a small batch all belong to one expert, and a loop per expert would write them one by one.
+  for (int64_t b = threadIdx.x; b < N; b += BB_THREADS) {
+    int lo = 0, hi = (int)E;  // s_first[lo] <= b < s_first[hi]  (s_first[0] == 0, s_first[E] = infinity)
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_first[mid] <= b) lo = mid;
+      else hi = mid;
+    }
+    block_to_expert[b] = lo;
   }
   if (conditions) {
     // ones, then zeros over the trailing (npad + n_conditions - N) entries

@@ -195,14 +195,21 @@ __device__ __forceinline__ void build_chunks(const int32_t* __restrict__ b2e, co
     atomicAdd(&s_cnt[key], 1);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int k = 0; k < 8 * CHUNK_CLASSES; ++k) {
-      const int c = s_cnt[k];
+  {
+    // exclusive scan of the (XCD, class) counts: the queues' first items (a thread per count; one thread walking
+    // all of them took longer than the rest of a decode-sized call)
+    static_assert(8 * CHUNK_CLASSES <= 256, "a thread per queue");
+    // queue entries and the LDS chunk list pack (expert << 16 | rows) into one non-negative int
+    static_assert(CHUNK_ROWS_MAX < (1 << 16) && COMBINE_MAX_K <= (1 << 15), "rows | expert << 16 fits an int32");
+    const int k = threadIdx.x;
+    const bool mine = k < 8 * CHUNK_CLASSES;
+    const int c = mine ? s_cnt[k] : 0;
+    int total;
+    const int run = block_excl_scan(c, s_ws, &total);
+    if (mine) {
       s_cnt[k] = run;
       q_off[(k / CHUNK_CLASSES) * (CHUNK_CLASSES + 1) + k % CHUNK_CLASSES] = run;
-      run += c;
-      if (k % CHUNK_CLASSES == CHUNK_CLASSES - 1) q_off[(k / CHUNK_CLASSES) * (CHUNK_CLASSES + 1) + CHUNK_CLASSES] = run;
+      if (k % CHUNK_CLASSES == CHUNK_CLASSES - 1) q_off[(k / CHUNK_CLASSES) * (CHUNK_CLASSES + 1) + CHUNK_CLASSES] = run + c;
     }
   }
   __syncthreads();
@@ -299,10 +306,12 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
   if (threadIdx.x == 0) *n_active = na;
   // a wave per block: valid rows = 1 + last row with a real token; slots per token
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-  for (int64_t b = wave; b < N; b += nwaves) {
+  // (blocks from the first zero condition on hold nothing: a decode-sized batch is mostly such blocks)
+  for (int64_t b = na + threadIdx.x; b < N; b += blockDim.x) valid_rows[b] = 0;
+  for (int64_t b = wave; b < na; b += nwaves) {
     int v = 0;
     const int e = b2e[b];
-    if (b < na && e >= 0 && e < E) {
+    if (e >= 0 && e < E) {
       for (int64_t r = lane; r < B; r += 64) {
         const int id = tp2id[b * B + r];
         if (id >= 0 && id < n_real) {
@@ -324,7 +333,7 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
   __threadfence_block();
   __syncthreads();
   // (a wave per block again, over the block's valid rows only: decode-sized problems are mostly padding)
-  for (int64_t b = wave; b < N; b += nwaves) {
+  for (int64_t b = wave; b < na; b += nwaves) {
     const int vr = valid_rows[b];
     for (int64_t r = lane; r < vr; r += 64) {
       const int64_t s = b * B + r;
@@ -352,7 +361,8 @@ __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict
   }
 }
 
-// One workgroup per output row.  D: bf16 [N*B, H] contributions.
+// One workgroup per output row (a few, side by side along the row, when the rows are too few to fill the GPU:
+// gridDim.y).  D: bf16 [N*B, H] contributions.
 __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict__ D, const int32_t* __restrict__ off,
                                                       const int32_t* __restrict__ list, uint16_t* __restrict__ out,
                                                       uint16_t* __restrict__ out_shard1, int64_t out_row_stride,
@@ -377,8 +387,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
   uint16_t* zrow = out_shard1 ? out_shard1 + t * out_row_stride : nullptr;  // the other shard's row: zeros
   const bool vec = (H % 8 == 0) && ((out_row_stride % 8) == 0) && (((uintptr_t)out & 15) == 0) &&
                    (((uintptr_t)out_shard1 & 15) == 0);
+  const int64_t vt = (int64_t)blockIdx.y * blockDim.x + threadIdx.x, vstride = (int64_t)gridDim.y * blockDim.x;
   if (vec) {
-    for (int64_t c = (int64_t)threadIdx.x * 8; c < H; c += (int64_t)blockDim.x * 8) {
+    for (int64_t c = vt * 8; c < H; c += vstride * 8) {
       float acc[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) acc[k] = 0.f;
@@ -409,7 +420,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
       if (zrow) *(uint4*)(zrow + c) = make_uint4(0, 0, 0, 0);
     }
   } else {
-    for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
+    for (int64_t c = vt; c < H; c += vstride) {
       float acc = 0.f;
       for (int j = 0; j < cnt; ++j) acc = round_to_bf16(acc + bf16_bits_to_f32(D[(int64_t)s_sorted[j] * H + c]));
       orow[c] = f32_to_bf16_bits(acc);
@@ -485,7 +496,15 @@ int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hi
 }
 
 int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, int64_t n_real, hipStream_t s) {
-  hipLaunchKernelGGL(combine_kernel, dim3((unsigned)a->T1), dim3(256), 0, s, (const uint16_t*)D, k.off, k.list,
+  // few rows (decode): up to 8 workgroups share a row, 8 columns per thread each
+  unsigned split = 1;
+  if (a->T1 <= 256) {
+    const int64_t per_wg = 256 * 8;
+    split = (unsigned)((a->H + per_wg - 1) / per_wg);
+    if (split > 8) split = 8;
+    if (split < 1) split = 1;
+  }
+  hipLaunchKernelGGL(combine_kernel, dim3((unsigned)a->T1, split), dim3(256), 0, s, (const uint16_t*)D, k.off, k.list,
                      (uint16_t*)a->output, (uint16_t*)a->output_shard1, a->out_row_stride, a->H, n_real);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
