@@ -501,6 +501,8 @@ def main():
                                f"gate/up + down + combine",
                    "T": T, "H": H, "I": I, "E": E, "top_k": k, "block_size": B},
         "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
+        "experts_hit": e_hit,
+        "expert_weight_bytes": int(weight_bytes),
         "gemm_phase_TFLOPs": round(flops_layer / ((stage_ms["gate_up"] + stage_ms["down"]) * 1e-3) / 1e12, 2),
         "pct_of_fp8_mfma_peak": round(100.0 * tflops / PEAK_FP8_TFLOPS, 2),
         "stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
