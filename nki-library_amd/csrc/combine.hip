@@ -293,6 +293,7 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
   __shared__ int s_ws[16];
   __shared__ int s_first_zero;
   for (int64_t i = threadIdx.x; i < clear_words; i += blockDim.x) cnt[i] = 0;  // cnt and cursor are adjacent
+  for (int64_t b = threadIdx.x; b < N; b += blockDim.x) valid_rows[b] = 0;
   if (threadIdx.x == 0) s_first_zero = (int)N;
   __threadfence_block();
   __syncthreads();
@@ -304,26 +305,47 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
   __syncthreads();
   const int na = s_first_zero;
   if (threadIdx.x == 0) *n_active = na;
-  // a wave per block: valid rows = 1 + last row with a real token; slots per token
+  // A wave per active block, four blocks at a time so that a wave has their loads in flight together (blocks from
+  // the first zero condition on hold nothing: a decode-sized batch is mostly such blocks, and their valid rows
+  // were cleared above).  body(u, slot, row, id) runs for every slot that holds a token in a block with a valid
+  // expert; after(u, block) once per block.
+  constexpr int U = 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-  // (blocks from the first zero condition on hold nothing: a decode-sized batch is mostly such blocks)
-  for (int64_t b = na + threadIdx.x; b < N; b += blockDim.x) valid_rows[b] = 0;
-  for (int64_t b = wave; b < na; b += nwaves) {
-    int v = 0;
-    const int e = b2e[b];
-    if (e >= 0 && e < E) {
-      for (int64_t r = lane; r < B; r += 64) {
-        const int id = tp2id[b * B + r];
-        if (id >= 0 && id < n_real) {
-          v = (int)r + 1;
-          atomicAdd(&cnt[id], 1);
-        }
-      }
-    }
+  const int iB = (int)B;
+  auto over_blocks = [&](auto&& body, auto&& after) {
+    for (int b0 = wave * U; b0 < na; b0 += nwaves * U) {
+      int e[U];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
-    if (lane == 0) valid_rows[b] = v;
-  }
+      for (int u = 0; u < U; ++u) e[u] = (b0 + u < na) ? b2e[b0 + u] : -1;
+      for (int r0 = 0; r0 < iB; r0 += 64) {
+        const int r = r0 + lane;
+        int id[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) id[u] = (b0 + u < na && r < iB) ? tp2id[(b0 + u) * iB + r] : -1;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (e[u] >= 0 && e[u] < E && id[u] >= 0 && id[u] < n_real) body(u, (b0 + u) * iB + r, r, id[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (b0 + u < na) after(u, b0 + u);
+    }
+  };
+  int v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) v[u] = 0;
+  over_blocks(
+      [&](int u, int, int r, int id) {
+        v[u] = r + 1;  // rows ascend: the last one stays
+        atomicAdd(&cnt[id], 1);
+      },
+      [&](int u, int b) {
+        int m = v[u];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) m = max(m, __shfl_xor(m, o, 64));
+        if (lane == 0) valid_rows[b] = m;  // valid rows = 1 + last row with a real token
+        v[u] = 0;
+      });
   __threadfence_block();
   __syncthreads();
   build_chunks(b2e, n_active, valid_rows, N, B, E, n_chunks, chunk_slot, chunk_rows, chunk_expert, chunk_xcd, q_chunk,
@@ -332,18 +354,12 @@ __global__ __launch_bounds__(1024) void prep_small_kernel(
   inv_scan(cnt, off, n_real, s_ws);
   __threadfence_block();
   __syncthreads();
-  // (a wave per block again, over the block's valid rows only: decode-sized problems are mostly padding)
-  for (int64_t b = wave; b < na; b += nwaves) {
-    const int vr = valid_rows[b];
-    for (int64_t r = lane; r < vr; r += 64) {
-      const int64_t s = b * B + r;
-      const int id = tp2id[s];
-      if (id >= 0 && id < n_real) {
+  over_blocks(
+      [&](int, int sl, int, int id) {
         const int p = atomicAdd(&cursor[id], 1);
-        list[off[id] + p] = (int32_t)s;
-      }
-    }
-  }
+        list[off[id] + p] = sl;
+      },
+      [&](int, int) {});
 }
 
 __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict__ tp2id,
