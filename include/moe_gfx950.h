@@ -36,7 +36,9 @@ extern "C" {
 const char* moe_error_string(int code);
 /* ABI version of this header; bumped on any signature change. */
 int moe_abi_version(void);
-/* 0 when the current HIP device is gfx950, MOE_E_NO_DEVICE otherwise. */
+/* 0 when the current HIP device is gfx950, MOE_E_NO_DEVICE otherwise.  Also the library's per-device set-up: it
+ * looks up the address of that device's built-in scratch (moe_build_blocks_static), so call it once per device,
+ * outside any stream capture, before recording calls of the library into a HIP graph. */
 int moe_check_device(void);
 
 /* ---- element types ----------------------------------------------------------------- */
@@ -135,7 +137,10 @@ int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, i
  * per-slab counts live in a device array built into the library, MOE_BUILD_BLOCKS_STATIC_BYTES per GPU for the
  * life of the process.  Calls no hipMalloc / hipFree or any other allocating routine.  E above
  * MOE_BUILD_BLOCKS_STATIC_MAX_E returns MOE_E_STATIC_LIMIT (use moe_build_blocks with a workspace instead).  The
- * array is looked up once per device on the first call there (the device of `stream` must be current).  All calls
+ * array's address is looked up once per device, with that device current (the device of `stream` must be current
+ * in every call): by moe_check_device(), else by the first call of this entry point there.  That lookup is not
+ * guaranteed to be legal while a stream is being captured: before recording this call into a HIP graph on a device,
+ * call moe_check_device() or make one call outside the capture there.  All calls
  * on one GPU share that GPU's array: calls that overlap on one GPU (different streams, or threads) race; calls in
  * stream order do not.  Nothing in the array has to be cleared between calls. */
 #define MOE_BUILD_BLOCKS_STATIC_MAX_E 512

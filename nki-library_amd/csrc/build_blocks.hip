@@ -343,6 +343,15 @@ int static_scratch(void** out) {
 
 }  // namespace
 
+namespace moe {
+// Called by moe_check_device(): looks the current device's scratch up ahead of the first moe_build_blocks_static
+// call, so that a caller who records that call into a graph has no symbol lookup inside the capture.
+int build_blocks_static_setup() {
+  void* p = nullptr;
+  return static_scratch(&p);
+}
+}  // namespace moe
+
 extern "C" int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
                                 int skip_token, int use_split_padding, int32_t* token_position_to_id,
                                 int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions, void* workspace,

@@ -31,7 +31,8 @@ extern "C" int moe_check_device(void) {
   if (hipGetDevice(&dev) != hipSuccess) return MOE_E_NO_DEVICE;
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return MOE_E_NO_DEVICE;
-  return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? MOE_OK : MOE_E_NO_DEVICE;
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return MOE_E_NO_DEVICE;
+  return moe::build_blocks_static_setup();  // per-device set-up of the entry point that allocates nothing
 }
 
 namespace {

@@ -195,4 +195,7 @@ __device__ __forceinline__ float mx_inv_scale(uint32_t sbyte) { return __uint_as
 
 __device__ __forceinline__ float clip448(float v) { return fminf(fmaxf(v, -448.0f), 448.0f); }
 
+// csrc/build_blocks.hip: address of the current device's built-in scratch, looked up once per device
+int build_blocks_static_setup();
+
 }  // namespace moe

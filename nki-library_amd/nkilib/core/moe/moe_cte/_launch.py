@@ -31,7 +31,7 @@ _STAGES = (
 
 # K-contiguous copies of the dense (bf16 / fp8) expert weights, kept per weight tensor pair: the GEMMs of the bf16
 # and fp8-row kinds read both operands along K while the reference's layouts are N-contiguous, and the copies
-# depend on the weights only.  An entry lives as long as both weight tensor objects do and is remade when either
+# depend on the weights only.  An entry lives as long as both weight allocations do and is remade when either
 # was modified in place (torch's version counter).  Costs one more copy of the weights in HBM (two for fp8 weights
 # of the bf16 kind, which are widened); ``kmajor_weight_cache = False`` makes every call build its copies in the
 # workspace instead.
@@ -53,15 +53,23 @@ def clear_kmajor_weight_cache():
     _kmajor.clear()
 
 
+def _bytes_of(t):
+    """Where a weight tensor's bytes are: (address of its storage, byte offset, byte length).  Views and casts of one
+    allocation (``w.view(torch.int32)`` made anew for every call, say) name the same bytes."""
+    return (t.untyped_storage().data_ptr(), t.storage_offset() * t.element_size(), t.numel() * t.element_size())
+
+
 def _kmajor_weights(L, a, guw, dw, dev):
-    """``guw`` / ``dw``: the weight tensor objects as the caller of the operator passed them (an entry is found again
-    only through the same two objects: a caller that makes a new view of its weights for every call gets new copies
-    every time and should switch the copies off or keep the view)."""
-    key = (id(guw), id(dw))
-    sig = (guw._version, dw._version, guw.data_ptr(), dw.data_ptr(), tuple(guw.shape), tuple(dw.shape), guw.dtype,
-           dw.dtype, int(a.kind), int(a.weight_dtype), int(a.I_pad))
+    """``guw`` / ``dw``: the weight tensors as the caller of the operator passed them.  An entry is found through the
+    bytes the tensors name and how the call reads them (kind, weight type, expert shape), so a fresh view of the same
+    allocation hits; it is valid while both allocations are alive (weak references to the storages: an address that
+    was freed and handed out again is a different storage) and unchanged (torch's version counters, which views
+    share with their base)."""
+    st0, st1 = guw.untyped_storage(), dw.untyped_storage()
+    key = (_bytes_of(guw), _bytes_of(dw), int(a.kind), int(a.weight_dtype), int(a.E), int(a.H), int(a.I), int(a.I_pad))
+    sig = (guw._version, dw._version)
     ent = _kmajor.get(key)
-    if ent is not None and ent[0]() is guw and ent[1]() is dw and ent[2] == sig:
+    if ent is not None and ent[0]() is st0 and ent[1]() is st1 and ent[2] == sig:
         return ent[3], ent[4]
     n0 = L.moe_kmajor_weights_bytes(ctypes.byref(a), 0)
     n1 = L.moe_kmajor_weights_bytes(ctypes.byref(a), 1)
@@ -75,7 +83,7 @@ def _kmajor_weights(L, a, guw, dw, dev):
     if len(_kmajor) >= _KMAJOR_MAX_ENTRIES:
         _kmajor.pop(next(iter(_kmajor)))
     drop = lambda _ref, key=key: _kmajor.pop(key, None)
-    _kmajor[key] = (weakref.ref(guw, drop), weakref.ref(dw, drop), sig, k0, k1)
+    _kmajor[key] = (weakref.ref(st0, drop), weakref.ref(st1, drop), sig, k0, k1)
     return k0, k1
 
 

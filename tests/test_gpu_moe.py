@@ -286,6 +286,13 @@ def test_kmajor_weight_cache(fp8_row):
         first, second = run(), run()
         assert len(_launch._kmajor) == 1
         assert torch.equal(first, plain) and torch.equal(second, plain)
+        # a fresh view of the same allocations for every call finds the same entry
+        kept = _launch._kmajor[next(iter(_launch._kmajor))][3]
+        gu0, dw0 = gu, dw
+        gu, dw = gu0.view(gu0.dtype)[:], dw0.view(dw0.dtype)[:]
+        assert gu is not gu0 and torch.equal(run(), plain)
+        assert len(_launch._kmajor) == 1 and _launch._kmajor[next(iter(_launch._kmajor))][3] is kept
+        gu, dw = gu0, dw0
         # in-place change of one expert's down weights: the cached copies must not survive it
         if fp8_row:
             dw.view(torch.uint8)[0].bitwise_xor_(0x80)  # flips the sign of every weight of expert 0
@@ -745,3 +752,20 @@ def test_smoke_entry():
     import __graft_entry__ as ge
 
     ge.smoke()
+
+
+@pytest.mark.parametrize("T,lo,hi", [(62000, 1900, 2048), (68000, 2049, 4096), (134000, 4097, 5000)])
+def test_many_chunks_queue_paths(T, lo, hi):
+    """The work-queue builder keeps the chunk list in LDS up to 2048 chunks and the chunks' sort keys up to 4096
+    (beyond that the chunk-interleaved item order, which needs the keys, is switched off): one call on either side of
+    both limits, on a small expert shape of the large-tile bf16 kernels (64 experts of about 1000 / 1060 / 2100
+    rows each, i.e. several chunks per expert, the interleaved order where it applies), against the golden."""
+    H, I, E, k, B = 256, 128, 64, 8, 128
+    c = dense_case(T, H, I, E, k, B, seed=21)
+    rows = c["mask"].sum(axis=0).astype(np.int64)
+    n_chunks = int(sum(0 if r == 0 else 1 if r <= 320 else -(-(r - 320) // 256) + 1 for r in rows))
+    assert lo <= n_chunks <= hi, f"T={T}: {n_chunks} chunks, meant to lie in [{lo}, {hi}]"
+    out = from_bf16_tensor(_run_dense(c))
+    assert not out[:, 1].any()
+    g = _golden_dense(c)
+    _check(out[:T, 0], g[:T], f"{n_chunks} chunks (T={T})")
