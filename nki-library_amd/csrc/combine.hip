@@ -377,6 +377,8 @@ __global__ __launch_bounds__(256) void inv_fill_kernel(const int32_t* __restrict
   }
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 // One workgroup per output row (a few, side by side along the row, when the rows are too few to fill the GPU:
 // gridDim.y).  D: bf16 [N*B, H] contributions.
 __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict__ D, const int32_t* __restrict__ off,
@@ -412,14 +414,16 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
       // the additions form one dependent chain (bf16 rounding after each, in slot order), so the loads
       // are what can overlap: up to eight rows are requested before the first is added
       for (int j0 = 0; j0 < cnt; j0 += 8) {
-        uint4 d[8];
+        // (the contributions are read once and the result rows are not read again by this kernel: non-temporal,
+        // so that neither displaces the other in the caches)
+        u32x4 d[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-          if (j0 + j < cnt) d[j] = *(const uint4*)(D + (int64_t)s_sorted[j0 + j] * H + c);
+          if (j0 + j < cnt) d[j] = __builtin_nontemporal_load((const u32x4*)(D + (int64_t)s_sorted[j0 + j] * H + c));
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           if (j0 + j < cnt) {
-            const uint32_t w[4] = {d[j].x, d[j].y, d[j].z, d[j].w};
+            const uint32_t w[4] = {d[j][0], d[j][1], d[j][2], d[j][3]};
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
               acc[2 * k] = round_to_bf16(acc[2 * k] + bf16_bits_to_f32((uint16_t)(w[k] & 0xffff)));
@@ -432,8 +436,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
 #pragma unroll
       for (int k = 0; k < 4; ++k)
         o[k] = (uint32_t)f32_to_bf16_bits(acc[2 * k]) | ((uint32_t)f32_to_bf16_bits(acc[2 * k + 1]) << 16);
-      *(uint4*)(orow + c) = make_uint4(o[0], o[1], o[2], o[3]);
-      if (zrow) *(uint4*)(zrow + c) = make_uint4(0, 0, 0, 0);
+      __builtin_nontemporal_store((u32x4){o[0], o[1], o[2], o[3]}, (u32x4*)(orow + c));
+      if (zrow) __builtin_nontemporal_store((u32x4){0, 0, 0, 0}, (u32x4*)(zrow + c));
     }
   } else {
     for (int64_t c = vt; c < H; c += vstride) {
