@@ -49,13 +49,13 @@ def build(verbose=True, jobs=None):
     os.makedirs(OUT_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)
     inc = ["-I", os.path.join(ROOT, "include"), "-I", CSRC]
-    units = []  # (object path, extra defines, source)
-    for s in SOURCES:
-        units.append((os.path.join(OBJ_DIR, s.replace(".hip", ".o")), MX_FLAGS if s in M0_CLOBBER_SOURCES else [],
-                      os.path.join(CSRC, s)))
+    units = []  # (object path, extra defines, source); the long-running instances of the large-tile GEMM go first
     for stage, fmt in MX_INSTANCES:
         units.append((os.path.join(OBJ_DIR, f"bwmm_mx_s{stage}_f{fmt}.o"),
                       [*MX_FLAGS, f"-DMX_INST_STAGE={stage}", f"-DMX_INST_WFMT={fmt}"], os.path.join(CSRC, "bwmm_mx.hip")))
+    for s in SOURCES:
+        units.append((os.path.join(OBJ_DIR, s.replace(".hip", ".o")), MX_FLAGS if s in M0_CLOBBER_SOURCES else [],
+                      os.path.join(CSRC, s)))
     cmds = [["hipcc", *FLAGS, *defs, *inc, "-c", src, "-o", obj] for obj, defs, src in units]
     if verbose:
         for c in cmds:
