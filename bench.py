@@ -84,6 +84,9 @@ def parse_args():
     ap.add_argument("--no-mx-weight-copies", action="store_true",
                     help="diagnostic: read the MXFP8 expert weights in the reference layout in place instead of the "
                          "copies in the kernels' read order that moe_cte makes once per weight tensor pair")
+    ap.add_argument("--no-block-plans", action="store_true",
+                    help="diagnostic: build_token_blocks makes the three tables only and moe_cte derives its chunk / "
+                         "slot bookkeeping from them itself (four more small launches per step)")
     ap.add_argument("--routing", default="router", choices=["router", "balanced"],
                     help="router: top-k of synthetic scores (the reported workload); balanced: every expert gets "
                          "exactly T*k/E rows (diagnostic, shows the cost of ragged expert loads)")
@@ -179,6 +182,8 @@ def bench_fp8_row(args):
     from nkilib.core.moe.moe_cte import (MoECTEImplementation, MoECTESpec, QuantizationConfig, build_token_blocks,
                                          get_n_blocks, moe_cte)
     from nkilib.core.moe.moe_cte import _launch
+    from nkilib.core.moe.moe_cte import block_index
+    block_index.block_plans = not args.no_block_plans
     from nkilib.core.rmsnorm import RmsNormQuantKernelArgs, rmsnorm_quant_kernel
 
     dev = torch.device("cuda:0")
@@ -319,6 +324,8 @@ def main():
                                          get_n_blocks, moe_cte)
     from nkilib.core.moe.moe_cte import _launch
     _launch.mx_weight_copies = not args.no_mx_weight_copies
+    from nkilib.core.moe.moe_cte import block_index
+    block_index.block_plans = not args.no_block_plans
     from nkilib.core.subkernels.rmsnorm_mx_quantize_tkg import rmsnorm_mx_quantize
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"

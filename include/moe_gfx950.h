@@ -131,6 +131,24 @@ int moe_build_blocks(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, i
                      int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
                      void* workspace, size_t workspace_bytes, int32_t* status_out, void* stream);
 
+/* moe_build_blocks that also hands the blockwise layer its bookkeeping.  No counterpart in the reference (whose
+ * kernels walk the blocks of token_position_to_id as they are, bwmm_shard_on_block_mx.py:972-1347): moe_blockwise
+ * otherwise derives, from token_position_to_id and block_to_expert, the valid rows of every block, every token's
+ * list of slots and the expert chunks and work queues of its GEMM launches, in four small launches that read every
+ * slot twice; the block build knows all of that while it sorts.  Same arguments and the same three tables, bit for
+ * bit, as moe_build_blocks, plus `plan`: device memory of at least moe_block_plan_bytes(T, B, N, skip_token) bytes,
+ * 256-byte aligned, which this call fills (one more single-workgroup launch) and which moe_bwmm_args.block_plan
+ * passes to moe_blockwise.  A plan describes exactly the tables written by the same call: pass it only together
+ * with those token_position_to_id / block_to_expert buffers, unchanged, with the same B, N and token count
+ * (T1 = T + 1, or T with skip_token), and with `conditions` either NULL or the array this call wrote.
+ * T >= 1, T * k <= N * B and E <= 512 (MOE_E_BAD_SHAPE otherwise: use moe_build_blocks); use_split_padding
+ * returns MOE_E_UNSUPPORTED (which blocks run then depends on whether `conditions` is passed on). */
+size_t moe_block_plan_bytes(int64_t T, int64_t B, int64_t N, int skip_token);
+int moe_build_blocks_plan(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                          int skip_token, int use_split_padding, int32_t* token_position_to_id,
+                          int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions, void* workspace,
+                          size_t workspace_bytes, int32_t* status_out, void* plan, size_t plan_bytes, void* stream);
+
 /* moe_build_blocks for callers that cannot allocate or pass device scratch memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
  * the same results, bit for bit, as moe_build_blocks minus (workspace, workspace_bytes): the first slots and
@@ -282,6 +300,12 @@ typedef struct moe_bwmm_args {
    * instruction, the down GEMM the same into [2], [3]: cycles / ticks x 0.1 is the shader clock in GHz that the
    * part held under that launch (it is set by power management, not by the data sheet).  Read by bench.py. */
   int64_t* gemm_clocks;
+  /* Nullable, no counterpart in the reference: the bookkeeping that moe_build_blocks_plan wrote for exactly these
+   * token_position_to_id / block_to_expert tables (see there for the conditions under which it may be passed).
+   * With it moe_blockwise launches no bookkeeping kernels of its own.  Ignored when activation checkpoints are
+   * requested (their chunks cover whole blocks).  The plan is read only; it may be passed to any number of calls. */
+  const void* block_plan;
+  size_t block_plan_bytes;
 } moe_bwmm_args;
 
 /* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /

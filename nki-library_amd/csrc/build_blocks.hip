@@ -14,6 +14,8 @@
 // The work is latency bound (a few hundred KB of int32), so each step is a single small launch.
 #include <mutex>
 
+#include "chunks.hpp"
+#include "combine.hpp"
 #include "common.hpp"
 
 namespace moe {
@@ -24,6 +26,20 @@ constexpr int BB_SLABS_MAX = 64;
 constexpr int64_t BB_SINGLE_MAX_TOKENS = 1024;  // up to this many tokens form one slab, built by a single launch
 constexpr int64_t BB_SINGLE_MAX_SLOTS = 1 << 17;  // one workgroup fills the pad ids of up to this many slots itself
 constexpr int BB_E_MAX = 1024;  // bitmaps and running counts of all experts in LDS: 36 bytes per expert
+constexpr size_t BB_CHUNKS_STATIC_LDS = 46 * 1024;  // static LDS of build_chunks (csrc/chunks.hpp), rounded up
+
+// What the block build can tell the blockwise layer without another pass over the slots (all null: nothing):
+// the blocks in use, the valid rows of every block, and for every routed (token, j) pair the slot it was given.
+struct BlockPlanOut {
+  int32_t* n_active;    // [1]   blocks that hold tokens' experts (those before the padding blocks)
+  int32_t* valid_rows;  // [N]   rows of a block that hold tokens (they are packed from the block's first row)
+  int32_t* off;         // [T+1] first list entry of token t: t * k
+  int32_t* list;        // [T*k] slot of (t, j), or -1 (id outside [0, E), an id listed before in the row, no room)
+  // The layout step's workgroup goes on to cut the expert chunks and fill the work queues (build_chunks) when
+  // chunks_inline is set: the tables that takes (all of the blockwise layer's Bookkeeping).
+  int chunks_inline;
+  Bookkeeping k;
+};
 
 // The bitmaps of 256 tokens: bit (tid & 31) of word bm[(tid >> 5) * E + e] says that token t0 + tid selected
 // expert e.  Ids outside [0, E) are ignored; an id listed twice sets its bit once.
@@ -105,23 +121,26 @@ __global__ __launch_bounds__(BB_THREADS) void bb_count_kernel(const int32_t* __r
 // ws layout: first_slot[E] | slab_counts[BB_SLABS_MAX][E]
 // One workgroup: blocks per expert (padding blocks to the last expert, or split), exclusive scan ->
 // first slot of every expert, block_to_expert, conditions; sums and scans over the experts are
-// workgroup-wide (shuffles + one exchange), a tile of BB_THREADS experts at a time.
+// workgroup-wide (shuffles + one exchange), a tile of one expert per thread at a time.
 __device__ __forceinline__ void bb_layout_body(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
                                                int32_t* __restrict__ first_slot, int32_t* __restrict__ block_to_expert,
                                                int32_t* __restrict__ conditions, int64_t n_conditions, int64_t E,
                                                int64_t B, int64_t N, int use_split_padding,
-                                               int32_t* __restrict__ status, int* s_nb) {
-  // s_nb: [E] blocks per expert, then [E] first block of every expert
+                                               int32_t* __restrict__ status, int* s_nb, const BlockPlanOut plan) {
+  // s_nb: [E] blocks per expert, then [E] first block of every expert, then [E] tokens of every expert
   int* s_first = s_nb + E;
+  int* s_count = s_nb + 2 * E;
+  const int64_t nthr = blockDim.x;  // 256 in the single launch of a small batch, 1024 in a launch of its own
   __shared__ int s_npad;
   __shared__ int s_ws[16];
   // blocks per expert and their sum
   int mine = 0;
-  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
+  for (int64_t e = threadIdx.x; e < E; e += nthr) {
     int64_t count = 0;
 #pragma unroll 8
     for (int64_t sl = 0; sl < n_slabs; ++sl) count += slab_counts[sl * E + e];
     const int nb = (int)((count + B - 1) / B);
+    s_count[e] = (int)count;
     s_nb[e] = nb;
     mine += nb;
   }
@@ -140,9 +159,9 @@ __device__ __forceinline__ void bb_layout_body(const int32_t* __restrict__ slab_
     }
   }
   __syncthreads();
-  // first block of every expert: exclusive scan over the experts, a tile of BB_THREADS at a time
+  // first block of every expert: exclusive scan over the experts, a tile of nthr at a time
   int carry = 0;
-  for (int64_t base = 0; base < E; base += BB_THREADS) {
+  for (int64_t base = 0; base < E; base += nthr) {
     const int64_t e = base + threadIdx.x;
     const int v = (e < E) ? s_nb[e] : 0;
     int total;
@@ -151,11 +170,11 @@ __device__ __forceinline__ void bb_layout_body(const int32_t* __restrict__ slab_
     carry += total;
   }
   __syncthreads();
-  for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) first_slot[e] = (int32_t)((int64_t)s_first[e] * B);
+  for (int64_t e = threadIdx.x; e < E; e += nthr) first_slot[e] = (int32_t)((int64_t)s_first[e] * B);
   // A block's expert is the last one whose first block is not beyond it (experts without blocks share their first
   // block with the next expert, so the last of equals is the one that owns the block).  A search per block: the
   // padding blocks of a small batch all belong to one expert, and a loop per expert would write them one by one.
-  for (int64_t b = threadIdx.x; b < N; b += BB_THREADS) {
+  for (int64_t b = threadIdx.x; b < N; b += nthr) {
     int lo = 0, hi = (int)E;  // s_first[lo] <= b < s_first[hi]  (s_first[0] == 0, s_first[E] = infinity)
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
@@ -163,24 +182,38 @@ __device__ __forceinline__ void bb_layout_body(const int32_t* __restrict__ slab_
       else hi = mid;
     }
     block_to_expert[b] = lo;
+    if (plan.valid_rows) {
+      // tokens of expert lo less those in its earlier blocks
+      const int64_t left = (int64_t)s_count[lo] - (b - s_first[lo]) * B;
+      plan.valid_rows[b] = (int32_t)(left < 0 ? 0 : left > B ? B : left);
+    }
   }
+  if (plan.n_active && threadIdx.x == 0) *plan.n_active = (int32_t)(N - s_npad);
   if (conditions) {
     // ones, then zeros over the trailing (npad + n_conditions - N) entries
     const int64_t n_zero = s_npad + (n_conditions - N);
-    for (int64_t i = threadIdx.x; i < n_conditions; i += BB_THREADS)
+    for (int64_t i = threadIdx.x; i < n_conditions; i += nthr)
       conditions[i] = (i < n_conditions - n_zero) ? 1 : 0;
+  }
+  if (plan.chunks_inline) {
+    // block_to_expert, the valid rows and the number of blocks in use were written by this workgroup
+    __threadfence_block();
+    __syncthreads();
+    build_chunks(block_to_expert, plan.n_active, plan.valid_rows, N, B, E, plan.k.n_chunks, plan.k.chunk_slot,
+                 plan.k.chunk_rows, plan.k.chunk_expert, plan.k.chunk_xcd, plan.k.q_chunk, plan.k.q_off,
+                 plan.k.max_chunks, s_ws, false);
   }
 }
 
-__global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
+__global__ __launch_bounds__(1024) void bb_layout_kernel(const int32_t* __restrict__ slab_counts, int64_t n_slabs,
                                                               int32_t* __restrict__ first_slot,
                                                               int32_t* __restrict__ block_to_expert,
                                                               int32_t* __restrict__ conditions, int64_t n_conditions,
                                                               int64_t E, int64_t B, int64_t N, int use_split_padding,
-                                                              int32_t* __restrict__ status) {
+                                                              int32_t* __restrict__ status, const BlockPlanOut plan) {
   extern __shared__ int s_nb_dyn[];
   bb_layout_body(slab_counts, n_slabs, first_slot, block_to_expert, conditions, n_conditions, E, B, N,
-                 use_split_padding, status, s_nb_dyn);
+                 use_split_padding, status, s_nb_dyn, plan);
 }
 
 // Workgroup = slab.  A token's slot for expert e: first slot of e + tokens of e in the slabs before (summed here
@@ -188,7 +221,7 @@ __global__ __launch_bounds__(BB_THREADS) void bb_layout_kernel(const int32_t* __
 __device__ __forceinline__ void bb_scatter_body(const int32_t* __restrict__ ids, int64_t T, int64_t k, int64_t E,
                                                 int64_t slab_tokens, const int32_t* __restrict__ slab_counts,
                                                 const int32_t* __restrict__ first_slot, int32_t* __restrict__ tp2id,
-                                                int64_t NB, int64_t slab, uint32_t* bb_lds) {
+                                                int64_t NB, int64_t slab, uint32_t* bb_lds, const BlockPlanOut plan) {
   uint32_t* bm = bb_lds;
   int* run = (int*)(bb_lds + 8 * E);
   for (int64_t e = threadIdx.x; e < E; e += BB_THREADS) {
@@ -209,14 +242,44 @@ __device__ __forceinline__ void bb_scatter_body(const int32_t* __restrict__ ids,
     bb_mark(ids, t, live, k, E, bm, my);
     __syncthreads();
     if (live) {
-      const int64_t kk = (k == 8) ? 8 : k;
-      for (int64_t j = 0; j < kk; ++j) {
-        const int e = (k == 8) ? my[j] : ids[t * k + j];
-        if (e < 0 || e >= E) continue;
+      // the slot of token t under expert e: the expert's first free slot + the tokens of e before t in this pass
+      auto place = [&](int e) -> int32_t {
+        if (e < 0 || e >= E) return -1;
         int r = __popc(bm[wd * E + e] & below);
         for (int w = 0; w < wd; ++w) r += __popc(bm[w * E + e]);
         const int64_t pos = (int64_t)run[e] + r;
-        if (pos < NB) tp2id[pos] = (int32_t)t;
+        if (pos >= NB) return -1;
+        tp2id[pos] = (int32_t)t;
+        return (int32_t)pos;
+      };
+      // (for the plan: an id that the row lists twice owns one slot, the second mention adds nothing)
+      if (k == 8) {
+        int32_t slot[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          slot[j] = place(my[j]);
+#pragma unroll
+          for (int j2 = 0; j2 < j; ++j2)
+            if (my[j2] == my[j]) slot[j] = -1;
+        }
+        if (plan.list) {  // two 16-byte stores (the plan is 256-byte aligned)
+          ((int4*)(plan.list + t * 8))[0] = make_int4(slot[0], slot[1], slot[2], slot[3]);
+          ((int4*)(plan.list + t * 8))[1] = make_int4(slot[4], slot[5], slot[6], slot[7]);
+        }
+      } else {
+        for (int64_t j = 0; j < k; ++j) {
+          const int e = ids[t * k + j];
+          int32_t slot = place(e);
+          if (plan.list) {
+            for (int64_t j2 = 0; j2 < j; ++j2)
+              if (ids[t * k + j2] == e) slot = -1;
+            plan.list[t * k + j] = slot;
+          }
+        }
+      }
+      if (plan.off) {
+        plan.off[t] = (int32_t)(t * k);
+        if (t == T - 1) plan.off[T] = (int32_t)(T * k);
       }
     }
     __syncthreads();
@@ -229,9 +292,10 @@ __global__ __launch_bounds__(BB_THREADS) void bb_scatter_kernel(const int32_t* _
                                                                int64_t E, int64_t slab_tokens,
                                                                const int32_t* __restrict__ slab_counts,
                                                                const int32_t* __restrict__ first_slot,
-                                                               int32_t* __restrict__ tp2id, int64_t NB) {
+                                                               int32_t* __restrict__ tp2id, int64_t NB,
+                                                               const BlockPlanOut plan) {
   extern __shared__ uint32_t bb_lds[];
-  bb_scatter_body(ids, T, k, E, slab_tokens, slab_counts, first_slot, tp2id, NB, blockIdx.x, bb_lds);
+  bb_scatter_body(ids, T, k, E, slab_tokens, slab_counts, first_slot, tp2id, NB, blockIdx.x, bb_lds, plan);
 }
 
 // Few tokens (one slab): the three steps in one launch by one workgroup.  What one step leaves in global memory
@@ -241,14 +305,14 @@ __global__ __launch_bounds__(BB_THREADS) void bb_single_slab_kernel(
     const int32_t* __restrict__ ids, int64_t T, int64_t k, int64_t E, int64_t slab_tokens,
     int32_t* __restrict__ slab_counts, int32_t* __restrict__ first_slot, int32_t* __restrict__ tp2id, int64_t NB,
     int pad_id, int32_t* __restrict__ block_to_expert, int32_t* __restrict__ conditions, int64_t n_conditions, int64_t B,
-    int64_t N, int use_split_padding, int32_t* __restrict__ status) {
-  extern __shared__ uint32_t bb_lds[];  // 9 E words of the count / scatter steps, then 2 E of the layout step
+    int64_t N, int use_split_padding, int32_t* __restrict__ status, const BlockPlanOut plan) {
+  extern __shared__ uint32_t bb_lds[];  // 9 E words of the count / scatter steps, then 3 E of the layout step
   bb_count_body(ids, T, k, E, slab_tokens, slab_counts, tp2id, NB, pad_id, 0, 1, bb_lds);
   __syncthreads();
   bb_layout_body(slab_counts, 1, first_slot, block_to_expert, conditions, n_conditions, E, B, N, use_split_padding,
-                 status, (int*)(bb_lds + 9 * E));
+                 status, (int*)(bb_lds + 9 * E), plan);
   __syncthreads();
-  bb_scatter_body(ids, T, k, E, slab_tokens, slab_counts, first_slot, tp2id, NB, 0, bb_lds);
+  bb_scatter_body(ids, T, k, E, slab_tokens, slab_counts, first_slot, tp2id, NB, 0, bb_lds, plan);
 }
 
 }  // namespace moe
@@ -267,7 +331,8 @@ namespace {
 // first slot), so stale contents of an earlier call are never seen and nothing has to be cleared.
 int build_blocks_launch(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N, int skip_token,
                         int use_split_padding, int32_t* token_position_to_id, int32_t* block_to_expert,
-                        int32_t* conditions, int64_t n_conditions, int32_t* ws, int32_t* status_out, hipStream_t s) {
+                        int32_t* conditions, int64_t n_conditions, int32_t* ws, int32_t* status_out, hipStream_t s,
+                        BlockPlanOut plan = BlockPlanOut{}) {
   // at most BB_SLABS_MAX slabs of a multiple of 256 tokens
   int64_t slab_tokens = (T + BB_SLABS_MAX - 1) / BB_SLABS_MAX;
   slab_tokens = (slab_tokens + BB_THREADS - 1) / BB_THREADS * BB_THREADS;
@@ -279,22 +344,28 @@ int build_blocks_launch(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E
   int32_t* first_slot = ws;
   int32_t* slab_counts = first_slot + E;
   const size_t lds = (size_t)9 * E * sizeof(int32_t);
+  const bool planned = plan.valid_rows != nullptr;
   if (n_slabs == 1 && N * B <= BB_SINGLE_MAX_SLOTS) {
-    hipLaunchKernelGGL(bb_single_slab_kernel, dim3(1), dim3(BB_THREADS), lds + 2 * E * sizeof(int32_t), s, topk_ids, T,
+    // (the chunk builder's tables are static LDS of the kernel: it runs in this launch while both fit in 64 KB)
+    plan.chunks_inline = planned && lds + 3 * E * sizeof(int32_t) + BB_CHUNKS_STATIC_LDS <= 65536;
+    hipLaunchKernelGGL(bb_single_slab_kernel, dim3(1), dim3(BB_THREADS), lds + 3 * E * sizeof(int32_t), s, topk_ids, T,
                        k, E, slab_tokens, slab_counts, first_slot, token_position_to_id, N * B,
                        skip_token ? -1 : (int)T, block_to_expert, conditions, n_conditions, B, N, use_split_padding,
-                       status_out);
+                       status_out, plan);
     MOE_CHECK_LAUNCH();
+    if (planned && !plan.chunks_inline) return launch_plan_chunks(plan.k, block_to_expert, N, B, E, s);
     return MOE_OK;
   }
   hipLaunchKernelGGL(bb_count_kernel, dim3((unsigned)n_slabs), dim3(BB_THREADS), lds, s, topk_ids, T, k, E, slab_tokens,
                      slab_counts, token_position_to_id, N * B, skip_token ? -1 : (int)T);
   MOE_CHECK_LAUNCH();
-  hipLaunchKernelGGL(bb_layout_kernel, dim3(1), dim3(BB_THREADS), 2 * E * sizeof(int), s, slab_counts, n_slabs,
-                     first_slot, block_to_expert, conditions, n_conditions, E, B, N, use_split_padding, status_out);
+  plan.chunks_inline = planned;  // (3 E words of dynamic LDS beside the chunk builder's tables: E <= 1024 fits)
+  hipLaunchKernelGGL(bb_layout_kernel, dim3(1), dim3(planned ? 1024 : BB_THREADS), 3 * E * sizeof(int), s, slab_counts, n_slabs,
+                     first_slot, block_to_expert, conditions, n_conditions, E, B, N, use_split_padding, status_out,
+                     plan);
   MOE_CHECK_LAUNCH();
   hipLaunchKernelGGL(bb_scatter_kernel, dim3((unsigned)n_slabs), dim3(BB_THREADS), lds, s, topk_ids, T, k, E,
-                     slab_tokens, slab_counts, first_slot, token_position_to_id, N * B);
+                     slab_tokens, slab_counts, first_slot, token_position_to_id, N * B, plan);
   MOE_CHECK_LAUNCH();
   return MOE_OK;
 }
@@ -377,4 +448,37 @@ extern "C" int moe_build_blocks_static(const int32_t* topk_ids, int64_t T, int64
   if (rc != MOE_OK) return rc;
   return build_blocks_launch(topk_ids, T, k, E, B, N, skip_token, use_split_padding, token_position_to_id,
                              block_to_expert, conditions, n_conditions, (int32_t*)ws, status_out, (hipStream_t)stream);
+}
+
+// ---- the block build that also hands the blockwise layer its bookkeeping ----------------------------------
+extern "C" size_t moe_block_plan_bytes(int64_t T, int64_t B, int64_t N, int skip_token) {
+  if (T < 1 || B <= 0 || N <= 0) return 0;
+  return bookkeeping_bytes(skip_token ? T : T + 1, N, B);
+}
+
+extern "C" int moe_build_blocks_plan(const int32_t* topk_ids, int64_t T, int64_t k, int64_t E, int64_t B, int64_t N,
+                                     int skip_token, int use_split_padding, int32_t* token_position_to_id,
+                                     int32_t* block_to_expert, int32_t* conditions, int64_t n_conditions,
+                                     void* workspace, size_t workspace_bytes, int32_t* status_out, void* plan,
+                                     size_t plan_bytes, void* stream) {
+  const int rc = build_blocks_check(topk_ids, T, k, E, B, N, token_position_to_id, block_to_expert, conditions, n_conditions);
+  if (rc != MOE_OK) return rc;
+  if (!workspace || !plan || ((uintptr_t)plan & 255) != 0) return MOE_E_BAD_ARG;
+  // (split padding puts padding blocks in the middle of the list while `conditions` still ends with as many zeros:
+  // which blocks run then depends on whether the caller passes `conditions`, which a plan cannot know)
+  if (use_split_padding) return MOE_E_UNSUPPORTED;
+  if (workspace_bytes < moe_build_blocks_workspace_bytes(E)) return MOE_E_WORKSPACE;
+  // a plan lists T * k slots in the N * B words that the slot lists of the blockwise layer occupy
+  if (T < 1 || T * k > N * B || E > COMBINE_MAX_K) return MOE_E_BAD_SHAPE;
+  if (plan_bytes < moe_block_plan_bytes(T, B, N, skip_token)) return MOE_E_WORKSPACE;
+  const Bookkeeping bk = carve_bookkeeping(plan, skip_token ? T : T + 1, N, B);
+  BlockPlanOut out{};
+  out.n_active = bk.n_active;
+  out.valid_rows = bk.valid_rows;
+  out.off = bk.off;
+  out.list = bk.list;
+  out.k = bk;
+  return build_blocks_launch(topk_ids, T, k, E, B, N, skip_token, use_split_padding, token_position_to_id,
+                             block_to_expert, conditions, n_conditions, (int32_t*)workspace, status_out,
+                             (hipStream_t)stream, out);
 }

@@ -24,7 +24,7 @@ extern "C" const char* moe_error_string(int code) {
   }
 }
 
-extern "C" int moe_abi_version(void) { return 6; }
+extern "C" int moe_abi_version(void) { return 7; }
 
 extern "C" int moe_check_device(void) {
   int dev = 0;
@@ -336,8 +336,14 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
   hipStream_t s = (hipStream_t)stream;
   uint8_t* ws = (uint8_t*)a->workspace;
   const int64_t n_real = a->skip_token ? a->T1 : a->T1 - 1;
-  const Bookkeeping bk = carve_bookkeeping(ws + p.book, a->T1, a->N, a->B);
-  if (stages & MOE_STAGE_PREP) {
+  // The chunk / slot bookkeeping: derived here from token_position_to_id, or taken as the block build left it
+  // (moe_build_blocks_plan).  Activation checkpoints cover whole blocks, which a plan's chunks do not: the plan is
+  // then left aside.
+  const bool planned = a->block_plan != nullptr && !a->gate_up_activations_T && !a->down_activations;
+  if (planned && (a->block_plan_bytes < bookkeeping_bytes(a->T1, a->N, a->B) || ((uintptr_t)a->block_plan & 255) != 0))
+    return MOE_E_BAD_ARG;
+  const Bookkeeping bk = carve_bookkeeping(planned ? (void*)a->block_plan : (void*)(ws + p.book), a->T1, a->N, a->B);
+  if ((stages & MOE_STAGE_PREP) && !planned) {
     rc = launch_prep(bk, a, n_real, s);
     if (rc != MOE_OK) return rc;
   }

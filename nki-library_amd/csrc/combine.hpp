@@ -52,6 +52,7 @@ __host__ __device__ inline int chunk_class(int rows, bool last) {
 }
 
 constexpr int CHUNK_ROWS = 256;      // rows of every chunk of a run but the last
+constexpr int CHUNK_FIXED_COST_TILES = 20;  // a chunk's loads per K slice, in row tiles of MFMA time (XCD balance)
 constexpr int CHUNK_ROWS_MAX = 320;  // the last chunk of a run takes up to this many
 inline int64_t max_chunks_for(int64_t N, int64_t B) { return N * ((B + CHUNK_ROWS - 1) / CHUNK_ROWS); }
 
@@ -59,6 +60,10 @@ size_t bookkeeping_bytes(int64_t T1, int64_t N, int64_t B);
 Bookkeeping carve_bookkeeping(void* base, int64_t T1, int64_t N, int64_t B);
 // n_real: number of real token rows (ids in [0, n_real) are tokens, everything else is padding).
 int launch_prep(const Bookkeeping& k, const moe_bwmm_args* a, int64_t n_real, hipStream_t s);
+// The chunk list and the work queues alone, from valid_rows / n_active that the caller has filled in (the block
+// build's hand-over, see moe_build_blocks_plan).
+int launch_plan_chunks(const Bookkeeping& k, const int32_t* block_to_expert, int64_t N, int64_t B, int64_t E,
+                       hipStream_t s);
 int launch_combine(const Bookkeeping& k, const moe_bwmm_args* a, const void* D, int64_t n_real, hipStream_t s);
 // Zero `bytes` bytes at p (a multiple of 4, p 4-byte aligned) with a kernel, so that callers may capture it in a graph.
 int launch_fill_zero_bytes(void* p, size_t bytes, hipStream_t s);

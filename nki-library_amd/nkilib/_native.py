@@ -35,6 +35,8 @@ EXPORTED_SYMBOLS = (
     "moe_build_blocks_workspace_bytes",
     "moe_build_blocks",
     "moe_build_blocks_static",
+    "moe_block_plan_bytes",
+    "moe_build_blocks_plan",
     "moe_find_nonzero_indices_workspace_bytes",
     "moe_find_nonzero_indices",
     "moe_indexed_flatten",
@@ -100,6 +102,8 @@ class BwmmArgs(ctypes.Structure):
         ("down_proj_weight_kmajor", c_void_p),
         ("output_shard1", c_void_p),
         ("gemm_clocks", c_void_p),
+        ("block_plan", c_void_p),
+        ("block_plan_bytes", c_size_t),
     ]
 
 
@@ -141,6 +145,12 @@ def lib():
     L.moe_build_blocks_static.restype = c_int
     L.moe_build_blocks_static.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p,
                                           c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
+    L.moe_block_plan_bytes.restype = c_size_t
+    L.moe_block_plan_bytes.argtypes = [c_int64, c_int64, c_int64, c_int]
+    L.moe_build_blocks_plan.restype = c_int
+    L.moe_build_blocks_plan.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p,
+                                        c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_void_p, c_size_t,
+                                        c_void_p]
     L.moe_find_nonzero_indices_workspace_bytes.restype = c_size_t
     L.moe_find_nonzero_indices_workspace_bytes.argtypes = [c_int64, c_int64]
     L.moe_find_nonzero_indices.restype = c_int

@@ -220,6 +220,13 @@ def run_blockwise(
         ck_down = torch.empty((N, B, H), dtype=torch.bfloat16, device=dev)
         a.down_activations = nv.ptr(ck_down)
 
+    plan = None
+    if not (checkpoint_gate_up or checkpoint_down):
+        from . import block_index
+
+        plan = block_index.plan_for(tp2id, b2e, cond, B, N, T1)
+        if plan is not None:
+            a.block_plan, a.block_plan_bytes = plan
     if gemm_clock_probe is not None:
         kernel_assert(gemm_clock_probe.dtype == torch.int64 and gemm_clock_probe.numel() >= 4 and gemm_clock_probe.is_cuda,
                       "gemm_clock_probe must be a device int64 tensor of 4 elements")

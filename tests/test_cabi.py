@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported():
     for name in declared:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
     assert set(nv.EXPORTED_SYMBOLS) == set(declared)
-    assert L.moe_abi_version() == 6
+    assert L.moe_abi_version() == 7
     assert b"workspace" in L.moe_error_string(-3)
 
 
