@@ -579,9 +579,13 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   //                         first slice of every D
   //   then NBL              weights (16 bytes per lane each, into a raw register set)
   //   then 1                weight scales
+  // (SCALED: the MX formats.  The fp8-row and bf16 kinds have block scales of 2^0 throughout: their K loop loads
+  // no scales at all and hands the MFMAs the constant)
+  constexpr bool SCALED = !ROW8;
+  constexpr int UNIT_SCALES = 0x7f7f7f7f;
   constexpr int NBL = 8;
-  constexpr int NSC = BIG ? 2 : 1;
-  constexpr int NLB = NBL + 1;              // weight loads of a slice
+  constexpr int NSC = SCALED ? (BIG ? 2 : 1) : 0;
+  constexpr int NLB = NBL + (SCALED ? 1 : 0);  // weight loads of a slice
   constexpr int N1 = NAJ + NLB;             // loads of a slice that carries no activation scales
   constexpr int N0 = N1 + NSC;              // loads of one that does
   typedef typename std::conditional<D == 3, v3i, v2i>::type ScaleRegs;
@@ -695,7 +699,8 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       if constexpr (FP4) ld_b64<LASTUSE>(b.d[i], w_voff, rw_, w_soff[i] + sa.w_off);
       else ld_b128<LASTUSE>(b.d[i], w_voff, rw_, w_soff[i] + sa.w_off);
     } else {
-      ld_b32(b.sc, s_voff, rs_, s_soff + sa.s_off);
+      static_assert(SCALED || idx < NAJ + NSC + NBL, "no scale load without scales");
+      if constexpr (SCALED) ld_b32(b.sc, s_voff, rs_, s_soff + sa.s_off);
     }
   };
   // The MFMA wants a lane's scale byte to be that of row 16*mt + c and K block g, one byte per row
@@ -739,16 +744,19 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     acc_fence();
     const uint8_t* plo = sA + st * SA + rd_lo;
     const uint8_t* phi = sA + st * SA + rd_hi;
-    const v4i asc = *(const v4i*)(sS + st * SS + (g * 16 + c) * SSP);
-    int asc_hi = 0;
-    if constexpr (BIG) asc_hi = *(const int*)(sS + st * SS + (g * 16 + c) * SSP + 16);
+    v4i asc = (v4i){UNIT_SCALES, UNIT_SCALES, UNIT_SCALES, UNIT_SCALES};
+    int asc_hi = UNIT_SCALES;
+    if constexpr (SCALED) {
+      asc = *(const v4i*)(sS + st * SS + (g * 16 + c) * SSP);
+      if constexpr (BIG) asc_hi = *(const int*)(sS + st * SS + (g * 16 + c) * SSP + 16);
+    }
     // first fragments of this slice: in flight while the weights are transposed
     v8i af[2][2];
     af[0][0] = frag_from_lds(plo, phi);
     af[0][1] = frag_from_lds(plo + 16 * MXROW, phi + 16 * MXROW);
     asm volatile("" ::: "memory");
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NLB + (D - 2) * N1) : "memory");
-    if constexpr (U == D - 1) {  // activation scales of slices ks+1 .. ks+D
+    if constexpr (SCALED && U == D - 1) {  // activation scales of slices ks+1 .. ks+D
       asm volatile("" : "+v"(asr));
       if constexpr (BIG) asm volatile("" : "+v"(asr2));
     }
@@ -781,7 +789,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
         b.f[3][r] = braw.d[r][3];
       }
     }
-    b.sc = braw.sc;
+    b.sc = SCALED ? braw.sc : UNIT_SCALES;
     asm volatile("s_nop 1" : "+v"(b.f[0]), "+v"(b.f[1]), "+v"(b.f[2]), "+v"(b.f[3]), "+v"(b.sc));
     SliceAddr sad;
     static_for<0, NG>([&](auto gi_) {
@@ -811,7 +819,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
           asm volatile("" : "+s"(ksd));
           sad = slice_addr(ksd, wrapst(st + D));
         }
-        if constexpr (U == D - 1 && m >= 3 && m < 3 + D) {
+        if constexpr (SCALED && U == D - 1 && m >= 3 && m < 3 + D) {
           scales_to_operand_order(wrapst(st + m - 2), (uint32_t)asr[m - 3], tid);
           if constexpr (BIG) scales_to_operand_order(wrapst(st + m - 2), (uint32_t)asr2[m - 3], row_hi);
         }
@@ -875,13 +883,16 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) accv[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  // (the activation rows of slice 0, and the activation scales of the first D slices, are in)
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NLB + (D - 1) * N1) : "memory");
-  asm volatile("" : "+v"(asr));
-  if constexpr (BIG) asm volatile("" : "+v"(asr2));
+  if constexpr (SCALED) {
+    asm volatile("" : "+v"(asr));
+    if constexpr (BIG) asm volatile("" : "+v"(asr2));
 #pragma unroll
-  for (int j = 0; j < D; ++j) {
-    scales_to_operand_order(j, (uint32_t)asr[j], tid);
-    if constexpr (BIG) scales_to_operand_order(j, (uint32_t)asr2[j], row_hi);
+    for (int j = 0; j < D; ++j) {
+      scales_to_operand_order(j, (uint32_t)asr[j], tid);
+      if constexpr (BIG) scales_to_operand_order(j, (uint32_t)asr2[j], row_hi);
+    }
   }
   __syncthreads();
   int st = 0;
