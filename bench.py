@@ -63,8 +63,8 @@ def profiled_traffic(workload, routing):
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sustain-seconds", type=float, default=2.0,
@@ -171,6 +171,41 @@ def cpu_baseline(cfg, t, tp2id, b2e, n_blocks):
     }
 
 
+class StepEvents:
+    """HIP events of one step: three recorded here (torch's current stream: the stream every kernel of the path is
+    launched on) around the front end and the block build, seven recorded by the library itself between the stages
+    of the one moe_blockwise call (moe_bwmm_args.stage_events), so that the step is the ordinary step.  An event
+    costs the GPU 7-8 us on this part (a barrier and a timestamp in the queue), so the K timed steps carry only the
+    two around the dominant kernel (``gemm_only``: the gate/up launch, which the roofline prices); the per-stage
+    table comes from K more steps, run after the timed ones, that carry all ten."""
+
+    def __init__(self, torch, gemm_only=False):
+        self.py = [None if gemm_only else torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        self.lib = [torch.cuda.Event(enable_timing=True) if (not gemm_only or i in (2, 3)) else None for i in range(7)]
+        for e in self.py + self.lib:
+            if e is not None:
+                e.record()  # creates the HIP event, whose handle the library is given
+
+    def mark(self, i):
+        if self.py[i] is not None:
+            self.py[i].record()
+
+    def gate_up_ms(self):
+        return self.lib[2].elapsed_time(self.lib[3])
+
+    def stage_ms(self, with_requant):
+        t = lambda a, b: a.elapsed_time(b)
+        out = {"norm_quant": t(self.py[0], self.py[1]), "build_blocks": t(self.py[1], self.py[2]),
+               "prep": t(self.py[2], self.lib[2]), "gate_up": t(self.lib[2], self.lib[3])}
+        if with_requant:
+            out["requant"] = t(self.lib[3], self.lib[4])
+            out["down"] = t(self.lib[4], self.lib[5])
+        else:
+            out["down"] = t(self.lib[3], self.lib[5])
+        out["combine"] = t(self.lib[5], self.lib[6])
+        return out
+
+
 def bench_fp8_row(args):
     """BASELINE config 2: RMSNorm-Quant (fp8 rows + fp32 row scale) -> block build -> fp8-row blockwise layer.
     `--workload bf16` runs the same stages on the bf16 kind (bf16 hidden states and weights, no front end, no row
@@ -211,41 +246,40 @@ def bench_fp8_row(args):
         kw = {"quantization_config": QuantizationConfig(gu_s, d_s)}
         gu8, d8 = gu_q.view(torch.float8_e4m3fn), d_q.view(torch.float8_e4m3fn)
         names = ["norm_quant", "build_blocks", "prep", "gate_up", "requant", "down", "combine"]
-    events = []
+    timed_events = [StepEvents(torch, gemm_only=True) for _ in range(args.steps)]
+    events = [StepEvents(torch) for _ in range(args.steps)]
 
-    def rec():
-        ev = torch.cuda.Event(enable_timing=True)
-        ev.record()
-        events[-1].append(ev)
-
-    def step(timed):
-        if timed:
-            events.append([])
-            rec()
+    def step(ev):
+        if ev:
+            ev.mark(0)
         recs = x if bf16 else rmsnorm_quant_kernel(x, gamma, RmsNormQuantKernelArgs())
-        if timed:
-            rec()
+        if ev:
+            ev.mark(1)
         tp2id, b2e, cond = build_token_blocks(ids, E, B, N)
-        if timed:
-            rec()
-        _launch.stage_callback = (lambda name: rec()) if timed else None
+        if ev:
+            ev.mark(2)
+        _launch.stage_events = ev.lib if ev else None
         out = moe_cte[2](recs, aff.reshape(-1, 1), gu8, d8, tp2id, b2e, B, spec, **kw)
-        _launch.stage_callback = None
+        _launch.stage_events = None
         return out, recs, tp2id, b2e
 
     for _ in range(args.warmup):
-        step(False)
+        step(None)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out, recs, tp2id, b2e = step(True)
+    for i in range(args.steps):
+        out, recs, tp2id, b2e = step(timed_events[i])
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    gate_up_timed_ms = sum(ev.gate_up_ms() for ev in timed_events) / args.steps
+    for i in range(args.steps):  # the per-stage table: the same steps again, every stage boundary recorded
+        step(events[i])
+    torch.cuda.synchronize()
     stage_ms = {n: 0.0 for n in names}
-    for evs in events:
-        assert len(evs) == len(names) + 1, (len(evs), names)
-        for i, n in enumerate(names):
-            stage_ms[n] += evs[i].elapsed_time(evs[i + 1]) / args.steps
+    for ev in events:
+        for n, v in ev.stage_ms(with_requant=not bf16).items():
+            stage_ms[n] += v / args.steps
+    stage_ms["gate_up"] = gate_up_timed_ms  # (the launch duration the roofline uses: from the timed steps)
     routed = int((tp2id.reshape(-1) < T).sum().item())
     flops_layer, flops_gu = 6.0 * routed * H * I, 4.0 * routed * H * I
     tflops = flops_layer / (ms_per_step * 1e-3) / 1e12
@@ -349,52 +383,57 @@ def main():
         g = torch.Generator(device=dev)
         g.manual_seed(77)
         w_router = (torch.randn((H, E), generator=g, device=dev) * 0.05).to(torch.bfloat16)
-    events = []
+    timed_events = [StepEvents(torch, gemm_only=True) for _ in range(args.steps)]
+    events = [StepEvents(torch) for _ in range(args.steps)]
+    router_events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
 
-    def rec():
-        ev = torch.cuda.Event(enable_timing=True)
-        ev.record()  # torch's current stream: the stream every kernel of the path is launched on
-        events[-1].append(ev)
-
-    def step(timed):
-        if timed:
-            events.append([])
-            rec()
+    def step(timed, i=0, all_stages=False):
+        ev = (events[i] if all_stages else timed_events[i]) if timed else None
         if args.with_router:
+            if all_stages:
+                router_events[i][0].record()
             t["ids"], t["aff"] = route_for_moe(t["x"], w_router, None, k, RouterActFnType.SIGMOID, norm_topk_prob=True)
-            if timed:
-                rec()
+            if all_stages:
+                router_events[i][1].record()
+        if ev:
+            ev.mark(0)
         xq, xs = rmsnorm_mx_quantize(t["x"], t["gamma"])
-        if timed:
-            rec()
+        if ev:
+            ev.mark(1)
         tp2id, b2e, cond = build_token_blocks(t["ids"], E, B, N, n_conditions=N + 2)
-        if timed:
-            rec()
-        _launch.stage_callback = (lambda name: rec()) if timed else None
+        if ev:
+            ev.mark(2)
+        _launch.stage_events = ev.lib if ev else None
         out = moe_cte[2](xq, t["aff"].reshape(-1, 1), gu_x4, t["d_q"], tp2id, b2e, B, spec, conditions=cond,
                          quantization_config=qcfg, hidden_states_scale=xs)
-        _launch.stage_callback = None
+        _launch.stage_events = None
         return out, tp2id, b2e
 
     for _ in range(args.warmup):
         step(False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out, tp2id, b2e = step(True)
+    for i in range(args.steps):
+        out, tp2id, b2e = step(True, i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
+    gate_up_timed_ms = sum(ev.gate_up_ms() for ev in timed_events) / args.steps
+    for i in range(args.steps):  # the per-stage table: the same steps again, every stage boundary recorded
+        step(True, i, all_stages=True)
+    torch.cuda.synchronize()
     stage_ms = {n: 0.0 for n in names}
-    for evs in events:
-        assert len(evs) == len(names) + 1, (len(evs), names)
-        for i, n in enumerate(names):
-            stage_ms[n] += evs[i].elapsed_time(evs[i + 1])
+    for i, ev in enumerate(events):
+        for n, v in ev.stage_ms(with_requant=False).items():
+            stage_ms[n] += v
+        if args.with_router:
+            stage_ms["router"] += router_events[i][0].elapsed_time(router_events[i][1])
     stage_ms = {n: v / args.steps for n, v in stage_ms.items()}
+    stage_ms["gate_up"] = gate_up_timed_ms  # (the launch duration the roofline uses: from the timed steps)
 
     # Sustained pace: the same step, back to back, for at least --sustain-seconds more (the clock under load is a
-    # power-management outcome with a time constant far beyond the 20 timed steps).  Workgroup 0 of each GEMM launch
+    # power-management outcome with a time constant beyond the timed steps).  Workgroup 0 of each GEMM launch
     # reports its shader cycles and the ticks of the constant 100 MHz counter: their ratio is the clock it ran at.
     sustained = None
     if args.sustain_seconds > 0:

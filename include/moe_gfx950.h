@@ -306,6 +306,12 @@ typedef struct moe_bwmm_args {
    * requested (their chunks cover whole blocks).  The plan is read only; it may be passed to any number of calls. */
   const void* block_plan;
   size_t block_plan_bytes;
+  /* Nullable, no counterpart in the reference: seven hipEvent_t of the caller's (null entries are skipped).  The
+   * call records them on `stream`: [0] on entry, [1] after the bookkeeping, [2] ahead of the gate/up stage (after
+   * the online activation quantisation and any per-call weight copies), [3] after the gate/up GEMM, [4] after the
+   * fp8-row re-quantisation, [5] after the down GEMM, [6] after the combine.  Lets a benchmark time the stages of one
+   * ordinary call instead of calling moe_blockwise_stages once per stage.  Read by bench.py. */
+  void* const* stage_events;
 } moe_bwmm_args;
 
 /* Replaces bwmm_shard_on_block / blockwise_mm_baseline_shard_intermediate* /

@@ -339,6 +339,11 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
   // The chunk / slot bookkeeping: derived here from token_position_to_id, or taken as the block build left it
   // (moe_build_blocks_plan).  Activation checkpoints cover whole blocks, which a plan's chunks do not: the plan is
   // then left aside.
+  // (measurement hook: HIP events of the caller's, recorded on the stream between the stages)
+  auto mark = [&](int i) {
+    if (a->stage_events && a->stage_events[i]) (void)hipEventRecord((hipEvent_t)a->stage_events[i], s);
+  };
+  mark(0);
   const bool planned = a->block_plan != nullptr && !a->gate_up_activations_T && !a->down_activations;
   if (planned && (a->block_plan_bytes < bookkeeping_bytes(a->T1, a->N, a->B) || ((uintptr_t)a->block_plan & 255) != 0))
     return MOE_E_BAD_ARG;
@@ -347,6 +352,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     rc = launch_prep(bk, a, n_real, s);
     if (rc != MOE_OK) return rc;
   }
+  mark(1);
 
   GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -484,6 +490,7 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     }
   }
   const unsigned gyc = (unsigned)bk.max_chunks;
+  mark(2);
   // checkpoints of blocks that never run stay zero
   if (a->gate_up_activations_T && (stages & MOE_STAGE_GATE_UP)) {
     rc = launch_fill_zero_bytes(a->gate_up_activations_T, (size_t)a->N * 2 * a->I * a->B * 2, s);
@@ -525,10 +532,12 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     }
     if (rc != MOE_OK) return rc;
   }
+  mark(3);
   if (a->kind == MOE_KIND_FP8_ROW && (stages & MOE_STAGE_REQUANT)) {
     rc = launch_row_requant((const float*)(ws + p.y), ws + p.yq, (float*)(ws + p.ys), bk, a->N, a->B, a->I, p.Iw, s);
     if (rc != MOE_OK) return rc;
   }
+  mark(4);
   if (stages & MOE_STAGE_DOWN) {
     if (mx_fast) {
       MxArgs m2 = m;
@@ -563,6 +572,11 @@ extern "C" int moe_blockwise_stages(const moe_bwmm_args* a, unsigned stages, voi
     }
     if (rc != MOE_OK) return rc;
   }
-  if (stages & MOE_STAGE_COMBINE) return launch_combine(bk, a, ws + p.d, n_real, s);
+  mark(5);
+  if (stages & MOE_STAGE_COMBINE) {
+    rc = launch_combine(bk, a, ws + p.d, n_real, s);
+    if (rc != MOE_OK) return rc;
+  }
+  mark(6);
   return MOE_OK;
 }

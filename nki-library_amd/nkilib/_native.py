@@ -104,6 +104,7 @@ class BwmmArgs(ctypes.Structure):
         ("gemm_clocks", c_void_p),
         ("block_plan", c_void_p),
         ("block_plan_bytes", c_size_t),
+        ("stage_events", c_void_p),
     ]
 
 

@@ -45,6 +45,10 @@ mx_weight_copies = True
 # Measurement hook: an int64 device tensor of 4 elements that the large-tile GEMMs fill with the shader cycles and
 # the 100 MHz ticks of their workgroup 0 (gate/up, then down): cycles / ticks * 0.1 = the clock in GHz under load.
 gemm_clock_probe = None
+# Measurement hook: seven ``torch.cuda.Event(enable_timing=True)`` (each recorded at least once before, so that its
+# HIP event exists) which the library records on the stream on entry and after the bookkeeping, the activation
+# quantisation, the gate/up GEMM, the fp8-row re-quantisation, the down GEMM and the combine of the next call.
+stage_events = None
 _KMAJOR_MAX_ENTRIES = 64
 _kmajor = {}
 
@@ -239,6 +243,12 @@ def run_blockwise(
         a.gate_up_proj_weight_kmajor = nv.ptr(kmajor[0])
         a.down_proj_weight_kmajor = nv.ptr(kmajor[1])
 
+    ev_handles = None
+    if stage_events is not None:
+        kernel_assert(len(stage_events) == 7, "stage_events must hold seven events")
+        # (entries may be None: that stage boundary is not recorded; the array is kept alive until the call returns)
+        ev_handles = (ctypes.c_void_p * 7)(*[None if e is None else e.cuda_event for e in stage_events])
+        a.stage_events = ctypes.cast(ev_handles, ctypes.c_void_p)
     need = L.moe_blockwise_workspace_bytes(ctypes.byref(a))
     if need == 0:
         # validation failed inside the library: run the call to obtain the precise code
