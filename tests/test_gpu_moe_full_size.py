@@ -113,6 +113,15 @@ def test_c4_sampled_tokens_and_invariants():
     out2 = _layer(t, cfg, ids, aff, x)
     assert torch.equal(out, out2), "two runs of the same layer differ"
 
+    # the bookkeeping handed over by the block build (used above) and the one the layer derives itself: same bits
+    from nkilib.core.moe.moe_cte import block_index
+    block_index.block_plans = False
+    try:
+        out3 = _layer(t, cfg, ids, aff, x)
+    finally:
+        block_index.block_plans = True
+    assert torch.equal(out, out3), "the layer's result depends on where its bookkeeping came from"
+
     # permutation of the tokens permutes the rows, bit for bit
     g = torch.Generator(device=dev)
     g.manual_seed(5)
