@@ -16,6 +16,7 @@ weights with per-channel scales, Mixtral-8x7B shape) through the same entry poin
 """
 
 import argparse
+import gc
 import json
 import math
 import os
@@ -266,11 +267,14 @@ def bench_fp8_row(args):
     for _ in range(args.warmup):
         step(None)
     torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()  # (as timeit does: a collection in the middle of the timed steps is the host's time, not the path's)
     t0 = time.perf_counter()
     for i in range(args.steps):
         out, recs, tp2id, b2e = step(timed_events[i])
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    gc.enable()
     gate_up_timed_ms = sum(ev.gate_up_ms() for ev in timed_events) / args.steps
     for i in range(args.steps):  # the per-stage table: the same steps again, every stage boundary recorded
         step(events[i])
@@ -412,11 +416,14 @@ def main():
     for _ in range(args.warmup):
         step(False)
     torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()  # (as timeit does: a collection in the middle of the timed steps is the host's time, not the path's)
     t0 = time.perf_counter()
     for i in range(args.steps):
         out, tp2id, b2e = step(True, i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    gc.enable()
     ms_per_step = wall * 1e3 / args.steps
 
     gate_up_timed_ms = sum(ev.gate_up_ms() for ev in timed_events) / args.steps
