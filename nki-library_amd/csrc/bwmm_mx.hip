@@ -970,7 +970,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     }
     const int pl0 = 4 * cl_e;
     constexpr int NPS = (NMT + 3) / 4;  // passes of 64 rows (the last one may hold two row tiles only)
-    // Clamps as unconditional min/max against +-inf, and the activation kind as a compile-time
+    // Clamps as an unconditional median of three against +-inf, and the activation kind as a compile-time
     // constant of the pass: a lane evaluates 128 elements here, and per-element decisions made this
     // code longer (and slower) than the K loop.
     // (derived here, behind a statement the compiler cannot look through, and kept in scalar registers: computed
@@ -981,10 +981,12 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     auto limit = [&](int bit, float v, float none) {
       return __builtin_bit_cast(float, uni(__builtin_bit_cast(int, (cmask & bit) ? v : none)));
     };
-    const float g_lo = limit(MOE_CLAMP_GATE_LO, a.clamp[1], -inf);
+    // min(max(v, lo), hi) as one median of three: the same value whenever lo <= hi, and with lo > hi (every v
+    // then becomes hi) once lo is lowered to hi
     const float g_hi = limit(MOE_CLAMP_GATE_HI, a.clamp[0], inf);
-    const float u_lo = limit(MOE_CLAMP_UP_LO, a.clamp[3], -inf);
+    const float g_lo = limit(MOE_CLAMP_GATE_LO, fminf(a.clamp[1], g_hi), -inf);
     const float u_hi = limit(MOE_CLAMP_UP_HI, a.clamp[2], inf);
+    const float u_lo = limit(MOE_CLAMP_UP_LO, fminf(a.clamp[3], u_hi), -inf);
     auto passes = [&](auto act_) {
     constexpr int ACT = decltype(act_)::value;
     static_for<0, NPS>([&](auto ps_) {
@@ -1015,18 +1017,17 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
           for (int t = 0; t < 4; ++t) {
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
-              const float lo = av[t][k], hi = av[t][2 + k];
-              const float mine = hcol_e ? hi : lo;
-              const float send = hcol_e ? lo : hi;
-              const float recv = __builtin_bit_cast(
-                  float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
-              float gv = hcol_e ? recv : mine, uv = hcol_e ? mine : recv;
+              // (the rotation writes one half of the 16 lanes only: banks 2, 3 = the up lanes take the gate lanes'
+              // rows 2, 3; banks 0, 1 = the gate lanes take the up lanes' rows 0, 1; the other half keeps its own)
+              const int lo = __builtin_bit_cast(int, av[t][k]), hi = __builtin_bit_cast(int, av[t][2 + k]);
+              float gv = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(lo, hi, 0x128 /* row_ror:8 */, 0xf, 0xc, false));
+              float uv = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(hi, lo, 0x128 /* row_ror:8 */, 0xf, 0x3, false));
               if constexpr (ROW8) {
                 gv = (gv * sg[t]) * rsk[k];
                 uv = (uv * su[t]) * rsk[k];
               }
-              const float gg = fminf(fmaxf(gv + bg[t], g_lo), g_hi);
-              const float uu = fminf(fmaxf(uv + bu[t], u_lo), u_hi);
+              const float gg = __builtin_amdgcn_fmed3f(gv + bg[t], g_lo, g_hi);
+              const float uu = __builtin_amdgcn_fmed3f(uv + bu[t], u_lo, u_hi);
               y[k][t] = act_apply(gg, ACT) * uu;
               if constexpr (BF16) {
                 ckg[t][k] = gg;
