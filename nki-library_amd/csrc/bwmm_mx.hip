@@ -987,8 +987,10 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     const float g_lo = limit(MOE_CLAMP_GATE_LO, fminf(a.clamp[1], g_hi), -inf);
     const float u_hi = limit(MOE_CLAMP_UP_HI, a.clamp[2], inf);
     const float u_lo = limit(MOE_CLAMP_UP_LO, fminf(a.clamp[3], u_hi), -inf);
-    auto passes = [&](auto act_) {
+    // (PLAIN: neither bias nor clamps, the fused act(gate) * up of most layers; their adds and medians are left out)
+    auto passes = [&](auto act_, auto plain_) {
     constexpr int ACT = decltype(act_)::value;
+    constexpr bool PLAIN = decltype(plain_)::value;
     static_for<0, NPS>([&](auto ps_) {
       constexpr int ps = decltype(ps_)::value;
       if (ps * 64 < cur.nrows) {
@@ -1026,8 +1028,8 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
                 gv = (gv * sg[t]) * rsk[k];
                 uv = (uv * su[t]) * rsk[k];
               }
-              const float gg = __builtin_amdgcn_fmed3f(gv + bg[t], g_lo, g_hi);
-              const float uu = __builtin_amdgcn_fmed3f(uv + bu[t], u_lo, u_hi);
+              const float gg = PLAIN ? gv : __builtin_amdgcn_fmed3f(gv + bg[t], g_lo, g_hi);
+              const float uu = PLAIN ? uv : __builtin_amdgcn_fmed3f(uv + bu[t], u_lo, u_hi);
               y[k][t] = act_apply(gg, ACT) * uu;
               if constexpr (BF16) {
                 ckg[t][k] = gg;
@@ -1133,11 +1135,16 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       }
     });
     };
+    // (the plain form exists for SiLU alone: every instance of this code lengthens the build)
+    const bool plain = cmask == 0 && a.bias == nullptr;
     switch (a.act_fn) {
-      case MOE_ACT_SILU: passes(std::integral_constant<int, MOE_ACT_SILU>{}); break;
-      case MOE_ACT_GELU: passes(std::integral_constant<int, MOE_ACT_GELU>{}); break;
-      case MOE_ACT_GELU_TANH: passes(std::integral_constant<int, MOE_ACT_GELU_TANH>{}); break;
-      default: passes(std::integral_constant<int, MOE_ACT_SWISH>{}); break;
+      case MOE_ACT_SILU:
+        if (plain) passes(std::integral_constant<int, MOE_ACT_SILU>{}, std::true_type{});
+        else passes(std::integral_constant<int, MOE_ACT_SILU>{}, std::false_type{});
+        break;
+      case MOE_ACT_GELU: passes(std::integral_constant<int, MOE_ACT_GELU>{}, std::false_type{}); break;
+      case MOE_ACT_GELU_TANH: passes(std::integral_constant<int, MOE_ACT_GELU_TANH>{}, std::false_type{}); break;
+      default: passes(std::integral_constant<int, MOE_ACT_SWISH>{}, std::false_type{}); break;
     }
     // the scale stages that the exchange buffer reaches into are written at the top of the next tile
     lds_barrier();
