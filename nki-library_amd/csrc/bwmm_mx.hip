@@ -242,6 +242,9 @@ __device__ __forceinline__ void ld_b128(v4i& d, uint32_t voff, const v4i& rsrc, 
 __device__ __forceinline__ void st_b64(const v2i& d, uint32_t voff, const v4i& rsrc, int soff) {
   asm volatile(MX_SGPR_WAIT "buffer_store_dwordx2 %0, %1, %2, %3 offen nt" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
+__device__ __forceinline__ void st_b128(const v4i& d, uint32_t voff, const v4i& rsrc, int soff) {
+  asm volatile(MX_SGPR_WAIT "buffer_store_dwordx4 %0, %1, %2, %3 offen nt" : : "v"(d), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
 // 16 bytes per lane straight into LDS at lds + 16 * lane (no destination registers).  The instruction takes its
 // LDS base from M0, which is set in the same statement.  M0 is declared clobbered: the compiler warns that it
 // does not save reserved registers around a statement, which is what is wanted here -- on this target it never
@@ -988,13 +991,23 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
     const float u_hi = limit(MOE_CLAMP_UP_HI, a.clamp[2], inf);
     const float u_lo = limit(MOE_CLAMP_UP_LO, fminf(a.clamp[3], u_hi), -inf);
     // (PLAIN: neither bias nor clamps, the fused act(gate) * up of most layers; their adds and medians are left out)
+    // fp8-row and bf16 kinds: the results go out in natural column order, which is the order the lanes hold them in
+    // (a lane's four partitions are four neighbouring columns), so they are stored straight from the registers, through
+    // a descriptor that ends behind the chunk's last row (rows past it are dropped by the range check); only the MX
+    // formats, whose blocks of 32 columns span the four waves, go through the exchange buffer.
+    const int y_rowb = uni(BF16 ? (int)(a.y_stride * 2) : (int)(a.y32_stride * 4));
+    const v4i rdy = make_rsrc(BF16 ? (const void*)((const uint8_t*)a.Yq + (int64_t)cur.slot0 * y_rowb)
+                                   : (const void*)((const uint8_t*)a.Y32 + (int64_t)cur.slot0 * y_rowb),
+                              ROW8 ? (uint32_t)(cur.nrows * y_rowb) : 0u);
+    const uint32_t y_voff = (uint32_t)((4 * g_e + 2 * hcol_e) * y_rowb) +
+                            (uint32_t)(tile_tI(cur) * 512 + q * tile_Pt(cur) + tile_p0(cur) + pl0) * (BF16 ? 2u : 4u);
     auto passes = [&](auto act_, auto plain_) {
     constexpr int ACT = decltype(act_)::value;
     constexpr bool PLAIN = decltype(plain_)::value;
     static_for<0, NPS>([&](auto ps_) {
       constexpr int ps = decltype(ps_)::value;
       if (ps * 64 < cur.nrows) {
-        lds_barrier();
+        if constexpr (!ROW8) lds_barrier();
         static_for<0, 4>([&](auto m_) {
           constexpr int ml = decltype(m_)::value;
           constexpr int mt = ps * 4 + ml;
@@ -1069,45 +1082,30 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
           }
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
-            const int rl = ml * 16 + 4 * g_e + 2 * hcol_e + k;
-            *(float4*)(E + rl * MX_EP + q * 32 + pl0) = make_float4(y[k][0], y[k][1], y[k][2], y[k][3]);
+            if constexpr (BF16) {
+              typedef __bf16 v2bf_ __attribute__((ext_vector_type(2)));
+              typedef float v2f_ __attribute__((ext_vector_type(2)));
+              const v2f_ p0 = {y[k][0], y[k][1]}, p1 = {y[k][2], y[k][3]};
+              const v2i o = {__builtin_bit_cast(int, __builtin_convertvector(p0, v2bf_)),
+                             __builtin_bit_cast(int, __builtin_convertvector(p1, v2bf_))};
+              st_b64(o, y_voff, rdy, (ps * 64 + ml * 16 + k) * y_rowb);
+            } else if constexpr (ROW8) {
+              const v4i o = {__builtin_bit_cast(int, y[k][0]), __builtin_bit_cast(int, y[k][1]),
+                             __builtin_bit_cast(int, y[k][2]), __builtin_bit_cast(int, y[k][3])};
+              st_b128(o, y_voff, rdy, (ps * 64 + ml * 16 + k) * y_rowb);
+            } else {
+              const int rl = ml * 16 + 4 * g_e + 2 * hcol_e + k;
+              *(float4*)(E + rl * MX_EP + q * 32 + pl0) = make_float4(y[k][0], y[k][1], y[k][2], y[k][3]);
+            }
           }
           }
         });
+        if constexpr (!ROW8) {
         lds_barrier();
         // thread (rl = tid/4, j = tid%4): MX block of chunk row ps*64 + rl, partitions 8j .. 8j+7 of the 32 (x 4 q)
         const int rl = tid_e >> 2, j = tid_e & 3;
         const int row = ps * 64 + rl;
-        if (BF16 && row < cur.nrows) {
-          // bf16 rows in natural column order: the thread's 4 x 8 values are four runs of 8 columns
-          typedef __bf16 v2bf_ __attribute__((ext_vector_type(2)));
-          typedef float v2f_ __attribute__((ext_vector_type(2)));
-          const float* src = E + rl * MX_EP + 8 * j;
-          uint16_t* dst = (uint16_t*)a.Yq + (int64_t)(cur.slot0 + row) * a.y_stride + tile_tI(cur) * 512 + tile_p0(cur) + 8 * j;
-          const int Pt = tile_Pt(cur);
-#pragma unroll
-          for (int qq = 0; qq < 4; ++qq) {
-            const float4 lo = *(const float4*)(src + qq * 32), hi = *(const float4*)(src + qq * 32 + 4);
-            const v2f_ p0 = {lo.x, lo.y}, p1 = {lo.z, lo.w}, p2 = {hi.x, hi.y}, p3 = {hi.z, hi.w};
-            *(uint4*)(dst + qq * Pt) = make_uint4(__builtin_bit_cast(uint32_t, __builtin_convertvector(p0, v2bf_)),
-                                                  __builtin_bit_cast(uint32_t, __builtin_convertvector(p1, v2bf_)),
-                                                  __builtin_bit_cast(uint32_t, __builtin_convertvector(p2, v2bf_)),
-                                                  __builtin_bit_cast(uint32_t, __builtin_convertvector(p3, v2bf_)));
-          }
-        }
-        if (ROW8 && !BF16 && row < cur.nrows) {
-          // fp32 rows in natural column order: the thread's 4 x 8 values are four runs of 8 columns
-          const float* src = E + rl * MX_EP + 8 * j;
-          float* dst = a.Y32 + (int64_t)(cur.slot0 + row) * a.y32_stride + tile_tI(cur) * 512 + tile_p0(cur) + 8 * j;
-          const int Pt = tile_Pt(cur);
-#pragma unroll
-          for (int qq = 0; qq < 4; ++qq) {
-            const float4 lo = *(const float4*)(src + qq * 32), hi = *(const float4*)(src + qq * 32 + 4);
-            *(float4*)(dst + qq * Pt) = lo;
-            *(float4*)(dst + qq * Pt + 4) = hi;
-          }
-        }
-        if (!ROW8 && row < cur.nrows) {
+        if (row < cur.nrows) {
           const float* src = E + rl * MX_EP + 8 * j;
           float yv[4][8];
           float am = 0.f;
@@ -1132,6 +1130,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
           o[1] = make_uint4(d[4], d[5], d[6], d[7]);
           a.Ys[slot * a.ys_stride + tile_tI(cur) * 16 + (pw >> 3)] = (uint8_t)sb;
         }
+        }
       }
     });
     };
@@ -1147,7 +1146,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       default: passes(std::integral_constant<int, MOE_ACT_SWISH>{}, std::false_type{}); break;
     }
     // the scale stages that the exchange buffer reaches into are written at the top of the next tile
-    lds_barrier();
+    if constexpr (!ROW8) lds_barrier();
   } else {
     const int64_t col0 = tile_h0(cur) + 64 * q + 4 * c_e;
     float bd[4];
