@@ -839,13 +839,18 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
 
   // The first D slices of a tile are requested at once (for the first tile before anything else, for every later
   // one ahead of the epilogue of the tile before it).
-  auto request_first_slices = [&]() {
-    static_for<0, D>([&](auto u_) {
-      constexpr int u = decltype(u_)::value;
-      const SliceAddr sa = slice_addr(u, u);
-      static_for<0, N0>([&](auto i_) { issue_load(i_, sa, br[u], asr, asr2, std::integral_constant<bool, u == 0>{}); });
+  // (numbered 0 .. D * N0 - 1 in issue order, slice after slice, so that a part of them can be asked for at a time)
+  constexpr int NFIRST = D * N0;
+  SliceAddr sa_first;  // of the slice whose loads are being issued
+  auto request_first = [&](auto n0_, auto n1_) {
+    static_for<decltype(n0_)::value, (decltype(n1_)::value < NFIRST ? decltype(n1_)::value : NFIRST)>([&](auto n_) {
+      constexpr int n = decltype(n_)::value;
+      constexpr int u = n / N0, i = n % N0;
+      if constexpr (i == 0) sa_first = slice_addr(u, u);
+      issue_load(std::integral_constant<int, i>{}, sa_first, br[u], asr, asr2, std::integral_constant<bool, u == 0>{});
     });
   };
+  auto request_first_slices = [&]() { request_first(std::integral_constant<int, 0>{}, std::integral_constant<int, NFIRST>{}); };
 
   // ---- first tile: nothing is in flight yet, so plain loads and waits do ----------------------------------
   Tile cur = tile_at(L);
@@ -935,8 +940,9 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   const int nbuf = have_next ? buf ^ 1 : buf;  // (behind the last tile: its own row table, which holds valid ids)
   tile_live = have_next ? -1 : 0;
   aim_loads_at(nxt, nbuf);
-  request_first_slices();
-  tile_live = -1;
+  // (down stage: they go out a few at a time between the row tiles of the epilogue, see there)
+  constexpr bool SPREAD_FIRST = STAGE == 2;
+  if constexpr (!SPREAD_FIRST) request_first_slices();
   if (AFF_ROWS) aff_raw(nxt, nbuf, aff_n);
   rs_raw(nxt, nbuf, rs_n);
   bias_raw(nxt, bias_n);
@@ -1218,8 +1224,15 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
         }
         st_b64(o, d_voff, rd, (mt * 16 + r) * rowb);
       }
+      // The next tile's first slices, a share behind every row tile: asked for all at once ahead of the epilogue
+      // they fill the CU's load queue, the wave stands at the first instruction that does not fit until the memory
+      // system has worked the queue down, and this arithmetic and these stores, which could run meanwhile, wait
+      // behind it.
+      constexpr int PER = (NFIRST + NMT - 1) / NMT;
+      request_first(std::integral_constant<int, mt * PER>{}, std::integral_constant<int, (mt + 1) * PER>{});
     });
   }
+  tile_live = -1;
 
   // ---- hand over to the next tile ------------------------------------------------------------------------
   // Everything in flight lands here: the next tile's first slices, this tile's stores (stores and loads share
