@@ -940,8 +940,10 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
   const int nbuf = have_next ? buf ^ 1 : buf;  // (behind the last tile: its own row table, which holds valid ids)
   tile_live = have_next ? -1 : 0;
   aim_loads_at(nxt, nbuf);
-  // (down stage: they go out a few at a time between the row tiles of the epilogue, see there)
-  constexpr bool SPREAD_FIRST = STAGE == 2;
+  // (down stage: they go out a few at a time between the row tiles of the epilogue, see there; not for the smallest
+  // tiles, whose launches do little but stream weights: there every load asked for later is time lost, 2 % of the
+  // down launch at decode sizes)
+  constexpr bool SPREAD_FIRST = STAGE == 2 && NMT >= 8;
   if constexpr (!SPREAD_FIRST) request_first_slices();
   if (AFF_ROWS) aff_raw(nxt, nbuf, aff_n);
   rs_raw(nxt, nbuf, rs_n);
@@ -1229,7 +1231,7 @@ __device__ __forceinline__ int mx_gemm_tiles(const MxArgs& a, uint8_t* smem, int
       // system has worked the queue down, and this arithmetic and these stores, which could run meanwhile, wait
       // behind it.
       constexpr int PER = (NFIRST + NMT - 1) / NMT;
-      request_first(std::integral_constant<int, mt * PER>{}, std::integral_constant<int, (mt + 1) * PER>{});
+      if constexpr (SPREAD_FIRST) request_first(std::integral_constant<int, mt * PER>{}, std::integral_constant<int, (mt + 1) * PER>{});
     });
   }
   tile_live = -1;
