@@ -748,6 +748,42 @@ def test_mx_prequantised_equals_online():
     assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "fp8_weights", "mx"])
+def test_plain_gate_up_epilogue_equals_the_general_one(kind):
+    """A SiLU layer without bias and clamps runs a form of the large-tile gate/up epilogue that leaves their adds and
+    medians out; with biases of zero, or clamps that no value reaches, the same layer takes the general form.  All
+    three must give the same rows (the reference applies bias and clamps only where given:
+    test/integration/nkilib/core/moe/moe_cte/test_utils.py:474-735)."""
+    import math
+
+    big = {"gate_clamp_upper_limit": 1e30, "gate_clamp_lower_limit": -1e30, "up_clamp_upper_limit": 1e30,
+           "up_clamp_lower_limit": -1e30}
+    if kind == "mx":
+        T, H, I, E, k, B = 300, 1024, 640, 4, 2, 128
+        c = mx_case(T, H, I, E, k, B, seed=61)
+        plain = from_bf16_tensor(_run_mx(c))
+        nI, pI = math.ceil(I / 512), 128
+        z = dict(c)
+        z["gate_up_bias"] = to_bf16(np.zeros((E, pI, 2, nI, 4), np.float32))
+        z["down_bias"] = to_bf16(np.zeros((E, H), np.float32))
+        with_zero_bias = from_bf16_tensor(_run_mx(z))
+        with_far_clamps = from_bf16_tensor(_run_mx_options(c, 0, big, False))
+    else:
+        T, H, I, E, k, B = 300, 1024, 640, 4, 2, 128
+        fp8 = kind == "fp8_weights"
+        c = dense_case(T, H, I, E, k, B, seed=62, quant=fp8, hidden_std=1.0)
+        plain = from_bf16_tensor(_run_dense(c, fp8_weights=fp8))
+        z = dict(c)
+        z["gate_up_bias"] = to_bf16(np.zeros((E, 2, I), np.float32))
+        z["down_bias"] = to_bf16(np.zeros((E, H), np.float32))
+        with_zero_bias = from_bf16_tensor(_run_dense(z, fp8_weights=fp8))
+        with_far_clamps = from_bf16_tensor(_run_dense(c, clamps=big, fp8_weights=fp8))
+    assert np.abs(plain).max() > 0
+    # (a padding token's row is zero in all of them; -0 and +0 compare equal)
+    np.testing.assert_array_equal(plain, with_zero_bias)
+    np.testing.assert_array_equal(plain, with_far_clamps)
+
+
 def test_smoke_entry():
     import __graft_entry__ as ge
 
