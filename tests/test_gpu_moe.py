@@ -493,6 +493,7 @@ def _golden_mx(c, act=0):
         (256, 512, 96, 4, 2, 256, True, False, False, None, True),     # tiny I, B=256
         (300, 512, 256, 2, 2, 128, True, False, False, None, False),   # 300 rows per expert: one 320-row chunk each
         (330, 1024, 384, 2, 2, 128, False, False, False, None, False), # 330 rows per expert: chunks of 256 + 74
+        (280, 512, 128, 2, 2, 128, True, False, False, None, False),    # one K slice in the down stage (fewer than the lookahead)
     ],
 )
 def test_mx_variants(T, H, I, E, k, B, bias, skip, dynamic, alpha, prequant):
